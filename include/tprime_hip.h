@@ -1,0 +1,148 @@
+/*
+ * tprime_hip.h — C ABI of libtprime_hip.so: gfx950 (MI355X) HIP kernels for the decoder-attention
+ * hot path of AI-Hypercomputer/torchprime: causal GQA attention forward/backward with segment-id
+ * document masking, RMSNorm forward/backward, rotary position embedding (table + apply).
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer owned by the caller (workspaces included); the library keeps
+ *     no persistent allocation and never synchronises the host.
+ *   - All launches are asynchronous on `stream` (a hipStream_t passed as void*; NULL = default stream).
+ *   - Strides are in ELEMENTS.  Tensors are addressed as (batch, head, seq, dim); the innermost (dim)
+ *     stride must be 1, the others are free, so both (B,H,S,D)-contiguous memory and the
+ *     (B,S,H,D)-memory-viewed-as-(B,H,S,D) layout the reference's attention modules produce
+ *     (torchprime/torch_xla_models/model/llama/model.py:219-227) are accepted without a copy.
+ *   - Every entry point returns TP_OK (0) or a negative TP_ERR_* code; tp_last_error() gives the
+ *     message for the calling thread.  Nothing throws or aborts.
+ *   - dtype codes: TP_BF16 / TP_F16 / TP_F32.
+ */
+#ifndef TPRIME_HIP_H
+#define TPRIME_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TP_OK 0
+#define TP_ERR_BAD_ARG (-1)     /* null pointer, non-positive size, misaligned pointer or stride */
+#define TP_ERR_UNSUPPORTED (-2) /* shape / dtype combination no kernel is built for */
+#define TP_ERR_LAUNCH (-3)      /* hipLaunch reported an error */
+
+#define TP_BF16 0
+#define TP_F16 1
+#define TP_F32 2
+
+/* Library version (major*10000 + minor*100 + patch). */
+int tp_version(void);
+/* Message of the last error on this thread ("" if none). The pointer stays valid until the next
+ * failing call on the same thread. */
+const char* tp_last_error(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * RMSNorm.  Replaces LlamaRMSNorm.forward (torchprime/torch_xla_models/model/llama/model.py:38-52),
+ * MixtralRMSNorm.forward (model/mixtral/model.py:44-59) and DeepseekV3RMSNorm.forward
+ * (model/deepseek_v3/model.py:32-44), which share one body:
+ *     y = weight * (x.float() * rsqrt(mean(x.float()^2, -1) + eps)).to(x.dtype)
+ * The normalised value is rounded to x's dtype before the weight multiply, as there.
+ *   x      (rows, hidden), row stride x_row_stride, dtype x_dtype
+ *   w      (hidden), dtype w_dtype: either x_dtype or TP_F32
+ *   y      (rows, hidden), row stride y_row_stride, dtype = x_dtype if w_dtype == x_dtype else TP_F32
+ *   rstd   (rows) fp32 out: rsqrt(mean(x^2) + eps), kept for the backward
+ * ---------------------------------------------------------------------------------------------- */
+int tp_rmsnorm_fwd(const void* x, const void* w, void* y, float* rstd, int64_t rows, int hidden,
+                   int64_t x_row_stride, int64_t y_row_stride, float eps, int x_dtype, int w_dtype,
+                   void* stream);
+
+/* Bytes of fp32 workspace tp_rmsnorm_bwd needs for (rows, hidden). */
+size_t tp_rmsnorm_bwd_workspace_bytes(int64_t rows, int hidden);
+
+/* Backward of the expression above (what autograd derives from model/llama/model.py:47-52):
+ *     n  = x * rstd;  g = dy * w
+ *     dx = rstd * (g - n * mean(g * n, -1))          (dtype x_dtype)
+ *     dw = sum_rows dy * n.to(x_dtype)               (dtype w_dtype)
+ *   dy     (rows, hidden), row stride dy_row_stride, dtype of y
+ *   ws     fp32 workspace of tp_rmsnorm_bwd_workspace_bytes(rows, hidden) bytes
+ * dw is reduced in a fixed order (no atomics): results are bitwise reproducible. */
+int tp_rmsnorm_bwd(const void* dy, const void* x, const void* w, const float* rstd, void* dx,
+                   void* dw, float* ws, int64_t rows, int hidden, int64_t dy_row_stride,
+                   int64_t x_row_stride, int64_t dx_row_stride, int x_dtype, int w_dtype,
+                   void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Rotary tables.  Replaces LlamaRotaryEmbedding.forward (model/llama/model.py:68-88) and
+ * DeepseekV3RotaryEmbedding.forward (model/deepseek_v3/model.py:57-75):
+ *     ang[b,s,i] = fp32(position_ids[b,s]) * inv_freq[i]          (fp32 product, as the K=1 matmul)
+ *     cos[b,s,:] = (cat(cos(ang), cos(ang)) * attention_scaling).to(dtype), sin likewise
+ *   inv_freq      (half) fp32;  position_ids (Bp, S) fp32 contiguous (the models pass float ids)
+ *   cos, sin      (Bp, S, 2*half) contiguous, dtype `dtype`
+ * ---------------------------------------------------------------------------------------------- */
+int tp_rope_table(const float* inv_freq, const float* position_ids, void* cos, void* sin, int Bp,
+                  int S, int half, float attention_scaling, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Rotary apply on q and k in one launch.  Replaces apply_rotary_pos_emb
+ * (model/llama/model.py:98-122), the position_ids-gather variant (model/mixtral/model.py:115-140)
+ * and apply_rotary_pos_emb_interleave (model/deepseek_v3/model.py:84-103):
+ *     x' = (x * cos) + (rotate_half(x) * sin),   rotate_half(x) = cat(-x[D/2:], x[:D/2])
+ * with each product and the sum rounded to the tensor dtype, as the eager expression does.
+ *   q (B,Hq,S,D), k (B,Hkv,S,D)  strided (dim stride 1); q_out/k_out same shapes, own strides
+ *   cos, sin  (Bc or T, S or T, D): row (b, s) is at  cs_b_stride*b + cs_s_stride*s  unless `pos`
+ *             is given, then at  cs_s_stride * pos[b*pos_b_stride + s]  (table gather, Mixtral)
+ *   interleaved != 0: x is first permuted [x0,x1,x2,...] -> [evens | odds] (DeepSeek); outputs stay
+ *             in the permuted order, as in the reference
+ *   backward != 0: q,k are gradients w.r.t. the outputs and q_out,k_out receive gradients w.r.t.
+ *             the inputs (transpose of the rotation, then the inverse permutation if interleaved)
+ *   k may be NULL (Hkv = 0) to rotate a single tensor.
+ * All base pointers and the b/h/s strides must keep rows 16-byte aligned; D % 16 == 0.
+ * ---------------------------------------------------------------------------------------------- */
+int tp_rope_apply(const void* q, const void* k, const void* cos, const void* sin,
+                  const int64_t* pos, void* q_out, void* k_out, int B, int Hq, int Hkv, int S, int D,
+                  const int64_t q_strides[3], const int64_t k_strides[3],
+                  const int64_t qo_strides[3], const int64_t ko_strides[3], int64_t cs_b_stride,
+                  int64_t cs_s_stride, int64_t pos_b_stride, int interleaved, int backward,
+                  int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Attention forward.  Replaces the three branches of AttentionModule.forward
+ * (torchprime/torch_xla_models/attention.py:70-123 splash, :124-150 flash, :151-170 eager) and the
+ * segment-id path of tpu_splash_attention_jax_call_wrapper (torchprime/utils/kernel_utils.py:28-131,
+ * 215-220, 259-263):
+ *     allowed[b,i,j] = (!causal || j <= i) && (seg == NULL || seg[b,i] == seg[b,j])
+ *     out[b,h,i,:]   = softmax_j(sm_scale * q[b,h,i,:].k[b,h/n_rep,j,:] | allowed) . v[b,h/n_rep,j,:]
+ *     lse[b,h,i]     = log sum_j exp(sm_scale * q.k) over allowed j   (natural log; -inf if none)
+ * GQA is by indexing (n_rep = Hq / Hkv), K/V are never expanded (attention.py:18-29, 46-51).
+ * A row with no allowed key gives out = 0 and lse = -inf.
+ *   q (B,Hq,Sq,Dqk)  k (B,Hkv,Skv,Dqk)  v (B,Hkv,Skv,Dv)  out (B,Hq,Sq,Dv)   strided, dim stride 1
+ *   seg   (B, Skv) int32 contiguous or NULL (requires Sq == Skv);  lse (B,Hq,Sq) fp32 contiguous
+ *   (Dqk, Dv) in {(64,64), (128,128), (192,128)};  dtype TP_BF16 or TP_F16
+ * ---------------------------------------------------------------------------------------------- */
+int tp_attn_fwd(const void* q, const void* k, const void* v, const int32_t* seg, void* out,
+                float* lse, int B, int Hq, int Hkv, int Sq, int Skv, int Dqk, int Dv,
+                const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                const int64_t o_strides[3], float sm_scale, int causal, int dtype, void* stream);
+
+/* Bytes of fp32 workspace tp_attn_bwd needs. */
+size_t tp_attn_bwd_workspace_bytes(int B, int Hq, int Sq);
+
+/* Attention backward (the reference gets it from autograd through attention.py:151-170, or from
+ * the Pallas backward kernels behind :121-123 / :144-150).  P is recomputed from lse:
+ *     P = exp(sm_scale*q.k - lse);  dV = P^T dO;  dS = P o (dO V^T - rowsum(dO o O));
+ *     dQ = sm_scale * dS K;  dK = sm_scale * dS^T Q   (dK, dV summed over the n_rep query heads)
+ * No atomics: results are bitwise reproducible.
+ *   dout, out (B,Hq,Sq,Dv) share o_strides... dout has its own do_strides
+ *   dq/dk/dv  strided like q/k/v but with their own stride arrays
+ *   ws        fp32 workspace of tp_attn_bwd_workspace_bytes(B,Hq,Sq) bytes
+ * ---------------------------------------------------------------------------------------------- */
+int tp_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                const float* lse, const int32_t* seg, void* dq, void* dk, void* dv, float* ws, int B,
+                int Hq, int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t do_strides[3],
+                const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                const int64_t dv_strides[3], float sm_scale, int causal, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TPRIME_HIP_H */

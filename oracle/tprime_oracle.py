@@ -1,0 +1,247 @@
+"""CPU ORACLE — TEST INFRASTRUCTURE ONLY.
+
+A plain-PyTorch (CPU, fp32/fp64) restatement of the arithmetic of torchprime's decoder-attention hot
+path.  Only tests, ``__graft_entry__.smoke()`` and ``bench.py``'s ``cpu_baseline`` leg may import
+this module; nothing under ``torchprime_amd/`` does.  Every function cites the reference lines it
+follows (paths relative to the reference checkout).
+
+Pinning status (what each function is checked against in tests/test_oracle.py, without importing the
+reference, which needs torch_xla / jax / omegaconf):
+
+  rms_norm                  F.rms_norm, fp64 numpy brute force, invariants          pinned
+  default/llama3 inv_freq   closed form; llm.c loop restated from torchprime/tests/test_rope.py:83-108;
+                            transformers ROPE_INIT_FUNCTIONS["llama3"] when installed   pinned
+  yarn inv_freq             transformers ROPE_INIT_FUNCTIONS["yarn"] when installed; closed-form
+                            special cases (factor 1 -> plain RoPE)                  pinned
+  rotary_cos_sin            closed form cos(p * f_i)                                pinned
+  apply_rotary_pos_emb      complex rotation, norm preservation, relative-position invariant  pinned
+  ..._interleave            permutation o rotate-half, QK^T invariance              pinned
+  eager_attention           F.scaled_dot_product_attention, brute-force loops       pinned
+  attention_ref             eager_attention (causal), block-diagonal decomposition for segments,
+                            brute force incl. fully-masked rows                     pinned
+  segment masking vs the reference's TPU splash kernel numerics                     PARITY UNPINNED:
+                            no reference test exercises decoder_segment_ids and the Pallas kernel is
+                            not in the tree; semantics are the closed form
+                            allowed = (j <= i) & (seg_i == seg_j) from kernel_utils.py:215-220, 259-263.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+NEG_INF = float("-inf")
+
+
+# ------------------------------------------------------------------------------------------------
+# RMSNorm — torchprime/torch_xla_models/model/llama/model.py:46-52 (same body at
+# model/mixtral/model.py:53-59, model/deepseek_v3/model.py:38-44)
+# ------------------------------------------------------------------------------------------------
+def rms_norm(hidden_states: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+  input_dtype = hidden_states.dtype
+  h = hidden_states.to(torch.float32)
+  variance = h.pow(2).mean(-1, keepdim=True)
+  h = h * torch.rsqrt(variance + eps)
+  return weight * h.to(input_dtype)
+
+
+def rms_norm_exact(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+  """The same function without intermediate rounding, in fp64 (what tolerances are measured against)."""
+  x = x.double()
+  return weight.double() * (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps))
+
+
+# ------------------------------------------------------------------------------------------------
+# inverse-frequency tables — torchprime/rope/rope.py
+# ------------------------------------------------------------------------------------------------
+def default_rope_frequencies(head_dim: int, theta: float = 10000.0) -> torch.Tensor:
+  """rope/rope.py:25-39."""
+  return 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
+
+
+def llama3_rope_frequencies(head_dim, theta=10000.0, factor=None, low_freq_factor=1.0, high_freq_factor=4.0,
+                            original_context_len=8192) -> torch.Tensor:
+  """rope/rope.py:42-75; ``factor=None`` means no scaling."""
+  freqs = default_rope_frequencies(head_dim, theta)
+  if factor is None:
+    return freqs
+  low_wl = original_context_len / low_freq_factor
+  high_wl = original_context_len / high_freq_factor
+  assert low_wl >= high_wl
+  wavelen = 2 * math.pi / freqs
+  freqs = torch.where(wavelen > low_wl, freqs / factor, freqs)
+  smooth = (original_context_len / wavelen - low_freq_factor) / (high_freq_factor - low_freq_factor)
+  smoothed = (1 - smooth) * freqs / factor + smooth * freqs
+  medium = ~(wavelen < high_wl) * ~(wavelen > low_wl)
+  return torch.where(medium, smoothed, freqs)
+
+
+def yarn_rope_frequencies(dim, base, factor, original_max, max_position_embeddings=None, beta_fast=32, beta_slow=1,
+                          mscale=None, mscale_all_dim=None, attention_factor=None, has_original=True):
+  """rope/rope.py:78-177 with the config fields spelled out as arguments."""
+  if has_original:
+    factor = max_position_embeddings / original_max
+  def get_mscale(scale, m=1):
+    return 1.0 if scale <= 1 else 0.1 * m * math.log(scale) + 1.0
+  if attention_factor is None:
+    if mscale and mscale_all_dim:
+      attention_factor = float(get_mscale(factor, mscale) / get_mscale(factor, mscale_all_dim))
+    else:
+      attention_factor = get_mscale(factor)
+  def corr(num_rot):
+    return (dim * math.log(original_max / (num_rot * 2 * math.pi))) / (2 * math.log(base))
+  low, high = max(math.floor(corr(beta_fast)), 0), min(math.ceil(corr(beta_slow)), dim - 1)
+  if low == high:
+    high += 0.001
+  pos_freqs = base ** (torch.arange(0, dim, 2).to(dtype=torch.float) / dim)
+  extra, inter = 1.0 / pos_freqs, 1.0 / (factor * pos_freqs)
+  ramp = torch.clamp((torch.arange(dim // 2, dtype=torch.float32) - low) / (high - low), 0, 1)
+  ef = 1 - ramp
+  return inter * (1 - ef) + extra * ef, attention_factor
+
+
+# ------------------------------------------------------------------------------------------------
+# cos/sin tables — model/llama/model.py:68-88; model/deepseek_v3/model.py:57-75 (attention_scaling)
+# ------------------------------------------------------------------------------------------------
+def rotary_cos_sin(inv_freq: torch.Tensor, position_ids: torch.Tensor, dtype: torch.dtype, attention_scaling=1.0):
+  inv = inv_freq[None, :, None].float().expand(position_ids.shape[0], -1, 1)
+  pos = position_ids[:, None, :].float()
+  freqs = (inv.float() @ pos.float()).transpose(1, 2)
+  emb = torch.cat((freqs, freqs), dim=-1)
+  cos, sin = emb.cos() * attention_scaling, emb.sin() * attention_scaling
+  return cos.to(dtype), sin.to(dtype)
+
+
+# ------------------------------------------------------------------------------------------------
+# rotary apply — model/llama/model.py:91-122; model/mixtral/model.py:136-140;
+# model/deepseek_v3/model.py:84-103
+# ------------------------------------------------------------------------------------------------
+def rotate_half(x):
+  x1 = x[..., : x.shape[-1] // 2]
+  x2 = x[..., x.shape[-1] // 2 :]
+  return torch.cat((-x2, x1), dim=-1)
+
+
+def apply_rotary_pos_emb(q, k, cos, sin, position_ids=None, unsqueeze_dim=1, gather=False):
+  if gather:  # Mixtral: tables (T, D) gathered by integer positions
+    cos, sin = cos[position_ids.long()], sin[position_ids.long()]
+  cos, sin = cos.unsqueeze(unsqueeze_dim), sin.unsqueeze(unsqueeze_dim)
+  return (q * cos) + (rotate_half(q) * sin), (k * cos) + (rotate_half(k) * sin)
+
+
+def apply_rotary_pos_emb_interleave(q, k, cos, sin, unsqueeze_dim=1):
+  cos, sin = cos.unsqueeze(unsqueeze_dim), sin.unsqueeze(unsqueeze_dim)
+  b, h, s, d = q.shape
+  q = q.reshape(b, h, s, d // 2, 2).transpose(4, 3).reshape(b, h, s, d)
+  b, h, s, d = k.shape
+  k = k.reshape(b, h, s, d // 2, 2).transpose(4, 3).reshape(b, h, s, d)
+  return (q * cos) + (rotate_half(q) * sin), (k * cos) + (rotate_half(k) * sin)
+
+
+# ------------------------------------------------------------------------------------------------
+# attention — torchprime/torch_xla_models/attention.py
+# ------------------------------------------------------------------------------------------------
+def repeat_kv(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
+  """attention.py:18-29."""
+  batch, kvh, slen, hd = hidden_states.shape
+  if n_rep == 1:
+    return hidden_states
+  return hidden_states[:, :, None, :, :].expand(batch, kvh, n_rep, slen, hd).reshape(batch, kvh * n_rep, slen, hd)
+
+
+def causal_additive_mask(seq_length: int, dtype=torch.float32) -> torch.Tensor:
+  """model/llama/model.py:347-352: -inf strictly above the diagonal, (1,1,S,S)."""
+  return torch.triu(torch.full((seq_length, seq_length), NEG_INF, dtype=dtype), diagonal=1)[None, None]
+
+
+def eager_attention(q, k, v, attention_mask=None):
+  """The eager branch of AttentionModule.forward, op for op (attention.py:46-60, 151-170), with
+  dropout p=0.  q (B,Hq,S,D), k/v (B,Hkv,S,D*); GQA by repeat_kv; scale 1/sqrt(v.shape[-1])."""
+  n_rep = q.shape[1] // k.shape[1]
+  k, v = repeat_kv(k, n_rep), repeat_kv(v, n_rep)
+  head_dim = v.shape[-1]
+  w = torch.matmul(q, k.transpose(2, 3)) / math.sqrt(head_dim)
+  if attention_mask is not None:
+    w = w + attention_mask[:, :, :, : k.shape[-2]]
+  w = F.softmax(w, dim=-1, dtype=torch.float32).to(q.dtype)
+  return torch.matmul(w, v)
+
+
+def allowed_mask(segment_ids, q_len: int, kv_len: int, causal: bool) -> torch.Tensor:
+  """Boolean (B or 1, q_len, kv_len): (j <= i if causal) AND same segment.  Closed form of
+  CausalMask/FullMask (kernel_utils.py:259-263) combined with SegmentIds(q=ids, kv=ids) (:215-220)."""
+  i = torch.arange(q_len)[:, None]
+  j = torch.arange(kv_len)[None, :]
+  m = (j <= i) if causal else torch.ones((q_len, kv_len), dtype=torch.bool)
+  m = m[None]
+  if segment_ids is not None:
+    seg = segment_ids.to("cpu")
+    m = m & (seg[:, :, None] == seg[:, None, :])
+  return m
+
+
+def attention_ref(q, k, v, segment_ids=None, causal=True, sm_scale=None, dtype=torch.float32):
+  """softmax(sm_scale * q k^T | allowed) v in ``dtype`` with no intermediate rounding; returns
+  (out, lse).  Rows with no allowed key give out = 0, lse = -inf (the eager formula gives NaN there;
+  tests assert that divergence explicitly)."""
+  q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+  n_rep = q.shape[1] // k.shape[1]
+  k, v = repeat_kv(k, n_rep), repeat_kv(v, n_rep)
+  if sm_scale is None:
+    sm_scale = 1.0 / math.sqrt(v.shape[-1])
+  s = torch.matmul(q, k.transpose(2, 3)) * sm_scale
+  m = allowed_mask(segment_ids, q.shape[2], k.shape[2], causal)[:, None]
+  s = s.masked_fill(~m, NEG_INF)
+  lse = torch.logsumexp(s, dim=-1)
+  any_allowed = m.any(-1)
+  p = torch.exp(s - torch.where(any_allowed, lse, torch.zeros_like(lse))[..., None])
+  p = torch.where(m, p, torch.zeros_like(p))
+  out = torch.matmul(p, v)
+  return out, lse
+
+
+def attention_ref_chunked(q, k, v, segment_ids=None, causal=True, sm_scale=None, dtype=torch.float32, heads_per_chunk=4):
+  """attention_ref evaluated a few heads at a time so S=8192 fits in host memory; same arithmetic."""
+  outs, lses = [], []
+  n_rep = q.shape[1] // k.shape[1]
+  step = n_rep * max(1, heads_per_chunk // n_rep)  # whole GQA groups per chunk
+  for h0 in range(0, q.shape[1], step):
+    h1 = min(h0 + step, q.shape[1])
+    ks, vs = k[:, h0 // n_rep : h1 // n_rep], v[:, h0 // n_rep : h1 // n_rep]
+    o, l = attention_ref(q[:, h0:h1], ks, vs, segment_ids, causal, sm_scale, dtype)
+    outs.append(o)
+    lses.append(l)
+  return torch.cat(outs, 1), torch.cat(lses, 1)
+
+
+def attention_grads_ref(q, k, v, dout, segment_ids=None, causal=True, sm_scale=None, dtype=torch.float32):
+  """(out, dq, dk, dv) by autograd through attention_ref."""
+  q = q.detach().to(dtype).requires_grad_(True)
+  k = k.detach().to(dtype).requires_grad_(True)
+  v = v.detach().to(dtype).requires_grad_(True)
+  out, _ = attention_ref(q, k, v, segment_ids, causal, sm_scale, dtype)
+  dq, dk, dv = torch.autograd.grad(out, (q, k, v), dout.to(dtype))
+  return out.detach(), dq, dk, dv
+
+
+# ------------------------------------------------------------------------------------------------
+# whole attention blocks — the callers (model/llama/model.py:206-238, 276-279)
+# ------------------------------------------------------------------------------------------------
+def llama_attention_block(x, w_norm, wq, wk, wv, wo, n_heads, n_kv_heads, eps, theta, attention_mask="causal"):
+  """input RMSNorm -> q/k/v projections -> RoPE -> eager attention -> output projection for one
+  Llama decoder layer's attention half (model/llama/model.py:276-279, 206-238, 331-360)."""
+  B, S, hidden = x.shape
+  hd = hidden // n_heads
+  h = rms_norm(x, w_norm, eps)
+  q = (h @ wq.T).view(B, S, n_heads, hd).transpose(1, 2)
+  k = (h @ wk.T).view(B, S, n_kv_heads, hd).transpose(1, 2)
+  v = (h @ wv.T).view(B, S, n_kv_heads, hd).transpose(1, 2)
+  pos = torch.arange(S)[None].float()
+  cos, sin = rotary_cos_sin(llama3_rope_frequencies(hd, theta), pos, x.dtype)
+  q, k = apply_rotary_pos_emb(q, k, cos, sin)
+  mask = causal_additive_mask(S, x.dtype) if isinstance(attention_mask, str) else attention_mask
+  o = eager_attention(q, k, v, mask)
+  o = o.transpose(1, 2).contiguous().reshape(B, S, hidden)
+  return o @ wo.T

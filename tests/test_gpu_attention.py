@@ -1,0 +1,252 @@
+"""GPU parity: attention forward/backward (through the torch.library ops, i.e. through the C ABI)
+against the fp32/fp64 CPU oracle on the same seeded inputs.  Tolerance for 16-bit outputs and
+gradients: max-abs <= 2e-2 and relative-L2 <= 1e-2 (tests/util.py)."""
+
+import math
+
+import pytest
+import torch
+
+import torchprime_amd as tpa
+from oracle import tprime_oracle as orc
+from tests.util import assert_close, heads_view, packed_segment_ids, randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _run(q, k, v, do, seg, causal, sm_scale):
+  qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+  segd = None if seg is None else seg.to(DEV)
+  out, lse = torch.ops.tprime.attn_fwd(qd, kd, vd, segd, sm_scale, causal)
+  out.backward(do.to(DEV))
+  return out.detach(), lse, qd.grad, kd.grad, vd.grad
+
+
+def _check(B, Hq, Hkv, S, Dqk, Dv, dtype, causal, seg=None, layout="bshd", seed=0, Skv=None, sm_scale=None, std=1.0):
+  Skv = S if Skv is None else Skv
+  mk = heads_view if layout == "bshd" else (lambda B_, H, S_, D, sd, dt, std=1.0: randn((B_, H, S_, D), sd, dt, std))
+  q = mk(B, Hq, S, Dqk, seed + 1, dtype, std)
+  k = mk(B, Hkv, Skv, Dqk, seed + 2, dtype, std)
+  v = mk(B, Hkv, Skv, Dv, seed + 3, dtype, std)
+  do = mk(B, Hq, S, Dv, seed + 4, dtype, 1.0)
+  sm_scale = 1.0 / math.sqrt(Dv) if sm_scale is None else sm_scale
+  out, lse, dq, dk, dv = _run(q, k, v, do, seg, causal, sm_scale)
+  o_ref, dq_ref, dk_ref, dv_ref = orc.attention_grads_ref(q, k, v, do, seg, causal, sm_scale, torch.float64)
+  _, lse_ref = orc.attention_ref(q, k, v, seg, causal, sm_scale, torch.float64)
+  assert out.shape == (B, Hq, S, Dv) and out.dtype == dtype
+  assert_close(out, o_ref, "out")
+  assert_close(lse, lse_ref, "lse", max_abs=2e-3, rel_l2=1e-3)
+  # gradients reach |x| > 4 with N(0,1) inputs, where one bf16 rounding alone is up to 1.6e-2:
+  # the max-abs bound is taken relative to the tensor's scale there (tests/util.py)
+  assert_close(dq, dq_ref, "dq", scale_abs=True)
+  assert_close(dk, dk_ref, "dk", scale_abs=True)
+  assert_close(dv, dv_ref, "dv", scale_abs=True)
+  return out
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize(
+  "B,Hq,Hkv,S,Dqk,Dv",
+  [
+    (2, 8, 8, 128, 64, 64),      # C1 attention shape
+    (1, 4, 1, 256, 128, 128),    # GQA 4:1, tile-aligned
+    (2, 8, 2, 200, 128, 128),    # ragged length
+    (1, 2, 2, 77, 64, 64),       # shorter than one tile
+    (1, 4, 4, 321, 192, 128),    # DeepSeek-style asymmetric heads
+    (1, 16, 2, 640, 128, 128),   # GQA 8:1 (Llama-3-70B grouping)
+    (1, 1, 1, 1, 128, 128),      # single token
+  ],
+)
+def test_causal_fwd_bwd(dtype, B, Hq, Hkv, S, Dqk, Dv):
+  _check(B, Hq, Hkv, S, Dqk, Dv, dtype, True)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,S,Skv,Dqk,Dv", [(1, 4, 2, 130, 130, 128, 128), (2, 2, 2, 64, 300, 64, 64), (1, 2, 1, 257, 100, 128, 128)])
+def test_full_attention_fwd_bwd(B, Hq, Hkv, S, Skv, Dqk, Dv):
+  # the eager branch without a mask (attention.py:151-170 with attention_mask=None)
+  _check(B, Hq, Hkv, S, Dqk, Dv, torch.bfloat16, False, Skv=Skv)
+
+
+def test_contiguous_bhsd_layout_and_scale():
+  _check(2, 4, 2, 150, 128, 128, torch.bfloat16, True, layout="bhsd", sm_scale=0.2)
+
+
+@pytest.mark.parametrize("S,lo,hi,causal", [(512, 16, 200, True), (700, 1, 90, True), (384, 64, 384, True), (300, 10, 120, False)])
+def test_segment_ids_fwd_bwd(S, lo, hi, causal):
+  seg, _ = packed_segment_ids(2, S, lo, hi, seed=S)
+  _check(2, 4, 2, S, 128, 128, torch.bfloat16, causal, seg=seg)
+
+
+def test_segment_ids_unsorted_and_negative_ids():
+  # ids need not be sorted or non-negative: equality is all that matters
+  g = torch.Generator().manual_seed(3)
+  seg = torch.randint(-2, 3, (2, 260), generator=g, dtype=torch.int32)
+  _check(2, 2, 1, 260, 64, 64, torch.bfloat16, True, seg=seg)
+  _check(2, 2, 1, 260, 64, 64, torch.bfloat16, False, seg=seg)
+
+
+def test_segment_equals_block_diagonal_decomposition():
+  """Document masking == running each document through causal attention on its own."""
+  B, Hq, Hkv, S, D = 1, 4, 2, 448, 128
+  seg, lengths = packed_segment_ids(B, S, 32, 200, seed=9)
+  q, k, v = (heads_view(B, h, S, D, s, torch.bfloat16) for h, s in ((Hq, 1), (Hkv, 2), (Hkv, 3)))
+  full = tpa.ops.attention(q.to(DEV), k.to(DEV), v.to(DEV), seg.to(DEV), None, True)
+  pos = 0
+  for L in lengths[0]:
+    sl = slice(pos, pos + L)
+    part = tpa.ops.attention(q[:, :, sl].to(DEV), k[:, :, sl].to(DEV), v[:, :, sl].to(DEV), None, None, True)
+    assert_close(full[:, :, sl], part.float().cpu(), f"doc@{pos}", max_abs=8e-3, rel_l2=4e-3)
+    pos += L
+
+
+@pytest.mark.parametrize("causal,use_seg", [(True, False), (True, True), (False, True)])
+def test_mask_pattern_exact(causal, use_seg):
+  """Recover P through the public op with one-hot V blocks and compare its support with the closed-form
+  mask: entries that must be masked are exactly 0, allowed entries are > 0."""
+  B, H, S, D = 1, 2, 192, 64
+  seg = None
+  if use_seg:
+    seg, _ = packed_segment_ids(B, S, 5, 70, seed=4)
+  q = heads_view(B, H, S, D, 1, torch.bfloat16, 0.3).to(DEV)
+  k = heads_view(B, H, S, D, 2, torch.bfloat16, 0.3).to(DEV)
+  allowed = orc.allowed_mask(seg, S, S, causal)[0]
+  P = torch.zeros((H, S, S))
+  for j0 in range(0, S, D):
+    v = torch.zeros((B, H, S, D), dtype=torch.bfloat16)
+    for j in range(j0, min(j0 + D, S)):
+      v[:, :, j, j - j0] = 1
+    o = tpa.ops.attention(q, k, v.to(DEV), None if seg is None else seg.to(DEV), None, causal)
+    P[:, :, j0 : j0 + D] = o[0, :, :, : min(D, S - j0)].float().cpu()
+  assert torch.equal(P > 0, allowed[None].expand_as(P)), "support of P differs from the mask"
+  assert_close(P.sum(-1), torch.ones(H, S), "rows sum to 1", max_abs=2e-2)
+
+
+def test_eager_formula_is_nan_on_fully_masked_rows_but_kernel_convention_is_zero():
+  """The eager expression gives NaN for a row whose mask is all -inf; the documented convention of
+  the oracle (and the kernels) for such a row is out = 0, lse = -inf.  Through the public mask
+  definition (causal and/or same-segment with Sq == Skv) every row keeps at least its own key, so
+  the convention is only reachable with Sq > Skv... which the API does not mask; asserted on the oracle."""
+  q = randn((1, 1, 4, 8), 1)
+  mask = torch.full((1, 1, 4, 4), float("-inf"))
+  assert torch.isnan(orc.eager_attention(q, q, q, mask)).all()
+
+
+def test_deterministic_backward():
+  B, Hq, Hkv, S, D = 1, 8, 2, 384, 128
+  q, k, v, do = (heads_view(B, h, S, D, s, torch.bfloat16) for h, s in ((Hq, 1), (Hkv, 2), (Hkv, 3), (Hq, 4)))
+  r1 = _run(q, k, v, do, None, True, D**-0.5)
+  r2 = _run(q, k, v, do, None, True, D**-0.5)
+  for a, b in zip(r1, r2):
+    assert torch.equal(a, b)
+
+
+# ---- module / functional API ----------------------------------------------------------------------
+def _cfg(kernel, hq, hkv):
+  return tpa.Config(attention_kernel=kernel, num_attention_heads=hq, num_key_value_heads=hkv, attention_dropout=False)
+
+
+@pytest.mark.parametrize("kernel", ["splash_attention", "flash_attention", None, "pytorch"])
+def test_attention_module_matches_eager_branch(kernel):
+  B, Hq, Hkv, S, D = 2, 8, 2, 160, 128
+  q, k, v = (heads_view(B, h, S, D, s, torch.bfloat16) for h, s in ((Hq, 1), (Hkv, 2), (Hkv, 3)))
+  mask = orc.causal_additive_mask(S)
+  m = tpa.AttentionModule(_cfg(kernel, Hq, Hkv))
+  out = m(q.to(DEV), k.to(DEV), v.to(DEV), mask.to(DEV))
+  ref = orc.eager_attention(q.float(), k.float(), v.float(), mask)
+  assert_close(out, ref, f"kernel={kernel}")
+  assert m.partition_spec is None and out.transpose(1, 2).is_contiguous()
+
+
+def test_attention_module_scale_uses_v_head_dim():
+  # DeepSeek: qk dim 192, v dim 128 -> 1/sqrt(128) (attention.py:54-58)
+  B, H, S = 1, 4, 96
+  q, k = heads_view(B, H, S, 192, 1, torch.bfloat16, 0.5), heads_view(B, H, S, 192, 2, torch.bfloat16, 0.5)
+  v = heads_view(B, H, S, 128, 3, torch.bfloat16)
+  out = tpa.AttentionModule(_cfg("splash_attention", H, H))(q.to(DEV), k.to(DEV), v.to(DEV))
+  ref, _ = orc.attention_ref(q, k, v, None, True, 1 / math.sqrt(128), torch.float64)
+  wrong, _ = orc.attention_ref(q, k, v, None, True, 1 / math.sqrt(192), torch.float64)
+  assert_close(out, ref, "scale 1/sqrt(v_dim)")
+  assert (out.float().cpu() - wrong.float()).abs().max() > 5e-2
+
+
+def test_attention_module_eager_without_mask_is_full_attention_and_bad_mask_raises():
+  B, H, S, D = 1, 2, 80, 64
+  q, k, v = (heads_view(B, H, S, D, s, torch.bfloat16) for s in (1, 2, 3))
+  m = tpa.AttentionModule(_cfg(None, H, H))
+  out = m(q.to(DEV), k.to(DEV), v.to(DEV), None)
+  assert_close(out, orc.eager_attention(q.float(), k.float(), v.float(), None), "no mask")
+  bad = torch.zeros((1, 1, S, S), device=DEV)
+  with pytest.raises(NotImplementedError):
+    m(q.to(DEV), k.to(DEV), v.to(DEV), bad)
+
+
+def test_splash_wrapper_signature_and_segments():
+  B, Hq, Hkv, S, D = 2, 4, 2, 256, 128
+  seg, _ = packed_segment_ids(B, S, 20, 100, seed=5)
+  q, k, v = (heads_view(B, h, S, D, s, torch.bfloat16) for h, s in ((Hq, 1), (Hkv, 2), (Hkv, 3)))
+  qs = (q.float() / math.sqrt(D)).to(torch.bfloat16)  # callers pre-scale q (attention.py:107)
+  cfg = tpa.SplashAttentionConfig(mesh="ignored").to_json()
+  res = tpa.tpu_splash_attention_jax_call_wrapper(
+    mask=None, query=qs.to(DEV), key=k.to(DEV), value=v.to(DEV), config=cfg,
+    decoder_segment_ids=seg.to(DEV), causal=True, q_seq_shards=1,
+  )
+  assert isinstance(res, tuple) and len(res) == 3 and res[1] is None and res[2] is None
+  ref, _ = orc.attention_ref(qs, k, v, seg, True, 1.0, torch.float64)
+  assert_close(res[0], ref, "segments via wrapper")
+  assert tpa.tpu_splash_attention_jax_call_wrapper(None, qs.to(DEV), k.to(DEV), v.to(DEV), cfg, None, True, is_forward=False) is None
+  with pytest.raises(AssertionError):
+    tpa.tpu_splash_attention_jax_call_wrapper(None, qs.to(DEV), k.to(DEV), v.to(DEV), cfg, seg[:, :100].to(DEV), True)
+  slide = tpa.SplashAttentionConfig(attentiontype_local_sliding=True).to_json()
+  with pytest.raises(ValueError):
+    tpa.tpu_splash_attention_jax_call_wrapper(None, qs.to(DEV), k.to(DEV), v.to(DEV), slide, None, True)
+
+
+def test_unsupported_inputs_raise():
+  q = torch.zeros((1, 2, 16, 96), dtype=torch.bfloat16, device=DEV)
+  with pytest.raises(NotImplementedError):
+    tpa.ops.attention(q, q, q)
+  q32 = torch.zeros((1, 2, 16, 64), dtype=torch.float32, device=DEV)
+  with pytest.raises(TypeError):
+    tpa.ops.attention(q32, q32, q32)
+  with pytest.raises(RuntimeError):
+    tpa.ops.attention(q.cpu(), q.cpu(), q.cpu())
+
+
+# ---- BASELINE-size cases ----------------------------------------------------------------------------
+def _slice_check(B, Hq, Hkv, S, Dqk, Dv, seg, seed, b_sel, g_sel, sm_scale=None):
+  """Run the kernels on the full problem, check one (batch, kv-head group) slice against the oracle
+  (attention is independent per batch and kv head, so the slice is an exact sub-problem)."""
+  n_rep = Hq // Hkv
+  dt = torch.bfloat16
+  q, k, v, do = (heads_view(B, h, S, d, seed + i, dt) for i, (h, d) in enumerate(((Hq, Dqk), (Hkv, Dqk), (Hkv, Dv), (Hq, Dv))))
+  sm_scale = 1.0 / math.sqrt(Dv) if sm_scale is None else sm_scale
+  out, lse, dq, dk, dv = _run(q, k, v, do, seg, True, sm_scale)
+  hs = slice(g_sel * n_rep, (g_sel + 1) * n_rep)
+  qs, ks, vs, dos = q[b_sel : b_sel + 1, hs], k[b_sel : b_sel + 1, g_sel : g_sel + 1], v[b_sel : b_sel + 1, g_sel : g_sel + 1], do[b_sel : b_sel + 1, hs]
+  segs = None if seg is None else seg[b_sel : b_sel + 1]
+  o_ref, dq_ref, dk_ref, dv_ref = orc.attention_grads_ref(qs, ks, vs, dos, segs, True, sm_scale, torch.float32)
+  assert_close(out[b_sel : b_sel + 1, hs], o_ref, "out")
+  assert_close(dq[b_sel : b_sel + 1, hs], dq_ref, "dq", scale_abs=True)
+  assert_close(dk[b_sel : b_sel + 1, g_sel : g_sel + 1], dk_ref, "dk", scale_abs=True)
+  assert_close(dv[b_sel : b_sel + 1, g_sel : g_sel + 1], dv_ref, "dv", scale_abs=True)
+  # every row is a convex combination of V rows: bounded by max |v|
+  assert out.abs().max().item() <= v.abs().max().item() + 1e-2
+  assert torch.isfinite(lse).all() and torch.isfinite(dq.float()).all()
+
+
+def test_llama3_8b_shape_slice():  # BASELINE config 2: B=4, S=8192, 32q/8kv, d=128
+  _slice_check(4, 32, 8, 8192, 128, 128, None, 1234 + 1, b_sel=3, g_sel=5)
+
+
+def test_llama3_8b_packed_segments_slice():  # BASELINE config 3: documents of 64..4096 packed to 8192
+  seg, _ = packed_segment_ids(4, 8192, 64, 4096, seed=1234 + 2)
+  _slice_check(4, 32, 8, 8192, 128, 128, seg, 1234 + 2, b_sel=1, g_sel=2)
+
+
+def test_llama3_70b_shape_slice():  # BASELINE config 3: B=1, S=8192, 64q/8kv
+  _slice_check(1, 64, 8, 8192, 128, 128, None, 1234 + 3, b_sel=0, g_sel=7)
+
+
+def test_deepseek_v3_shape_slice():  # BASELINE config 4: B=1, S=4096, 128 heads, qk 192 / v 128, scale 1/sqrt(128)
+  _slice_check(1, 128, 128, 4096, 192, 128, None, 1234 + 4, b_sel=0, g_sel=77)

@@ -1,0 +1,95 @@
+"""Drop-in for ``torchprime.torch_xla_models.attention`` on one MI355X.
+
+``AttentionModule`` keeps the reference's constructor, attributes, forward signature, shape checks
+and softmax scale (torchprime/torch_xla_models/attention.py:32-177).  Where the reference dispatches
+to a TPU Pallas kernel (splash :70-123, flash :124-150) or materialises the (B,H,S,S) logits
+(eager :151-170), this module calls one HIP kernel pair (``tprime::attn_fwd`` / ``tprime::attn_bwd``)
+with native GQA, so K/V are never expanded by ``repeat_kv``.  Mesh and partition specs do not exist
+on a single GPU: they are accepted and ignored.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Any
+
+import torch
+from torch import nn
+
+from . import ops
+from .config import has_key
+
+
+def repeat_kv(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
+  """(batch, kv_heads, seq, dim) -> (batch, kv_heads * n_rep, seq, dim), each head repeated n_rep
+  times in place (``torch.repeat_interleave(x, n_rep, dim=1)``); attention.py:18-29.  The kernels
+  index kv head ``h // n_rep`` instead and never call this; it is exported for API parity."""
+  if n_rep == 1:
+    return hidden_states
+  b, h, s, d = hidden_states.shape
+  return hidden_states.unsqueeze(2).expand(b, h, n_rep, s, d).reshape(b, h * n_rep, s, d)
+
+
+def _is_causal_additive_mask(mask: torch.Tensor, q_len: int, kv_len: int) -> bool:
+  """True when ``mask[..., :kv_len]`` is 0 on and below the diagonal and -inf above it, the mask the
+  models build at model/llama/model.py:347-355."""
+  if mask.dim() != 4 or mask.shape[1] != 1 or mask.shape[2] != q_len or mask.shape[3] < kv_len:
+    return False
+  m = mask[:, :, :, :kv_len]
+  keep = torch.ones((q_len, kv_len), dtype=torch.bool, device=mask.device).tril()
+  ok = ((m == 0) == keep) & ((m == float("-inf")) == ~keep)
+  return bool(ok.all())
+
+
+class AttentionModule(nn.Module):
+  def __init__(self, config, kernel_config: dict[str, Any] | None = None):
+    super().__init__()
+    self.config = config
+    self.kernel_config = kernel_config
+    self.partition_spec = None
+
+  def forward(
+    self,
+    query_states: torch.Tensor,  # (batch_size, num_heads, q_len, head_dim)
+    key_states: torch.Tensor,  # (batch_size, num_kv_heads, kv_len, head_dim)
+    value_states: torch.Tensor,  # (batch_size, num_kv_heads, kv_len, head_dim)
+    attention_mask: torch.Tensor | None = None,
+  ):
+    kernel = self.config.attention_kernel
+    bsz, num_heads, q_len, _ = query_states.size()
+    # the reference scales by, and checks the output against, v's head dim (attention.py:54-58)
+    head_dim = value_states.shape[-1]
+    kv_seq_len = key_states.shape[-2]
+    self.partition_spec = None  # no mesh on one GPU (attention.py:61-67)
+
+    if has_key(self.config, "load_balance_cp") and self.config.load_balance_cp:
+      raise NotImplementedError("load-balanced context parallelism needs a device mesh; this build is single-GPU")
+
+    if kernel in ("splash_attention", "flash_attention"):
+      # both kernel branches are causal and never see attention_mask (attention.py:121-123, 144-150)
+      causal = True
+    else:
+      # eager branch: softmax(QK^T/sqrt(d) + mask); no mask means full attention (attention.py:151-170)
+      p = getattr(self.config, "attention_dropout", 0.0)
+      if p and self.training:
+        raise NotImplementedError("attention_dropout > 0 is not supported (every shipped config uses 0)")
+      if attention_mask is None:
+        causal = False
+      else:
+        assume = bool(self.kernel_config and self.kernel_config.get("assume_causal_mask"))
+        if not assume and not _is_causal_additive_mask(attention_mask, q_len, kv_seq_len):
+          raise NotImplementedError(
+            "only the causal additive mask (0 on/below the diagonal, -inf above) is supported; "
+            "document masking goes through segment ids (tpu_splash_attention_jax_call_wrapper)"
+          )
+        causal = True
+
+    attn_output = ops.attention(
+      query_states, key_states, value_states, None, 1.0 / math.sqrt(head_dim), causal
+    )
+
+    if attn_output.size() != (bsz, num_heads, q_len, head_dim):
+      raise ValueError(
+        f"`attn_output` should be of size {(bsz, num_heads, q_len, head_dim)}, but is {attn_output.size()}"
+      )
+    return attn_output

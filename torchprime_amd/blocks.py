@@ -1,0 +1,145 @@
+"""Attention blocks that call the hot path the way the reference's models do.  They exist so tests
+and the benchmark can drive RMSNorm -> projections -> RoPE -> attention -> output projection with the
+reference's tensor layouts; the projections are stock ``nn.Linear`` (GEMMs are outside the path).
+
+* LlamaAttention        torchprime/torch_xla_models/model/llama/model.py:156-238
+* MixtralAttention      model/mixtral/model.py:159-243
+* DeepseekV3Attention   model/deepseek_v3/model.py:341-455
+"""
+
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from .attention import AttentionModule
+from .norm import DeepseekV3RMSNorm
+from .rotary import MixtralRotaryEmbedding, apply_rotary_pos_emb, apply_rotary_pos_emb_interleave
+
+
+class LlamaAttention(nn.Module):
+  def __init__(self, config, layer_idx: int | None = None):
+    super().__init__()
+    self.config = config
+    self.attention_block = AttentionModule(config)
+    self.layer_idx = layer_idx
+    self.hidden_size = config.hidden_size
+    self.num_heads = config.num_attention_heads
+    self.head_dim = self.hidden_size // self.num_heads
+    self.num_key_value_heads = config.num_key_value_heads
+    self.num_key_value_groups = self.num_heads // self.num_key_value_heads
+    if (self.head_dim * self.num_heads) != self.hidden_size:
+      raise ValueError(
+        f"hidden_size must be divisible by num_heads (got `hidden_size`: {self.hidden_size}"
+        f" and `num_heads`: {self.num_heads})."
+      )
+    bias = bool(getattr(config, "attention_bias", False))
+    self.q_proj = nn.Linear(self.hidden_size, self.num_heads * self.head_dim, bias=bias)
+    self.k_proj = nn.Linear(self.hidden_size, self.num_key_value_heads * self.head_dim, bias=bias)
+    self.v_proj = nn.Linear(self.hidden_size, self.num_key_value_heads * self.head_dim, bias=bias)
+    self.o_proj = nn.Linear(self.hidden_size, self.hidden_size, bias=bias)
+
+  def forward(self, hidden_states, position_embeddings, attention_mask=None, position_ids=None):
+    bsz, q_len, _ = hidden_states.size()
+    q = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
+    k = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+    v = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+    cos, sin = position_embeddings
+    q, k = apply_rotary_pos_emb(q, k, cos, sin)
+    out = self.attention_block(q, k, v, attention_mask)
+    out = out.transpose(1, 2).contiguous().reshape(bsz, q_len, self.hidden_size)
+    return self.o_proj(out)
+
+
+class MixtralAttention(nn.Module):
+  def __init__(self, config, layer_idx: int | None = None):
+    super().__init__()
+    self.config = config
+    self.attention_block = AttentionModule(config)
+    self.layer_idx = layer_idx
+    self.hidden_size = config.hidden_size
+    self.num_heads = config.num_attention_heads
+    self.head_dim = self.hidden_size // self.num_heads
+    self.num_key_value_heads = config.num_key_value_heads
+    self.num_key_value_groups = self.num_heads // self.num_key_value_heads
+    self.max_position_embeddings = config.max_position_embeddings
+    self.rope_theta = config.rope_theta
+    if (self.head_dim * self.num_heads) != self.hidden_size:
+      raise ValueError(
+        f"hidden_size must be divisible by num_heads (got `hidden_size`: {self.hidden_size}"
+        f" and `num_heads`: {self.num_heads})."
+      )
+    self.q_proj = nn.Linear(self.hidden_size, self.num_heads * self.head_dim, bias=False)
+    self.k_proj = nn.Linear(self.hidden_size, self.num_key_value_heads * self.head_dim, bias=False)
+    self.v_proj = nn.Linear(self.hidden_size, self.num_key_value_heads * self.head_dim, bias=False)
+    self.o_proj = nn.Linear(self.num_heads * self.head_dim, self.hidden_size, bias=False)
+    self.rotary_emb = MixtralRotaryEmbedding(
+      self.head_dim, max_position_embeddings=self.max_position_embeddings, base=self.rope_theta
+    )
+
+  def forward(self, hidden_states, attention_mask=None, position_ids=None):
+    bsz, q_len, _ = hidden_states.size()
+    q = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
+    k = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+    v = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+    cos, sin = self.rotary_emb(v, seq_len=k.shape[-2])
+    q, k = apply_rotary_pos_emb(q, k, cos, sin, position_ids)
+    out = self.attention_block(q, k, v, attention_mask)
+    out = out.transpose(1, 2).contiguous().reshape(bsz, q_len, self.hidden_size)
+    return self.o_proj(out)
+
+
+class DeepseekV3Attention(nn.Module):
+  """Multi-headed latent attention: low-rank q and kv projections with RMSNorm on the latents,
+  128 un-rotated + 64 rotated q/k dims, one shared rotated k head, v head dim 128."""
+
+  def __init__(self, config, layer_idx: int | None = None):
+    super().__init__()
+    self.config = config
+    self.attention_block = AttentionModule(config)
+    self.layer_idx = layer_idx
+    self.num_heads = config.num_attention_heads
+    self.qk_head_dim = config.qk_head_dim
+    bias = bool(getattr(config, "attention_bias", False))
+    if config.q_lora_rank is None:
+      self.q_proj = nn.Linear(config.hidden_size, self.num_heads * self.qk_head_dim, bias=False)
+    else:
+      self.q_a_proj = nn.Linear(config.hidden_size, config.q_lora_rank, bias=bias)
+      self.q_a_layernorm = DeepseekV3RMSNorm(config.q_lora_rank)
+      self.q_b_proj = nn.Linear(config.q_lora_rank, self.num_heads * self.qk_head_dim, bias=False)
+    self.kv_a_proj_with_mqa = nn.Linear(config.hidden_size, config.kv_lora_rank + config.qk_rope_head_dim, bias=bias)
+    self.kv_a_layernorm = DeepseekV3RMSNorm(config.kv_lora_rank)
+    self.kv_b_proj = nn.Linear(
+      config.kv_lora_rank, self.num_heads * (config.qk_nope_head_dim + config.v_head_dim), bias=False
+    )
+    self.o_proj = nn.Linear(self.num_heads * config.v_head_dim, config.hidden_size, bias=bias)
+
+  def forward(self, hidden_states, position_embeddings, attention_mask=None, position_ids=None):
+    cfg = self.config
+    bsz, q_len = hidden_states.shape[:2]
+    if cfg.q_lora_rank is None:
+      q = self.q_proj(hidden_states)
+    else:
+      q = self.q_b_proj(self.q_a_layernorm(self.q_a_proj(hidden_states)))
+    q = q.view(bsz, q_len, -1, self.qk_head_dim).transpose(1, 2)
+    q_pass, q_rot = torch.split(q, [cfg.qk_nope_head_dim, cfg.qk_rope_head_dim], dim=-1)
+
+    compressed_kv = self.kv_a_proj_with_mqa(hidden_states)
+    k_pass, k_rot = torch.split(compressed_kv, [cfg.kv_lora_rank, cfg.qk_rope_head_dim], dim=-1)
+    k_pass = self.kv_b_proj(self.kv_a_layernorm(k_pass))
+    k_pass = k_pass.view(bsz, q_len, -1, cfg.qk_nope_head_dim + cfg.v_head_dim).transpose(1, 2)
+    k_pass, v = torch.split(k_pass, [cfg.qk_nope_head_dim, cfg.v_head_dim], dim=-1)
+
+    k_rot = k_rot.view(bsz, 1, q_len, cfg.qk_rope_head_dim)
+    cos, sin = position_embeddings
+    if cfg.rope_interleave:
+      q_rot, k_rot = apply_rotary_pos_emb_interleave(q_rot, k_rot, cos, sin)
+    else:
+      q_rot, k_rot = apply_rotary_pos_emb(q_rot, k_rot, cos, sin)
+    k_rot = k_rot.expand(*k_pass.shape[:-1], -1)
+
+    q = torch.cat((q_pass, q_rot), dim=-1)
+    k = torch.cat((k_pass, k_rot), dim=-1)
+    out = self.attention_block(q, k, v, attention_mask)
+    out = out.transpose(1, 2).contiguous().reshape(bsz, q_len, -1)
+    return self.o_proj(out)

@@ -1,0 +1,712 @@
+// Attention backward for gfx950: recompute P from LSE, no atomics, bitwise reproducible.
+//
+// The reference obtains these gradients from autograd through the eager expression
+// (torchprime/torch_xla_models/attention.py:151-170) or from the Pallas backward kernels behind
+// attention.py:121-123 / 144-150.  With P = exp(sm_scale*QK^T - LSE), delta = rowsum(dO o O):
+//     dV = P^T dO;  dS = P o (dO V^T - delta);  dQ = sm_scale dS K;  dK = sm_scale dS^T Q
+// and dK, dV summed over the n_rep query heads that share a KV head.
+//
+// Three kernels:
+//   attn_delta_kernel     delta[b,h,i] = sum_d dO*O                                   (HBM-bound)
+//   attn_bwd_dkdv_kernel  one workgroup = 128 KV rows of one (batch, kv head); K and V fragments stay
+//                         in registers, Q / dO tiles of every query head of the group stream through
+//                         LDS in both orientations (row-major for S = QK^T and dP = dO V^T, transposed
+//                         for dV^T += dO^T P and dK^T += Q^T dS).  S is computed un-transposed here so
+//                         that a lane owns one KV column: P and dS converted to 16 bit are directly the
+//                         B operands of the two accumulating products.
+//   attn_bwd_dq_kernel    one workgroup = 128 query rows of one (batch, head); Q and dO fragments in
+//                         registers, K (row-major + transposed) and V (row-major) tiles stream through
+//                         LDS; S^T, dP^T are computed transposed (a lane owns one query column, so LSE
+//                         and delta are per-lane scalars) and dS^T feeds dQ^T += K^T dS^T.
+// Splitting dQ from dK/dV recomputes S and dP once more but needs no atomics: fp32 atomic adds reach
+// about 1.3 TB/s on this part, an order of magnitude short of what accumulating dQ tiles would need.
+#include "attn_common.hpp"
+
+namespace tp {
+
+struct BwdArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* out;
+  const void* dout;
+  const float* lse;
+  const int32_t* seg;
+  void* dq;
+  void* dk;
+  void* dv;
+  float* delta;
+  int B, Hq, Hkv, Sq, Skv, n_rep;
+  int64_t qs[3], ks[3], vs[3], os[3], dos[3], dqs[3], dks[3], dvs[3];
+  float scale_log2;  // sm_scale * log2(e)
+  float sm_scale;
+};
+
+// ------------------------------------------------------------------------------------------------
+// delta = rowsum(dO o O)
+// ------------------------------------------------------------------------------------------------
+template <typename T, int DV>
+__global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
+  constexpr int TPR = DV / 8;  // threads per row, one 16-byte chunk each
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t total = (int64_t)a.B * a.Hq * a.Sq;
+  int64_t rowid = idx / TPR;
+  const int ch = (int)(idx % TPR);
+  const bool valid = rowid < total;
+  if (!valid) rowid = total - 1;
+  const int s = (int)(rowid % a.Sq);
+  const int64_t bh = rowid / a.Sq;
+  const int h = (int)(bh % a.Hq), b = (int)(bh / a.Hq);
+  float o[8], g[8];
+  load_f<T, 8>((const T*)a.out + b * a.os[0] + h * a.os[1] + s * a.os[2] + ch * 8, o);
+  load_f<T, 8>((const T*)a.dout + b * a.dos[0] + h * a.dos[1] + s * a.dos[2] + ch * 8, g);
+  float acc = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) acc += o[e] * g[e];
+#pragma unroll
+  for (int off = TPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+  if (valid && ch == 0) a.delta[rowid] = acc;
+}
+
+// ------------------------------------------------------------------------------------------------
+// staging helpers: a tile of 64 rows x D 16-bit elements, each thread owning 4-row x 8-column blocks
+// so that one set of global loads serves both the row-major and the transposed LDS copy
+// ------------------------------------------------------------------------------------------------
+template <int D>
+struct Stage64 {
+  static constexpr int TOT = (D / 8) * 16;       // 4x8 blocks in the tile
+  static constexpr int ITEMS = (TOT + 255) / 256;
+  u32x4 r[ITEMS][4];
+
+  template <typename T>
+  __device__ __forceinline__ void load(const T* base, int64_t row_stride, int row0, int row_max, int tid) {
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+      const int item = tid + 256 * i;
+      if (item < TOT) {
+        const int c8 = item % (D / 8), rq = item / (D / 8);
+#pragma unroll
+        for (int ii = 0; ii < 4; ii++) {
+          const int row = min(row0 + 4 * rq + ii, row_max);
+          r[i][ii] = *(const u32x4*)(base + row * row_stride + c8 * 8);
+        }
+      }
+    }
+  }
+  __device__ __forceinline__ void store_rowmajor(unsigned char* dst, int tid) const {
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+      const int item = tid + 256 * i;
+      if (item < TOT) {
+        const int c8 = item % (D / 8), rq = item / (D / 8);
+#pragma unroll
+        for (int ii = 0; ii < 4; ii++) *(u32x4*)(dst + RowTile<D>::off(4 * rq + ii, c8 * 8)) = r[i][ii];
+      }
+    }
+  }
+  __device__ __forceinline__ void store_transposed(unsigned char* dst, int tid) const {
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+      const int item = tid + 256 * i;
+      if (item < TOT) {
+        const int c8 = item % (D / 8), rq = item / (D / 8);
+#pragma unroll
+        for (int j = 0; j < 8; j++) *(u32x2*)(dst + TrTile64::quad_off(c8 * 8 + j, rq)) = transpose_col(r[i], j);
+      }
+    }
+  }
+};
+
+// per-tile [min,max] of segment ids for 64-row tiles t0..t1-1 into LDS (lane = row of the tile)
+__device__ __forceinline__ void seg_tile_ranges(const int32_t* segb, int S, int t0, int t1, int* tmin, int* tmax,
+                                                int wave, int lane) {
+  for (int t = t0 + wave; t < t1; t += 4) {
+    int lo = segb[min(t * 64 + lane, S - 1)], hi = lo;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      lo = min(lo, __shfl_xor(lo, o, 64));
+      hi = max(hi, __shfl_xor(hi, o, 64));
+    }
+    if (lane == 0) { tmin[t - t0] = lo; tmax[t - t0] = hi; }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// dK / dV
+// ------------------------------------------------------------------------------------------------
+template <typename T, int DQK, int DV, int NBUF, bool CAUSAL, bool SEG>
+__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
+  typedef typename MT<T>::v8 v8;
+  constexpr int BMQ = 64;   // query rows per streamed tile
+  constexpr int BNK = 128;  // kv rows per workgroup, 32 per wave
+  constexpr int QB = BMQ / 32;
+  constexpr int KS_QK = DQK / 16, KS_DV = DV / 16;
+  constexpr int DKB = DQK / 32, DVB = DV / 32;
+  typedef RowTile<DQK> QT;
+  typedef RowTile<DV> OT;
+  constexpr int Q_BYTES = BMQ * QT::STRIDE, DO_BYTES = BMQ * OT::STRIDE;
+  constexpr int QTR_BYTES = DQK * TrTile64::ROW_BYTES, DOTR_BYTES = DV * TrTile64::ROW_BYTES;
+  constexpr int ROW_BYTES = BMQ * 4 * 3;  // lse (log2 units), delta, segment id per query row
+  constexpr int BUF_BYTES = Q_BYTES + DO_BYTES + QTR_BYTES + DOTR_BYTES + ROW_BYTES;
+
+  extern __shared__ __align__(16) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, ln = lane & 31;
+  const int hk = blockIdx.y, b = blockIdx.z;
+  const int kv0 = blockIdx.x * BNK;
+  const int wkv0 = kv0 + wave * 32;
+  const int Sq = a.Sq, Skv = a.Skv;
+  const int32_t* segb = SEG ? a.seg + (int64_t)b * Skv : nullptr;
+
+  // ---- K, V fragments of this wave's 32 kv rows (B operands: lane = kv column)
+  v8 kf[KS_QK], vf[KS_DV];
+  const int kvrow = min(wkv0 + ln, Skv - 1);
+  {
+    const T* kp = (const T*)a.k + b * a.ks[0] + hk * a.ks[1] + kvrow * a.ks[2] + 8 * g;
+    const T* vp = (const T*)a.v + b * a.vs[0] + hk * a.vs[1] + kvrow * a.vs[2] + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS_QK; ks++) kf[ks] = *(const v8*)(kp + 16 * ks);
+#pragma unroll
+    for (int ks = 0; ks < KS_DV; ks++) vf[ks] = *(const v8*)(vp + 16 * ks);
+  }
+  const int segk = SEG ? segb[kvrow] : 0;
+
+  // ---- query tiles to visit: causal => tiles that reach the first kv row; segments => id ranges overlap
+  const int nqt_all = (Sq + BMQ - 1) / BMQ;
+  const int qt_first = CAUSAL ? min(kv0 / BMQ, nqt_all) : 0;
+  const int nqt = nqt_all - qt_first;
+  int* qmin = (int*)(smem + NBUF * BUF_BYTES);
+  int* qmax = qmin + nqt;
+  int* active = qmax + nqt;
+  int* bk = active + nqt;  // 8 ints: per-wave (min,max) of kv ids
+  int nact = nqt;
+  int wkmin = 0, wkmax = 0;
+  if (SEG) {
+    wkmin = segk; wkmax = segk;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) {
+      wkmin = min(wkmin, __shfl_xor(wkmin, o, 64));
+      wkmax = max(wkmax, __shfl_xor(wkmax, o, 64));
+    }
+    wkmin = __builtin_amdgcn_readfirstlane(wkmin);
+    wkmax = __builtin_amdgcn_readfirstlane(wkmax);
+    if (lane == 0) { bk[2 * wave] = wkmin; bk[2 * wave + 1] = wkmax; }
+    seg_tile_ranges(segb, Sq, qt_first, nqt_all, qmin, qmax, wave, lane);
+    __syncthreads();
+    const int bkmin = min(min(bk[0], bk[2]), min(bk[4], bk[6]));
+    const int bkmax = max(max(bk[1], bk[3]), max(bk[5], bk[7]));
+    int cnt = 0;
+    for (int base = 0; base < nqt; base += 64) {
+      const int t = base + lane;
+      const bool act = t < nqt && !(qmax[t] < bkmin || qmin[t] > bkmax);
+      const unsigned long long m = __ballot(act);
+      if (act && wave == 0) active[cnt + __popcll(m & ((1ull << lane) - 1ull))] = t;
+      cnt += __popcll(m);
+    }
+    nact = cnt;
+    __syncthreads();
+  }
+  const int n_iter = nact * a.n_rep;
+
+  // ---- staging
+  Stage64<DQK> qst;
+  Stage64<DV> dost;
+  float lse_r = 0.f, delta_r = 0.f;
+  int segq_r = 0;
+  auto tile_of = [&](int it, int& hq, int& qi0) {
+    const int hl = it / nact, idx = it - hl * nact;
+    hq = hk * a.n_rep + hl;
+    qi0 = (qt_first + (SEG ? active[idx] : idx)) * BMQ;
+  };
+  auto load_tile = [&](int it) {
+    int hq, qi0;
+    tile_of(it, hq, qi0);
+    qst.load((const T*)a.q + b * a.qs[0] + hq * a.qs[1], a.qs[2], qi0, Sq - 1, tid);
+    dost.load((const T*)a.dout + b * a.dos[0] + hq * a.dos[1], a.dos[2], qi0, Sq - 1, tid);
+    if (tid < BMQ) {
+      const int row = min(qi0 + tid, Sq - 1);
+      const int64_t ro = ((int64_t)b * a.Hq + hq) * Sq + row;
+      const float l = a.lse[ro];
+      lse_r = (l == -INFINITY) ? INFINITY : l * LOG2E;  // a row with no allowed key gets P = 0
+      delta_r = a.delta[ro];
+      if (SEG) segq_r = segb[row];
+    }
+  };
+  auto store_tile = [&](int buf) {
+    unsigned char* base = smem + buf * BUF_BYTES;
+    qst.store_rowmajor(base, tid);
+    dost.store_rowmajor(base + Q_BYTES, tid);
+    qst.store_transposed(base + Q_BYTES + DO_BYTES, tid);
+    dost.store_transposed(base + Q_BYTES + DO_BYTES + QTR_BYTES, tid);
+    if (tid < BMQ) {
+      float* rf = (float*)(base + Q_BYTES + DO_BYTES + QTR_BYTES + DOTR_BYTES);
+      rf[tid] = lse_r;
+      rf[BMQ + tid] = delta_r;
+      ((int*)rf)[2 * BMQ + tid] = segq_r;
+    }
+  };
+
+  f32x16 dkacc[DKB], dvacc[DVB];
+#pragma unroll
+  for (int d = 0; d < DKB; d++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) dkacc[d][v] = 0.f;
+#pragma unroll
+  for (int d = 0; d < DVB; d++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) dvacc[d][v] = 0.f;
+  const float c = a.scale_log2;
+
+  if (n_iter > 0) {
+    load_tile(0);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  for (int it = 0; it < n_iter; it++) {
+    const int buf = NBUF == 2 ? (it & 1) : 0;
+    int hq, qi0;
+    tile_of(it, hq, qi0);
+    if (it + 1 < n_iter) load_tile(it + 1);
+
+    const unsigned char* ql = smem + buf * BUF_BYTES;
+    const unsigned char* dol = ql + Q_BYTES;
+    const unsigned char* qtl = dol + DO_BYTES;
+    const unsigned char* dotl = qtl + QTR_BYTES;
+    const float* lsel = (const float*)(dotl + DOTR_BYTES);
+    const float* deltal = lsel + BMQ;
+    const int* segl = (const int*)(deltal + BMQ);
+
+    // wave-level decisions (uniform): nothing to do if every query row precedes every kv row
+    bool skip = (CAUSAL && qi0 + BMQ - 1 < wkv0) || wkv0 >= Skv;
+    bool need_mask = (qi0 + BMQ > Sq) || (wkv0 + 32 > Skv) || (CAUSAL && qi0 < wkv0 + 31);
+    if (SEG) {
+      const int idx = it % nact;
+      const int lo = qmin[active[idx]], hi = qmax[active[idx]];
+      skip = skip || hi < wkmin || lo > wkmax;
+      need_mask = need_mask || !(lo == hi && wkmin == wkmax && lo == wkmin);
+    }
+    if (!skip) {
+      f32x16 sacc[QB], dpacc[QB];
+#pragma unroll
+      for (int qb = 0; qb < QB; qb++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) { sacc[qb][v] = 0.f; dpacc[qb][v] = 0.f; }
+      // S = Q K^T  (rows = queries, columns = this wave's kv rows)
+#pragma unroll
+      for (int ks = 0; ks < KS_QK; ks++)
+#pragma unroll
+        for (int qb = 0; qb < QB; qb++) {
+          const v8 qf = *(const v8*)(ql + QT::off(qb * 32 + ln, 16 * ks + 8 * g));
+          sacc[qb] = MT<T>::mfma32(qf, kf[ks], sacc[qb]);
+        }
+      // dP = dO V^T
+#pragma unroll
+      for (int ks = 0; ks < KS_DV; ks++)
+#pragma unroll
+        for (int qb = 0; qb < QB; qb++) {
+          const v8 dof = *(const v8*)(dol + OT::off(qb * 32 + ln, 16 * ks + 8 * g));
+          dpacc[qb] = MT<T>::mfma32(dof, vf[ks], dpacc[qb]);
+        }
+      // P = exp2(S*c - lse), dS = P o (dP - delta); rows of the C tile are queries
+      v8 pfr[BMQ / 16], dsf[BMQ / 16];
+      const int kvcol = wkv0 + ln;
+#pragma unroll
+      for (int qb = 0; qb < QB; qb++) {
+#pragma unroll
+        for (int vq = 0; vq < 4; vq++) {
+          const int r0 = qb * 32 + 8 * vq + 4 * g;
+          const f32x4 l4 = *(const f32x4*)(lsel + r0);
+          const f32x4 d4 = *(const f32x4*)(deltal + r0);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const int v = 4 * vq + e;
+            float p = fast_exp2(__builtin_fmaf(sacc[qb][v], c, -l4[e]));
+            if (need_mask) {
+              const int qrow = qi0 + r0 + e;
+              const bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || segl[r0 + e] == segk);
+              p = ok ? p : 0.f;
+            }
+            sacc[qb][v] = p;
+            dpacc[qb][v] = p * (dpacc[qb][v] - d4[e]);
+          }
+        }
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++) {
+          const f32x16& s = sacc[qb];
+          const f32x16& d = dpacc[qb];
+          pfr[qb * 2 + hh] = pack8<T>(s[8 * hh + 0], s[8 * hh + 1], s[8 * hh + 2], s[8 * hh + 3], s[8 * hh + 4],
+                                      s[8 * hh + 5], s[8 * hh + 6], s[8 * hh + 7]);
+          dsf[qb * 2 + hh] = pack8<T>(d[8 * hh + 0], d[8 * hh + 1], d[8 * hh + 2], d[8 * hh + 3], d[8 * hh + 4],
+                                      d[8 * hh + 5], d[8 * hh + 6], d[8 * hh + 7]);
+        }
+      }
+      // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 64 query rows)
+#pragma unroll
+      for (int ks = 0; ks < BMQ / 16; ks++) {
+#pragma unroll
+        for (int d = 0; d < DVB; d++) {
+          const v8 f = *(const v8*)(dotl + TrTile64::chunk_off(d * 32 + ln, ks, g));
+          dvacc[d] = MT<T>::mfma32(f, pfr[ks], dvacc[d]);
+        }
+#pragma unroll
+        for (int d = 0; d < DKB; d++) {
+          const v8 f = *(const v8*)(qtl + TrTile64::chunk_off(d * 32 + ln, ks, g));
+          dkacc[d] = MT<T>::mfma32(f, dsf[ks], dkacc[d]);
+        }
+      }
+    }
+    if (NBUF == 1) __syncthreads();
+    if (it + 1 < n_iter) store_tile(NBUF == 2 ? (buf ^ 1) : 0);
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane = kv row, 4 consecutive head-dim values per store
+  const int row = wkv0 + ln;
+  if (row < Skv) {
+    T* dkp = (T*)a.dk + b * a.dks[0] + hk * a.dks[1] + row * a.dks[2];
+    T* dvp = (T*)a.dv + b * a.dvs[0] + hk * a.dvs[1] + row * a.dvs[2];
+    const float sc = a.sm_scale;
+#pragma unroll
+    for (int d = 0; d < DKB; d++)
+#pragma unroll
+      for (int vq = 0; vq < 4; vq++) {
+        const f32x16& o = dkacc[d];
+        *(u32x2*)(dkp + d * 32 + 8 * vq + 4 * g) =
+            pack4<T>(o[4 * vq] * sc, o[4 * vq + 1] * sc, o[4 * vq + 2] * sc, o[4 * vq + 3] * sc);
+      }
+#pragma unroll
+    for (int d = 0; d < DVB; d++)
+#pragma unroll
+      for (int vq = 0; vq < 4; vq++) {
+        const f32x16& o = dvacc[d];
+        *(u32x2*)(dvp + d * 32 + 8 * vq + 4 * g) = pack4<T>(o[4 * vq], o[4 * vq + 1], o[4 * vq + 2], o[4 * vq + 3]);
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// dQ
+// ------------------------------------------------------------------------------------------------
+template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
+__global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
+  typedef typename MT<T>::v8 v8;
+  constexpr int BN = 64, BM = 128, NB = BN / 32;
+  constexpr int KS_QK = DQK / 16, KS_DV = DV / 16, DKB = DQK / 32;
+  typedef RowTile<DQK> KT;
+  typedef RowTile<DV> VT;
+  constexpr int K_BYTES = BN * KT::STRIDE, V_BYTES = BN * VT::STRIDE, KTR_BYTES = DQK * TrTile64::ROW_BYTES;
+  constexpr int BUF_BYTES = K_BYTES + V_BYTES + KTR_BYTES + BN * 4;
+  constexpr int VCH = DV / 8, V_ITEMS = BN * VCH / 256;
+
+  extern __shared__ __align__(16) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, ln = lane & 31;
+  const int qt = gridDim.x - 1 - blockIdx.x;
+  const int h = blockIdx.y, b = blockIdx.z, hk = h / a.n_rep;
+  const int q0 = qt * BM, wq0 = q0 + wave * 32;
+  const int Sq = a.Sq, Skv = a.Skv;
+  const T* kb = (const T*)a.k + b * a.ks[0] + hk * a.ks[1];
+  const T* vb = (const T*)a.v + b * a.vs[0] + hk * a.vs[1];
+  const int32_t* segb = SEG ? a.seg + (int64_t)b * Skv : nullptr;
+
+  const int kv_end = CAUSAL ? min(Skv, q0 + BM) : Skv;
+  const int ntiles = (kv_end + BN - 1) / BN;
+
+  // ---- Q, dO fragments (B operands: lane = query column), per-lane LSE / delta
+  const int qrow_c = min(wq0 + ln, Sq - 1);
+  v8 qf[KS_QK], dof[KS_DV];
+  {
+    const T* qp = (const T*)a.q + b * a.qs[0] + h * a.qs[1] + qrow_c * a.qs[2] + 8 * g;
+    const T* dp = (const T*)a.dout + b * a.dos[0] + h * a.dos[1] + qrow_c * a.dos[2] + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS_QK; ks++) qf[ks] = *(const v8*)(qp + 16 * ks);
+#pragma unroll
+    for (int ks = 0; ks < KS_DV; ks++) dof[ks] = *(const v8*)(dp + 16 * ks);
+  }
+  const int64_t ro = ((int64_t)b * a.Hq + h) * Sq + qrow_c;
+  const float lraw = a.lse[ro];
+  const float lse_s = (lraw == -INFINITY) ? INFINITY : lraw * LOG2E;
+  const float delta_s = a.delta[ro];
+  const int segq = SEG ? segb[qrow_c] : 0;
+
+  int* kvmin = (int*)(smem + 2 * BUF_BYTES);
+  int* kvmax = kvmin + ntiles;
+  int* active = kvmax + ntiles;
+  int* bq = active + ntiles;
+  int nact = ntiles;
+  int wqmin = 0, wqmax = 0;
+  if (SEG) {
+    wqmin = segq; wqmax = segq;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) {
+      wqmin = min(wqmin, __shfl_xor(wqmin, o, 64));
+      wqmax = max(wqmax, __shfl_xor(wqmax, o, 64));
+    }
+    wqmin = __builtin_amdgcn_readfirstlane(wqmin);
+    wqmax = __builtin_amdgcn_readfirstlane(wqmax);
+    if (lane == 0) { bq[2 * wave] = wqmin; bq[2 * wave + 1] = wqmax; }
+    seg_tile_ranges(segb, Skv, 0, ntiles, kvmin, kvmax, wave, lane);
+    __syncthreads();
+    const int bqmin = min(min(bq[0], bq[2]), min(bq[4], bq[6]));
+    const int bqmax = max(max(bq[1], bq[3]), max(bq[5], bq[7]));
+    int cnt = 0;
+    for (int base = 0; base < ntiles; base += 64) {
+      const int t = base + lane;
+      const bool act = t < ntiles && !(kvmax[t] < bqmin || kvmin[t] > bqmax);
+      const unsigned long long m = __ballot(act);
+      if (act && wave == 0) active[cnt + __popcll(m & ((1ull << lane) - 1ull))] = t;
+      cnt += __popcll(m);
+    }
+    nact = cnt;
+    __syncthreads();
+  }
+
+  Stage64<DQK> kst;
+  u32x4 vreg[V_ITEMS];
+  int sreg = 0;
+  auto load_tile = [&](int t) {
+    const int kv0 = t * BN;
+    kst.load(kb, a.ks[2], kv0, Skv - 1, tid);
+#pragma unroll
+    for (int i = 0; i < V_ITEMS; i++) {
+      const int item = tid + 256 * i;
+      const int row = min(kv0 + item / VCH, Skv - 1), ch = item % VCH;
+      vreg[i] = *(const u32x4*)(vb + row * a.vs[2] + ch * 8);
+    }
+    if (SEG && tid < BN) sreg = segb[min(kv0 + tid, Skv - 1)];
+  };
+  auto store_tile = [&](int buf) {
+    unsigned char* base = smem + buf * BUF_BYTES;
+    kst.store_rowmajor(base, tid);
+#pragma unroll
+    for (int i = 0; i < V_ITEMS; i++) {
+      const int item = tid + 256 * i;
+      *(u32x4*)(base + K_BYTES + VT::off(item / VCH, (item % VCH) * 8)) = vreg[i];
+    }
+    kst.store_transposed(base + K_BYTES + V_BYTES, tid);
+    if (SEG && tid < BN) ((int*)(base + K_BYTES + V_BYTES + KTR_BYTES))[tid] = sreg;
+  };
+
+  f32x16 dqacc[DKB];
+#pragma unroll
+  for (int d = 0; d < DKB; d++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) dqacc[d][v] = 0.f;
+  const float c = a.scale_log2;
+  const int wq_last = wq0 + 31;
+  const int qrow = wq0 + ln;
+
+  if (nact > 0) {
+    load_tile(SEG ? active[0] : 0);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  for (int it = 0; it < nact; it++) {
+    const int t = SEG ? active[it] : it;
+    const int kv0 = t * BN;
+    const int buf = it & 1;
+    if (it + 1 < nact) load_tile(SEG ? active[it + 1] : it + 1);
+
+    const unsigned char* kl = smem + buf * BUF_BYTES;
+    const unsigned char* vl = kl + K_BYTES;
+    const unsigned char* ktl = vl + V_BYTES;
+    const int* sl = (const int*)(ktl + KTR_BYTES);
+
+    bool skip = CAUSAL && kv0 > wq_last;
+    bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0);
+    if (SEG) {
+      const int lo = kvmin[t], hi = kvmax[t];
+      skip = skip || hi < wqmin || lo > wqmax;
+      need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
+    }
+    if (!skip) {
+      f32x16 sacc[NB], dpacc[NB];
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) { sacc[nb][v] = 0.f; dpacc[nb][v] = 0.f; }
+      // S^T = K Q^T, dP^T = V dO^T  (rows = kv, columns = this wave's queries)
+#pragma unroll
+      for (int ks = 0; ks < KS_QK; ks++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+          const v8 f = *(const v8*)(kl + KT::off(nb * 32 + ln, 16 * ks + 8 * g));
+          sacc[nb] = MT<T>::mfma32(f, qf[ks], sacc[nb]);
+        }
+#pragma unroll
+      for (int ks = 0; ks < KS_DV; ks++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) {
+          const v8 f = *(const v8*)(vl + VT::off(nb * 32 + ln, 16 * ks + 8 * g));
+          dpacc[nb] = MT<T>::mfma32(f, dof[ks], dpacc[nb]);
+        }
+      v8 dsf[BN / 16];
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          float p = fast_exp2(__builtin_fmaf(sacc[nb][v], c, -lse_s));
+          if (need_mask) {
+            const int kvl = nb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
+            const int kv = kv0 + kvl;
+            const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
+            p = ok ? p : 0.f;
+          }
+          dpacc[nb][v] = p * (dpacc[nb][v] - delta_s);
+        }
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++) {
+          const f32x16& d = dpacc[nb];
+          dsf[nb * 2 + hh] = pack8<T>(d[8 * hh + 0], d[8 * hh + 1], d[8 * hh + 2], d[8 * hh + 3], d[8 * hh + 4],
+                                      d[8 * hh + 5], d[8 * hh + 6], d[8 * hh + 7]);
+        }
+      }
+      // dQ^T += K^T dS^T  (contraction over the 64 kv rows)
+#pragma unroll
+      for (int ks = 0; ks < BN / 16; ks++)
+#pragma unroll
+        for (int d = 0; d < DKB; d++) {
+          const v8 f = *(const v8*)(ktl + TrTile64::chunk_off(d * 32 + ln, ks, g));
+          dqacc[d] = MT<T>::mfma32(f, dsf[ks], dqacc[d]);
+        }
+    }
+    if (it + 1 < nact) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  if (qrow < Sq) {
+    T* dqp = (T*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qrow * a.dqs[2];
+    const float sc = a.sm_scale;
+#pragma unroll
+    for (int d = 0; d < DKB; d++)
+#pragma unroll
+      for (int vq = 0; vq < 4; vq++) {
+        const f32x16& o = dqacc[d];
+        *(u32x2*)(dqp + d * 32 + 8 * vq + 4 * g) =
+            pack4<T>(o[4 * vq] * sc, o[4 * vq + 1] * sc, o[4 * vq + 2] * sc, o[4 * vq + 3] * sc);
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host dispatch
+// ------------------------------------------------------------------------------------------------
+template <typename K>
+static int set_max_lds(K kern, const char* what) {
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  TP_REQUIRE(e == hipSuccess, TP_ERR_LAUNCH, "%s: hipFuncSetAttribute failed: %s", what, hipGetErrorString(e));
+  return TP_OK;
+}
+
+template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
+static int launch_bwd(const BwdArgs& a, hipStream_t st) {
+  // delta
+  {
+    const int64_t threads = (int64_t)a.B * a.Hq * a.Sq * (DV / 8);
+    attn_delta_kernel<T, DV><<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st>>>(a);
+    int rc = check_launch("tp_attn_bwd(delta)");
+    if (rc) return rc;
+  }
+  // dK, dV
+  {
+    constexpr int BMQ = 64, BNK = 128;
+    constexpr int BUF = BMQ * RowTile<DQK>::STRIDE + BMQ * RowTile<DV>::STRIDE + (DQK + DV) * TrTile64::ROW_BYTES + BMQ * 12;
+    constexpr int NBUF = (2 * BUF + 4096 <= 160 * 1024) ? 2 : 1;
+    const int nqt = (a.Sq + BMQ - 1) / BMQ;
+    const size_t smem = (size_t)NBUF * BUF + (SEG ? (size_t)(3 * nqt + 8) * 4 : 0);
+    TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_bwd: Sq=%d needs %zu bytes of LDS (max 163840)", a.Sq, smem);
+    auto kern = attn_bwd_dkdv_kernel<T, DQK, DV, NBUF, CAUSAL, SEG>;
+    static bool attr_set = false;
+    if (!attr_set) {
+      int rc = set_max_lds(kern, "tp_attn_bwd(dkdv)");
+      if (rc) return rc;
+      attr_set = true;
+    }
+    kern<<<dim3((a.Skv + BNK - 1) / BNK, a.Hkv, a.B), dim3(256), smem, st>>>(a);
+    int rc = check_launch("tp_attn_bwd(dkdv)");
+    if (rc) return rc;
+  }
+  // dQ
+  {
+    constexpr int BN = 64, BM = 128;
+    constexpr int BUF = BN * RowTile<DQK>::STRIDE + BN * RowTile<DV>::STRIDE + DQK * TrTile64::ROW_BYTES + BN * 4;
+    const int nt = (a.Skv + BN - 1) / BN;
+    const size_t smem = 2 * (size_t)BUF + (SEG ? (size_t)(3 * nt + 8) * 4 : 0);
+    TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_bwd: Skv=%d needs %zu bytes of LDS (max 163840)", a.Skv, smem);
+    auto kern = attn_bwd_dq_kernel<T, DQK, DV, CAUSAL, SEG>;
+    static bool attr_set = false;
+    if (!attr_set) {
+      int rc = set_max_lds(kern, "tp_attn_bwd(dq)");
+      if (rc) return rc;
+      attr_set = true;
+    }
+    kern<<<dim3((a.Sq + BM - 1) / BM, a.Hq, a.B), dim3(256), smem, st>>>(a);
+    return check_launch("tp_attn_bwd(dq)");
+  }
+}
+
+template <typename T, int DQK, int DV>
+static int dispatch_bwd(const BwdArgs& a, int causal, hipStream_t st) {
+  if (causal) {
+    if (a.seg) return launch_bwd<T, DQK, DV, true, true>(a, st);
+    return launch_bwd<T, DQK, DV, true, false>(a, st);
+  }
+  if (a.seg) return launch_bwd<T, DQK, DV, false, true>(a, st);
+  return launch_bwd<T, DQK, DV, false, false>(a, st);
+}
+
+}  // namespace tp
+
+using namespace tp;
+
+extern "C" size_t tp_attn_bwd_workspace_bytes(int B, int Hq, int Sq) {
+  if (B <= 0 || Hq <= 0 || Sq <= 0) return 0;
+  return (size_t)B * Hq * Sq * sizeof(float);
+}
+
+extern "C" int tp_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                           const float* lse, const int32_t* seg, void* dq, void* dk, void* dv, float* ws, int B, int Hq,
+                           int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t do_strides[3],
+                           const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                           const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                           const int64_t dv_strides[3], float sm_scale, int causal, int dtype, void* stream) {
+  TP_REQUIRE(dout && q && k && v && out && lse && dq && dk && dv && ws, TP_ERR_BAD_ARG, "tp_attn_bwd: null pointer");
+  TP_REQUIRE(do_strides && q_strides && k_strides && v_strides && o_strides && dq_strides && dk_strides && dv_strides,
+             TP_ERR_BAD_ARG, "tp_attn_bwd: null stride array");
+  TP_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Sq > 0 && Skv > 0, TP_ERR_BAD_ARG, "tp_attn_bwd: non-positive size");
+  TP_REQUIRE(Hq % Hkv == 0, TP_ERR_BAD_ARG, "tp_attn_bwd: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
+  TP_REQUIRE(!seg || Sq == Skv, TP_ERR_BAD_ARG, "tp_attn_bwd: segment ids need Sq == Skv (got %d, %d)", Sq, Skv);
+  TP_REQUIRE(sm_scale > 0.f, TP_ERR_BAD_ARG, "tp_attn_bwd: sm_scale must be positive");
+  TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F16, TP_ERR_UNSUPPORTED, "tp_attn_bwd: dtype %d (bf16 and fp16 only)", dtype);
+  TP_REQUIRE(B <= 65535 && Hq <= 65535, TP_ERR_UNSUPPORTED, "tp_attn_bwd: batch and heads are limited to 65535");
+  BwdArgs a;
+  a.q = q; a.k = k; a.v = v; a.out = out; a.dout = dout; a.lse = lse; a.seg = seg;
+  a.dq = dq; a.dk = dk; a.dv = dv; a.delta = ws;
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.Sq = Sq; a.Skv = Skv; a.n_rep = Hq / Hkv;
+  bool ok = aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out) && aligned16(dout) && aligned16(dq) &&
+            aligned16(dk) && aligned16(dv);
+  for (int i = 0; i < 3; i++) {
+    a.qs[i] = q_strides[i]; a.ks[i] = k_strides[i]; a.vs[i] = v_strides[i]; a.os[i] = o_strides[i];
+    a.dos[i] = do_strides[i]; a.dqs[i] = dq_strides[i]; a.dks[i] = dk_strides[i]; a.dvs[i] = dv_strides[i];
+    ok = ok && q_strides[i] % 8 == 0 && k_strides[i] % 8 == 0 && v_strides[i] % 8 == 0 && o_strides[i] % 8 == 0 &&
+         do_strides[i] % 8 == 0 && dq_strides[i] % 4 == 0 && dk_strides[i] % 4 == 0 && dv_strides[i] % 4 == 0;
+  }
+  TP_REQUIRE(ok, TP_ERR_BAD_ARG, "tp_attn_bwd: pointers and strides must keep rows 16-byte aligned");
+  a.scale_log2 = sm_scale * LOG2E;
+  a.sm_scale = sm_scale;
+  hipStream_t st = (hipStream_t)stream;
+#define TP_BWD(T, DQ, DVV) return dispatch_bwd<T, DQ, DVV>(a, causal, st)
+  if (dtype == TP_BF16) {
+    if (Dqk == 128 && Dv == 128) TP_BWD(bf16_t, 128, 128);
+    if (Dqk == 64 && Dv == 64) TP_BWD(bf16_t, 64, 64);
+    if (Dqk == 192 && Dv == 128) TP_BWD(bf16_t, 192, 128);
+  } else {
+    if (Dqk == 128 && Dv == 128) TP_BWD(f16_t, 128, 128);
+    if (Dqk == 64 && Dv == 64) TP_BWD(f16_t, 64, 64);
+    if (Dqk == 192 && Dv == 128) TP_BWD(f16_t, 192, 128);
+  }
+#undef TP_BWD
+  TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_attn_bwd: head dims (qk=%d, v=%d) not built", Dqk, Dv);
+}

@@ -1,0 +1,119 @@
+// Shared pieces of the attention kernels: MFMA wrappers, fragment packing, LDS tile layouts.
+//
+// MFMA operand layouts used throughout (v_mfma_f32_32x32x16_{bf16,f16}, wave64; ln = lane % 32,
+// g = lane / 32):
+//   A (32 x 16): lane holds row ln,    k = 8*g + 0..7
+//   B (16 x 32): lane holds column ln, k = 8*g + 0..7
+//   C (32 x 32): lane holds column ln, rows 8*(v/4) + 4*g + v%4 for v = 0..15
+// The hardware pairs A and B element-for-element inside a lane group g, so any ordering of the 16
+// k-values works as long as both operands use the same one.  The kernels exploit that when a C tile
+// (lane <-> column) is fed back as a B operand: its values v = 8h..8h+7 cover rows
+// 16h + 8a + 4g + e (a = 0..1, e = 0..3), and the other operand is laid out in LDS so that a lane's
+// 16 bytes hold exactly those rows ("quad-swapped" order, see vt_offset).
+#pragma once
+#include "common.hpp"
+
+namespace tp {
+
+template <typename T> struct MT;
+template <> struct MT<bf16_t> {
+  typedef bf16x8 v8;
+  typedef bf16x2 v2;
+  static __device__ __forceinline__ f32x16 mfma32(v8 a, v8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct MT<f16_t> {
+  typedef f16x8 v8;
+  typedef f16x2 v2;
+  static __device__ __forceinline__ f32x16 mfma32(v8 a, v8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+// eight floats -> one 16-byte MFMA operand (round to nearest even)
+template <typename T>
+__device__ __forceinline__ typename MT<T>::v8 pack8(float a0, float a1, float a2, float a3, float a4, float a5,
+                                                    float a6, float a7) {
+  typename MT<T>::v8 r;
+  r[0] = (T)a0; r[1] = (T)a1; r[2] = (T)a2; r[3] = (T)a3;
+  r[4] = (T)a4; r[5] = (T)a5; r[6] = (T)a6; r[7] = (T)a7;
+  return r;
+}
+// four floats -> 8 bytes
+template <typename T>
+__device__ __forceinline__ u32x2 pack4(float a0, float a1, float a2, float a3) {
+  typedef T v4 __attribute__((ext_vector_type(4)));
+  v4 r;
+  r[0] = (T)a0; r[1] = (T)a1; r[2] = (T)a2; r[3] = (T)a3;
+  return __builtin_bit_cast(u32x2, r);
+}
+
+// Combine a value with the one held by the partner lane (lane ^ 32): max / sum across the two
+// half-waves.  v_permlane32_swap(old, src) returns x = {old.lo, src.lo}, y = {old.hi, src.hi}; with
+// old = src = v every lane gets its own half's value in one of x / y and the partner's in the other.
+// The elements are copied to scalars before the bit casts: __builtin_bit_cast applied directly to a
+// vector element expression (r.y) reads element 0 with this compiler.
+__device__ __forceinline__ void half_swap(float v, float& lo, float& hi) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  const u32x2 r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned x = r.x, y = r.y;
+  lo = __builtin_bit_cast(float, x);
+  hi = __builtin_bit_cast(float, y);
+}
+__device__ __forceinline__ float half_max(float v) {
+  float lo, hi;
+  half_swap(v, lo, hi);
+  return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float half_sum(float v) {
+  float lo, hi;
+  half_swap(v, lo, hi);
+  return lo + hi;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+// ---- LDS layouts ---------------------------------------------------------------------------------
+// Row-major tile [rows][D] of 16-bit elements: rows padded by 16 bytes so that 16-byte reads by lanes
+// in consecutive rows land in different banks.
+template <int D> struct RowTile {
+  static constexpr int STRIDE = D * 2 + 16;  // bytes
+  static __device__ __forceinline__ int off(int row, int elem) { return row * STRIDE + elem * 2; }
+};
+
+// Transposed tile [C columns][R rows-as-contraction-index] of 16-bit elements, R = 64: the element of
+// source row r (0..63) and column c lives in LDS row c.  Within each group of 16 source rows the
+// quads are stored in the order [0-3, 8-11, 4-7, 12-15] so that 16-byte chunk (2*ks + g) of LDS row c
+// holds source rows 16ks + {4g..4g+3, 8+4g..8+4g+3}: exactly what lane group g needs as the k-values
+// of an MFMA operand whose partner is a C tile converted in registers.  Chunks are XOR-swizzled by the
+// column so reads (lanes = consecutive columns) are bank-conflict free.
+struct TrTile64 {
+  static constexpr int ROW_BYTES = 128;
+  static __device__ __forceinline__ int swz(int c) { return ((c >> 1) ^ (c >> 4)) & 7; }
+  // byte offset of the 16-byte chunk for k-step ks (16 source rows) and lane group g, column c
+  static __device__ __forceinline__ int chunk_off(int c, int ks, int g) {
+    return c * ROW_BYTES + (((2 * ks + g) ^ swz(c)) << 4);
+  }
+  // byte offset at which the four values of source rows 4*rq..4*rq+3 (rq = 0..15), column c, are
+  // written as one 8-byte store
+  static __device__ __forceinline__ int quad_off(int c, int rq) {
+    return c * ROW_BYTES + (((2 * (rq >> 2) + (rq & 1)) ^ swz(c)) << 4) + (((rq >> 1) & 1) << 3);
+  }
+};
+
+// 4 x 8 block of 16-bit values held as four u32x4 rows -> column j (0..7) as 4 consecutive 16-bit
+// values (rows 0..3) packed into 8 bytes
+__device__ __forceinline__ u32x2 transpose_col(const u32x4 (&r)[4], int j) {
+  const unsigned sel = (j & 1) ? 0x07060302u : 0x05040100u;
+  const int w = j >> 1;
+  u32x2 o;
+  o.x = __builtin_amdgcn_perm(r[1][w], r[0][w], sel);
+  o.y = __builtin_amdgcn_perm(r[3][w], r[2][w], sel);
+  return o;
+}
+
+}  // namespace tp

@@ -1,0 +1,92 @@
+// Shared device/host helpers for the gfx950 kernels: element types, 16-byte vector access,
+// wavefront (64-lane) reductions, error plumbing for the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/tprime_hip.h"
+
+namespace tp {
+
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int WAVE = 64;
+
+// ---- error plumbing (host) -------------------------------------------------------------------
+void set_error(const char* fmt, ...);   // stores a message in the thread-local buffer
+int check_launch(const char* what);     // hipGetLastError -> TP_OK / TP_ERR_LAUNCH
+
+#define TP_REQUIRE(cond, code, ...)      \
+  do {                                   \
+    if (!(cond)) {                       \
+      ::tp::set_error(__VA_ARGS__);      \
+      return (code);                     \
+    }                                    \
+  } while (0)
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- element conversion ------------------------------------------------------------------------
+template <typename T> struct Elem;
+template <> struct Elem<bf16_t> {
+  static __device__ __forceinline__ float to_f(bf16_t v) { return (float)v; }
+  static __device__ __forceinline__ bf16_t from_f(float f) { return (bf16_t)f; }
+};
+template <> struct Elem<f16_t> {
+  static __device__ __forceinline__ float to_f(f16_t v) { return (float)v; }
+  static __device__ __forceinline__ f16_t from_f(float f) { return (f16_t)f; }
+};
+template <> struct Elem<float> {
+  static __device__ __forceinline__ float to_f(float v) { return v; }
+  static __device__ __forceinline__ float from_f(float f) { return f; }
+};
+// round a float through T and back (identity for float)
+template <typename T> __device__ __forceinline__ float round_to(float f) { return Elem<T>::to_f(Elem<T>::from_f(f)); }
+
+// ---- N-element vector load/store as floats -------------------------------------------------
+// N * sizeof(T) is 16 or 32 bytes and the address is 16-byte aligned.
+template <typename T, int N> struct alignas(sizeof(T) * N >= 16 ? 16 : sizeof(T) * N) Pack { T v[N]; };
+
+template <typename T, int N>
+__device__ __forceinline__ void load_f(const T* p, float (&out)[N]) {
+  Pack<T, N> r = *reinterpret_cast<const Pack<T, N>*>(p);
+#pragma unroll
+  for (int i = 0; i < N; i++) out[i] = Elem<T>::to_f(r.v[i]);
+}
+template <typename T, int N>
+__device__ __forceinline__ void store_f(T* p, const float (&in)[N]) {
+  Pack<T, N> r;
+#pragma unroll
+  for (int i = 0; i < N; i++) r.v[i] = Elem<T>::from_f(in[i]);
+  *reinterpret_cast<Pack<T, N>*>(p) = r;
+}
+
+// ---- wavefront reductions --------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+}  // namespace tp

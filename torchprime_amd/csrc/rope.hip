@@ -1,0 +1,195 @@
+// Rotary position embedding for gfx950: cos/sin table build and the rotate-half apply on q and k in
+// one launch.  HBM-bound: one pass, 16-byte loads/stores over strided (B,H,S,D) views.
+//
+// Table: LlamaRotaryEmbedding.forward (torchprime/torch_xla_models/model/llama/model.py:68-88),
+//        DeepseekV3RotaryEmbedding.forward (model/deepseek_v3/model.py:57-75).
+// Apply: rotate_half + apply_rotary_pos_emb (model/llama/model.py:91-122), the gather variant
+//        (model/mixtral/model.py:115-140), apply_rotary_pos_emb_interleave
+//        (model/deepseek_v3/model.py:84-103).
+//
+// The eager expression `(x * cos) + (rotate_half(x) * sin)` rounds each product and the sum to the
+// tensor dtype; the kernel reproduces those three roundings so bf16 results match it bit for bit.
+// The file is compiled with -ffp-contract=off so the fp32 path does not fuse mul+add either.
+#include "common.hpp"
+
+namespace tp {
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope_table_kernel(const float* __restrict__ inv_freq,
+                                                         const float* __restrict__ pos, T* __restrict__ cos_o,
+                                                         T* __restrict__ sin_o, int64_t n_rows, int half,
+                                                         float scaling) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n_rows * half) return;
+  const int64_t row = idx / half;
+  const int i = (int)(idx - row * half);
+  const float ang = inv_freq[i] * pos[row];
+  const float c = cosf(ang) * scaling, s = sinf(ang) * scaling;
+  const int64_t o = row * 2 * half + i;
+  cos_o[o] = Elem<T>::from_f(c);
+  cos_o[o + half] = Elem<T>::from_f(c);
+  sin_o[o] = Elem<T>::from_f(s);
+  sin_o[o + half] = Elem<T>::from_f(s);
+}
+
+struct RopeArgs {
+  const void* x[2];
+  void* y[2];
+  int64_t xs[2][3];  // element strides (b, h, s)
+  int64_t ys[2][3];
+  int H[2];
+  const void* cos;
+  const void* sin;
+  const int64_t* pos;
+  int64_t cs_b, cs_s, pos_b;
+  int B, S, D;
+};
+
+// One thread = one 16-byte vector of the first half and its partner in the second half
+// (E elements each), i.e. E rotation pairs.  Work item order: ((b*S + s) * Htot + h) * VH + j so a
+// wave sweeps the heads of one token, which are contiguous in (B,S,H,D) memory.
+template <typename T, bool INTERLEAVED, bool BACKWARD>
+__global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
+  constexpr int E = 16 / sizeof(T);
+  const int half = a.D / 2;
+  const int VH = half / E;  // vectors per half
+  const int Htot = a.H[0] + a.H[1];
+  const int64_t total = (int64_t)a.B * a.S * Htot * VH;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int j = (int)(idx % VH);
+  int64_t t = idx / VH;
+  int h = (int)(t % Htot);
+  t /= Htot;
+  const int s = (int)(t % a.S);
+  const int b = (int)(t / a.S);
+  const int which = h >= a.H[0] ? 1 : 0;
+  h -= which ? a.H[0] : 0;
+
+  const T* xp = (const T*)a.x[which] + b * a.xs[which][0] + h * a.xs[which][1] + s * a.xs[which][2];
+  T* yp = (T*)a.y[which] + b * a.ys[which][0] + h * a.ys[which][1] + s * a.ys[which][2];
+  int64_t crow;
+  if (a.pos) crow = a.cs_s * a.pos[b * a.pos_b + s];
+  else crow = a.cs_b * b + a.cs_s * s;
+  const T* cp = (const T*)a.cos + crow;
+  const T* sp = (const T*)a.sin + crow;
+
+  float c1[E], c2[E], s1[E], s2[E];
+  load_f<T, E>(cp + j * E, c1);
+  load_f<T, E>(cp + half + j * E, c2);
+  load_f<T, E>(sp + j * E, s1);
+  load_f<T, E>(sp + half + j * E, s2);
+
+  float x1[E], x2[E], o1[E], o2[E];
+  if (!INTERLEAVED || BACKWARD) {
+    load_f<T, E>(xp + j * E, x1);
+    load_f<T, E>(xp + half + j * E, x2);
+  } else {
+    // permuted input: first-half element i is x[2i], second-half element i is x[2i+1]
+    float lo[E], hi[E];
+    load_f<T, E>(xp + 2 * j * E, lo);
+    load_f<T, E>(xp + 2 * j * E + E, hi);
+#pragma unroll
+    for (int e = 0; e < E / 2; e++) {
+      x1[e] = lo[2 * e];
+      x2[e] = lo[2 * e + 1];
+      x1[E / 2 + e] = hi[2 * e];
+      x2[E / 2 + e] = hi[2 * e + 1];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < E; e++) {
+    if (!BACKWARD) {
+      // out[i] = x[i] cos[i] + (-x[i+h]) sin[i];  out[i+h] = x[i+h] cos[i+h] + x[i] sin[i+h]
+      o1[e] = round_to<T>(round_to<T>(x1[e] * c1[e]) + round_to<T>(-x2[e] * s1[e]));
+      o2[e] = round_to<T>(round_to<T>(x2[e] * c2[e]) + round_to<T>(x1[e] * s2[e]));
+    } else {
+      // dx[i] = g[i] cos[i] + g[i+h] sin[i+h];  dx[i+h] = g[i+h] cos[i+h] - g[i] sin[i]
+      // (autograd forms the two products and their sum in the tensor dtype as well)
+      o1[e] = round_to<T>(x1[e] * c1[e]) + round_to<T>(x2[e] * s2[e]);
+      o2[e] = round_to<T>(x2[e] * c2[e]) + round_to<T>(-x1[e] * s1[e]);
+    }
+  }
+  if (!INTERLEAVED || !BACKWARD) {
+    store_f<T, E>(yp + j * E, o1);
+    store_f<T, E>(yp + half + j * E, o2);
+  } else {
+    // inverse permutation: dx[2i] = d_first[i], dx[2i+1] = d_second[i]
+    float lo[E], hi[E];
+#pragma unroll
+    for (int e = 0; e < E / 2; e++) {
+      lo[2 * e] = o1[e];
+      lo[2 * e + 1] = o2[e];
+      hi[2 * e] = o1[E / 2 + e];
+      hi[2 * e + 1] = o2[E / 2 + e];
+    }
+    store_f<T, E>(yp + 2 * j * E, lo);
+    store_f<T, E>(yp + 2 * j * E + E, hi);
+  }
+}
+
+template <typename T>
+static int rope_typed(const RopeArgs& a, int interleaved, int backward, hipStream_t st) {
+  constexpr int E = 16 / sizeof(T);
+  const int64_t total = (int64_t)a.B * a.S * (a.H[0] + a.H[1]) * (a.D / 2 / E);
+  if (total == 0) return TP_OK;
+  const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  if (!interleaved && !backward) rope_apply_kernel<T, false, false><<<grid, block, 0, st>>>(a);
+  else if (!interleaved && backward) rope_apply_kernel<T, false, true><<<grid, block, 0, st>>>(a);
+  else if (interleaved && !backward) rope_apply_kernel<T, true, false><<<grid, block, 0, st>>>(a);
+  else rope_apply_kernel<T, true, true><<<grid, block, 0, st>>>(a);
+  return check_launch("tp_rope_apply");
+}
+
+}  // namespace tp
+
+using namespace tp;
+
+extern "C" int tp_rope_table(const float* inv_freq, const float* position_ids, void* cos, void* sin, int Bp, int S,
+                             int half, float attention_scaling, int dtype, void* stream) {
+  TP_REQUIRE(inv_freq && position_ids && cos && sin, TP_ERR_BAD_ARG, "tp_rope_table: null pointer");
+  TP_REQUIRE(Bp >= 0 && S >= 0 && half > 0, TP_ERR_BAD_ARG, "tp_rope_table: bad shape Bp=%d S=%d half=%d", Bp, S, half);
+  const int64_t rows = (int64_t)Bp * S;
+  if (rows == 0) return TP_OK;
+  const dim3 grid((unsigned)((rows * half + 255) / 256)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == TP_BF16) rope_table_kernel<bf16_t><<<grid, block, 0, st>>>(inv_freq, position_ids, (bf16_t*)cos, (bf16_t*)sin, rows, half, attention_scaling);
+  else if (dtype == TP_F16) rope_table_kernel<f16_t><<<grid, block, 0, st>>>(inv_freq, position_ids, (f16_t*)cos, (f16_t*)sin, rows, half, attention_scaling);
+  else if (dtype == TP_F32) rope_table_kernel<float><<<grid, block, 0, st>>>(inv_freq, position_ids, (float*)cos, (float*)sin, rows, half, attention_scaling);
+  else TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_rope_table: unsupported dtype %d", dtype);
+  return check_launch("tp_rope_table");
+}
+
+extern "C" int tp_rope_apply(const void* q, const void* k, const void* cos, const void* sin, const int64_t* pos,
+                             void* q_out, void* k_out, int B, int Hq, int Hkv, int S, int D, const int64_t q_strides[3],
+                             const int64_t k_strides[3], const int64_t qo_strides[3], const int64_t ko_strides[3],
+                             int64_t cs_b_stride, int64_t cs_s_stride, int64_t pos_b_stride, int interleaved,
+                             int backward, int dtype, void* stream) {
+  TP_REQUIRE(q && q_out && cos && sin && q_strides && qo_strides, TP_ERR_BAD_ARG, "tp_rope_apply: null pointer");
+  TP_REQUIRE((k == nullptr) == (Hkv == 0), TP_ERR_BAD_ARG, "tp_rope_apply: k must be NULL exactly when Hkv == 0");
+  TP_REQUIRE(Hkv == 0 || (k_out && k_strides && ko_strides), TP_ERR_BAD_ARG, "tp_rope_apply: null k output/strides");
+  TP_REQUIRE(B >= 0 && Hq > 0 && Hkv >= 0 && S >= 0 && D > 0, TP_ERR_BAD_ARG, "tp_rope_apply: bad shape");
+  const int esz = dtype == TP_F32 ? 4 : 2;
+  TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F16 || dtype == TP_F32, TP_ERR_UNSUPPORTED, "tp_rope_apply: unsupported dtype %d", dtype);
+  const int E = 16 / esz;
+  TP_REQUIRE(D % (2 * E) == 0, TP_ERR_UNSUPPORTED, "tp_rope_apply: D=%d must be a multiple of %d", D, 2 * E);
+  RopeArgs a;
+  a.x[0] = q; a.x[1] = k; a.y[0] = q_out; a.y[1] = k_out;
+  a.H[0] = Hq; a.H[1] = Hkv;
+  bool ok = aligned16(q) && aligned16(q_out) && aligned16(cos) && aligned16(sin) && aligned16(k) && aligned16(k_out);
+  for (int i = 0; i < 3; i++) {
+    a.xs[0][i] = q_strides[i]; a.ys[0][i] = qo_strides[i];
+    a.xs[1][i] = Hkv ? k_strides[i] : 0; a.ys[1][i] = Hkv ? ko_strides[i] : 0;
+    ok = ok && (a.xs[0][i] * esz) % 16 == 0 && (a.ys[0][i] * esz) % 16 == 0 && (a.xs[1][i] * esz) % 16 == 0 &&
+         (a.ys[1][i] * esz) % 16 == 0;
+  }
+  ok = ok && (cs_b_stride * esz) % 16 == 0 && (cs_s_stride * esz) % 16 == 0;
+  TP_REQUIRE(ok, TP_ERR_BAD_ARG, "tp_rope_apply: pointers and strides must keep rows 16-byte aligned");
+  a.cos = cos; a.sin = sin; a.pos = pos;
+  a.cs_b = cs_b_stride; a.cs_s = cs_s_stride; a.pos_b = pos_b_stride;
+  a.B = B; a.S = S; a.D = D;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == TP_BF16) return rope_typed<bf16_t>(a, interleaved, backward, st);
+  if (dtype == TP_F16) return rope_typed<f16_t>(a, interleaved, backward, st);
+  return rope_typed<float>(a, interleaved, backward, st);
+}
