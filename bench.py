@@ -1,0 +1,306 @@
+"""Benchmark of the attention hot path on one MI355X.
+
+One step = one forward + backward pass of causal GQA attention at the Llama-3-8B layer shape
+(BASELINE config 2: B=4, S=8192, 32 q heads / 8 kv heads, d=128, bf16) with q, k, v and dO already
+resident in HBM.  Prints ONE JSON line:
+
+  value        algorithmic TFLOP/s of the whole step, 6*B*Hq*S^2*d FLOP per step (the reference's own
+               MFU convention, torchprime/metrics/train_flops.py:208-228: causal forward 2*B*Hq*S^2*d,
+               backward twice that; recomputation is not counted)
+  roofline     the dominant kernel (dK/dV backward) against the 2.5 PFLOP/s dense bf16 MFMA peak;
+               its launch time comes from HIP events recorded on the launch stream inside the timed
+               region (tp_attn_bwd_ex), `kernels` lists the same for every kernel of the step
+  cpu_baseline the oracle's eager attention (fwd+bwd by autograd) timed on this host's cores on a
+               bounded sample of the same workload (one batch element, one kv-head group)
+  extra        RMSNorm and RoPE at the same layer shape: GB/s against the 8 TB/s HBM3E peak
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+"""
+
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+  sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_HBM_GBPS = 8000.0
+
+
+class HipEvents:
+  """hipEvent_t handles through the HIP runtime torch already loaded (timing on an explicit stream)."""
+
+  def __init__(self):
+    import torch  # noqa: F401
+
+    self.hip = None
+    for name in ("libamdhip64.so.7", "libamdhip64.so", "libamdhip64.so.6"):
+      try:
+        self.hip = ctypes.CDLL(name)
+        break
+      except OSError:
+        continue
+    if self.hip is None:
+      raise RuntimeError("HIP runtime not found")
+    self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+    self.hip.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    self.hip.hipEventSynchronize.argtypes = [ctypes.c_void_p]
+    self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+    self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+
+  def create(self, n):
+    out = []
+    for _ in range(n):
+      e = ctypes.c_void_p()
+      rc = self.hip.hipEventCreate(ctypes.byref(e))
+      if rc != 0:
+        raise RuntimeError(f"hipEventCreate failed: {rc}")
+      out.append(e)
+    return out
+
+  def record(self, e, stream):
+    rc = self.hip.hipEventRecord(e, ctypes.c_void_p(stream))
+    if rc != 0:
+      raise RuntimeError(f"hipEventRecord failed: {rc}")
+
+  def elapsed_ms(self, a, b):
+    self.hip.hipEventSynchronize(b)
+    ms = ctypes.c_float()
+    rc = self.hip.hipEventElapsedTime(ctypes.byref(ms), a, b)
+    if rc != 0:
+      raise RuntimeError(f"hipEventElapsedTime failed: {rc}")
+    return ms.value
+
+
+def make_inputs(B, Hq, Hkv, S, D, dev, seed=1235):
+  import torch
+
+  g = torch.Generator(device="cpu").manual_seed(seed)
+
+  def mk(h):
+    # (B,S,H,D) memory viewed as (B,H,S,D): what the attention modules hand over
+    return torch.randn((B, S, h, D), generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev).transpose(1, 2)
+
+  return mk(Hq), mk(Hkv), mk(Hkv), mk(Hq)
+
+
+def attention_step_fn(q, k, v, do, sm_scale, hipev=None, ev=None):
+  """Returns step(i): one fwd + bwd through the C ABI with caller-owned buffers, events optional."""
+  import torch
+
+  from torchprime_amd import _lib
+
+  lib = _lib.load()
+  B, Hq, S, D = q.shape
+  Hkv = k.shape[1]
+  dev = q.device
+  out = torch.empty((B, S, Hq, D), dtype=q.dtype, device=dev).transpose(1, 2)
+  lse = torch.empty((B, Hq, S), dtype=torch.float32, device=dev)
+  dq, dk, dv = (torch.empty_like(t.transpose(1, 2)).transpose(1, 2) for t in (q, k, v))
+  ws = torch.empty((lib.tp_attn_bwd_workspace_bytes(B, Hq, S) // 4,), dtype=torch.float32, device=dev)
+  st = _lib.stream_ptr(dev)
+  s3 = _lib.strides3
+  code = _lib.dtype_code(q.dtype)
+  EvArr = ctypes.c_void_p * 4
+
+  def step(i):
+    if ev is not None:
+      hipev.record(ev[i][0], st)
+    _lib.call("tp_attn_fwd", q.data_ptr(), k.data_ptr(), v.data_ptr(), None, out.data_ptr(), lse.data_ptr(),
+              B, Hq, Hkv, S, S, D, D, s3(q), s3(k), s3(v), s3(out), sm_scale, 1, code, st)  # fmt: skip
+    arr = EvArr(*[e.value for e in ev[i][1:5]]) if ev is not None else None
+    _lib.call("tp_attn_bwd_ex", do.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+              None, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), B, Hq, Hkv, S, S, D, D,
+              s3(do), s3(q), s3(k), s3(v), s3(out), s3(dq), s3(dk), s3(dv), sm_scale, 1, code, st, arr)  # fmt: skip
+
+  return step, (out, lse, dq, dk, dv)
+
+
+def bench_attention(args, dev):
+  import torch
+
+  B, Hq, Hkv, S, D = 4, 32, 8, 8192, 128
+  sm_scale = 1.0 / math.sqrt(D)
+  q, k, v, do = make_inputs(B, Hq, Hkv, S, D, dev)
+  hipev = HipEvents()
+  ev = [hipev.create(5) for _ in range(args.steps)]
+  warm, _ = attention_step_fn(q, k, v, do, sm_scale)
+  step, _bufs = attention_step_fn(q, k, v, do, sm_scale, hipev, ev)
+  for _ in range(args.warmup):
+    warm(0)
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for i in range(args.steps):
+    step(i)
+  torch.cuda.synchronize()
+  t1 = time.perf_counter()
+  ms_per_step = (t1 - t0) * 1e3 / args.steps
+
+  unit = B * Hq * S * S * D  # one causal matmul over the attention matrix: 2 * (S^2/2) * d per (b, h)
+  flops_step = 6.0 * unit
+  # event layout per step: [before fwd, before delta, before dkdv, before dq, after dq]
+  names = ["attn_fwd", "attn_delta", "attn_bwd_dkdv", "attn_bwd_dq"]
+  algo = {"attn_fwd": 2.0 * unit, "attn_delta": 0.0, "attn_bwd_dkdv": 3.0 * unit, "attn_bwd_dq": 1.0 * unit}
+  avg = {}
+  for j, n in enumerate(names):
+    avg[n] = sum(hipev.elapsed_ms(ev[i][j], ev[i][j + 1]) for i in range(args.steps)) / args.steps
+  kernels = {
+    n: {"ms": round(avg[n], 4), "algorithmic_TFLOPs": round(algo[n] / (avg[n] * 1e-3) / 1e12, 2) if avg[n] > 0 else None}
+    for n in names
+  }
+  dom = max(("attn_fwd", "attn_bwd_dkdv", "attn_bwd_dq"), key=lambda n: avg[n])
+  achieved = algo[dom] / (avg[dom] * 1e-3) / 1e12
+  roofline = {
+    "bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+    "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None, "launch_ms": round(avg[dom], 4),
+    "step_frac_of_peak": round(flops_step / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+  }  # fmt: skip
+  return ms_per_step, flops_step, roofline, kernels, dict(B=B, Hq=Hq, Hkv=Hkv, S=S, D=D)
+
+
+def bench_norm_rope(dev, iters=20):
+  """RMSNorm fwd/bwd on x (4,8192,4096) and RoPE on q (4,32,8192,128) + k (4,8,8192,128), bf16."""
+  import torch
+
+  import torchprime_amd as tpa
+
+  res = {}
+  g = torch.Generator(device="cpu").manual_seed(7)
+  B, S, H = 4, 8192, 4096
+  x = torch.randn((B, S, H), generator=g).to(torch.bfloat16).to(dev)
+  w = torch.ones((H,), dtype=torch.bfloat16, device=dev)
+  dy = torch.randn((B, S, H), generator=g).to(torch.bfloat16).to(dev)
+  flush = torch.empty((256 << 20,), dtype=torch.int8, device=dev)  # evict L2 / MALL between iterations
+
+  def timed(fn):
+    fn()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(iters):
+      flush.zero_()
+      a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+      a.record()
+      fn()
+      b.record()
+      torch.cuda.synchronize()
+      ts.append(a.elapsed_time(b))
+    ts.sort()
+    return ts[len(ts) // 2]
+
+  n = B * S * H
+  y, rstd = torch.ops.tprime.rmsnorm_fwd(x, w, 1e-5)
+  ms = timed(lambda: torch.ops.tprime.rmsnorm_fwd(x, w, 1e-5))
+  res["rmsnorm_fwd"] = {"ms": round(ms, 4), "GBps": round(2 * n * 2 / ms / 1e6, 1)}
+  ms = timed(lambda: torch.ops.tprime.rmsnorm_bwd(dy, x, w, rstd))
+  res["rmsnorm_bwd"] = {"ms": round(ms, 4), "GBps": round(3 * n * 2 / ms / 1e6, 1)}
+  del y, dy
+
+  Hq, Hkv, D = 32, 8, 128
+  q = torch.randn((B, S, Hq, D), generator=g).to(torch.bfloat16).to(dev).transpose(1, 2)
+  k = torch.randn((B, S, Hkv, D), generator=g).to(torch.bfloat16).to(dev).transpose(1, 2)
+  inv = tpa.default_rope_frequencies(D, 500000.0).to(dev)
+  pos = torch.arange(S, device=dev)[None].float()
+  cos, sin = tpa.ops.rope_table(inv, pos, 1.0, torch.bfloat16)
+  ms = timed(lambda: torch.ops.tprime.rope_apply(q, k, cos, sin, None, False, False))
+  nb = 2 * (q.numel() + k.numel()) * 2
+  res["rope_fwd"] = {"ms": round(ms, 4), "GBps": round(nb / ms / 1e6, 1)}
+  ms = timed(lambda: torch.ops.tprime.rope_apply(q, k, cos, sin, None, False, True))
+  res["rope_bwd"] = {"ms": round(ms, 4), "GBps": round(nb / ms / 1e6, 1)}
+  for v in res.values():
+    v["frac_of_hbm_peak"] = round(v["GBps"] / PEAK_HBM_GBPS, 4)
+  return res
+
+
+def cpu_baseline(max_seconds=24.0):
+  """The oracle's eager attention (attention.py:151-170 restated), fwd + bwd by autograd, bf16 inputs, on
+  this host's cores: one batch element and one kv-head group (4 q heads) of the benchmark workload."""
+  import torch
+
+  from oracle import tprime_oracle as orc
+
+  S, D, n_rep = 8192, 128, 4
+  g = torch.Generator(device="cpu").manual_seed(1235)
+  q = torch.randn((1, n_rep, S, D), generator=g).to(torch.bfloat16).requires_grad_(True)
+  k = torch.randn((1, 1, S, D), generator=g).to(torch.bfloat16).requires_grad_(True)
+  v = torch.randn((1, 1, S, D), generator=g).to(torch.bfloat16).requires_grad_(True)
+  do = torch.randn((1, n_rep, S, D), generator=g).to(torch.bfloat16)
+  mask = orc.causal_additive_mask(S, torch.bfloat16)
+  cores = torch.get_num_threads()
+  t0 = time.perf_counter()
+  reps = 0
+  while True:
+    out = orc.eager_attention(q, k, v, mask)
+    out.backward(do)
+    q.grad = k.grad = v.grad = None
+    reps += 1
+    if time.perf_counter() - t0 > max_seconds / 2:
+      break
+  sec = (time.perf_counter() - t0) / reps
+  flops = 6.0 * 1 * n_rep * S * S * D
+  return {
+    "value": round(flops / sec / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+    "sample": f"oracle eager attention fwd+bwd (autograd), bf16, B=1, {n_rep} q heads / 1 kv head, S={S}, d={D}: "
+              f"1/32 of one step; {reps} rep(s), {sec:.2f} s each",
+  }  # fmt: skip
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=10)
+  ap.add_argument("--warmup", type=int, default=3)
+  ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+  ap.add_argument("--no-extra", action="store_true", help="skip the RMSNorm / RoPE bandwidth leg")
+  args = ap.parse_args()
+  if args.gpus != 1:
+    sys.exit("bench.py measures the one-GPU hot path only: run with --gpus 1 (no multi-GPU path is part of this build)")
+
+  import torch
+
+  import torchprime_amd  # noqa: F401
+
+  if not torch.cuda.is_available():
+    sys.exit("bench.py needs a GPU")
+  dev = torch.device("cuda", 0)
+  ms_per_step, flops_step, roofline, kernels, shape = bench_attention(args, dev)
+  extra = None if args.no_extra else bench_norm_rope(dev)
+  torch.cuda.empty_cache()
+  cpu = None if args.no_cpu else cpu_baseline()
+  value = flops_step / (ms_per_step * 1e-3) / 1e12
+  line = {
+    "metric": "attn fwd+bwd TFLOP/s & % bf16 MFMA peak, Llama-3-8B shape S=8192",
+    "value": round(value, 2),
+    "unit": "TFLOP/s",
+    "n_gpus": 1,
+    "steps": args.steps,
+    "warmup": args.warmup,
+    "ms_per_step": round(ms_per_step, 4),
+    "higher_is_better": True,
+    "scaling": "weak",
+    "vs_baseline": None,
+    "dtype": "bf16",
+    "data": "synthetic",
+    "config": {
+      "workload": "Llama-3-8B attention layer fwd+bwd, causal GQA, inputs resident in HBM",
+      "B": shape["B"], "S": shape["S"], "q_heads": shape["Hq"], "kv_heads": shape["Hkv"], "head_dim": shape["D"],
+      "algorithmic_flop_per_step": flops_step,
+    },
+    "pct_of_bf16_mfma_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
+    "roofline": roofline,
+    "kernels": kernels,
+    "cpu_baseline": cpu,
+    "extra": extra,
+  }  # fmt: skip
+  print(json.dumps(line))
+
+
+if __name__ == "__main__":
+  main()

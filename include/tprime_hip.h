@@ -131,7 +131,7 @@ size_t tp_attn_bwd_workspace_bytes(int B, int Hq, int Sq);
  *     P = exp(sm_scale*q.k - lse);  dV = P^T dO;  dS = P o (dO V^T - rowsum(dO o O));
  *     dQ = sm_scale * dS K;  dK = sm_scale * dS^T Q   (dK, dV summed over the n_rep query heads)
  * No atomics: results are bitwise reproducible.
- *   dout, out (B,Hq,Sq,Dv) share o_strides... dout has its own do_strides
+ *   dout, out (B,Hq,Sq,Dv), each with its own stride array (do_strides, o_strides)
  *   dq/dk/dv  strided like q/k/v but with their own stride arrays
  *   ws        fp32 workspace of tp_attn_bwd_workspace_bytes(B,Hq,Sq) bytes
  * ---------------------------------------------------------------------------------------------- */
@@ -141,6 +141,18 @@ int tp_attn_bwd(const void* dout, const void* q, const void* k, const void* v, c
                 const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
                 const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
                 const int64_t dv_strides[3], float sm_scale, int causal, int dtype, void* stream);
+
+/* tp_attn_bwd with timing marks.  No counterpart in the reference; for benchmarks and profilers that
+ * want per-kernel times without an external tracer.  `events` is NULL or an array of four
+ * hipEvent_t (as void*; individual entries may be NULL) recorded on `stream` before the delta
+ * kernel, before the dK/dV kernel, before the dQ kernel and after it.  Nothing is synchronised. */
+int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                   const float* lse, const int32_t* seg, void* dq, void* dk, void* dv, float* ws, int B,
+                   int Hq, int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t do_strides[3],
+                   const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                   const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                   const int64_t dv_strides[3], float sm_scale, int causal, int dtype, void* stream,
+                   void* const* events);
 
 #ifdef __cplusplus
 }

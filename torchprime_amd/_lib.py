@@ -50,6 +50,10 @@ SIGNATURES = {
     c_int,
     [c_void_p] * 11 + [c_int] * 7 + [_I64x3] * 8 + [c_float, c_int, c_int, c_void_p],
   ),
+  "tp_attn_bwd_ex": (
+    c_int,
+    [c_void_p] * 11 + [c_int] * 7 + [_I64x3] * 8 + [c_float, c_int, c_int, c_void_p, c_void_p],
+  ),
 }
 
 _lib = None

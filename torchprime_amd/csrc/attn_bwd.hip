@@ -600,8 +600,13 @@ static int set_max_lds(K kern, const char* what) {
   return TP_OK;
 }
 
+static inline void mark(void* const* events, int i, hipStream_t st) {
+  if (events && events[i]) (void)hipEventRecord((hipEvent_t)events[i], st);
+}
+
 template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
-static int launch_bwd(const BwdArgs& a, hipStream_t st) {
+static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
+  mark(ev, 0, st);
   // delta
   {
     const int64_t threads = (int64_t)a.B * a.Hq * a.Sq * (DV / 8);
@@ -609,6 +614,7 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st) {
     int rc = check_launch("tp_attn_bwd(delta)");
     if (rc) return rc;
   }
+  mark(ev, 1, st);
   // dK, dV
   {
     constexpr int BMQ = 64, BNK = 128;
@@ -628,6 +634,7 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st) {
     int rc = check_launch("tp_attn_bwd(dkdv)");
     if (rc) return rc;
   }
+  mark(ev, 2, st);
   // dQ
   {
     constexpr int BN = 64, BM = 128;
@@ -643,18 +650,21 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st) {
       attr_set = true;
     }
     kern<<<dim3((a.Sq + BM - 1) / BM, a.Hq, a.B), dim3(256), smem, st>>>(a);
-    return check_launch("tp_attn_bwd(dq)");
+    int rc = check_launch("tp_attn_bwd(dq)");
+    if (rc) return rc;
   }
+  mark(ev, 3, st);
+  return TP_OK;
 }
 
 template <typename T, int DQK, int DV>
-static int dispatch_bwd(const BwdArgs& a, int causal, hipStream_t st) {
+static int dispatch_bwd(const BwdArgs& a, int causal, hipStream_t st, void* const* ev) {
   if (causal) {
-    if (a.seg) return launch_bwd<T, DQK, DV, true, true>(a, st);
-    return launch_bwd<T, DQK, DV, true, false>(a, st);
+    if (a.seg) return launch_bwd<T, DQK, DV, true, true>(a, st, ev);
+    return launch_bwd<T, DQK, DV, true, false>(a, st, ev);
   }
-  if (a.seg) return launch_bwd<T, DQK, DV, false, true>(a, st);
-  return launch_bwd<T, DQK, DV, false, false>(a, st);
+  if (a.seg) return launch_bwd<T, DQK, DV, false, true>(a, st, ev);
+  return launch_bwd<T, DQK, DV, false, false>(a, st, ev);
 }
 
 }  // namespace tp
@@ -666,12 +676,13 @@ extern "C" size_t tp_attn_bwd_workspace_bytes(int B, int Hq, int Sq) {
   return (size_t)B * Hq * Sq * sizeof(float);
 }
 
-extern "C" int tp_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
-                           const float* lse, const int32_t* seg, void* dq, void* dk, void* dv, float* ws, int B, int Hq,
-                           int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t do_strides[3],
-                           const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
-                           const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
-                           const int64_t dv_strides[3], float sm_scale, int causal, int dtype, void* stream) {
+extern "C" int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                              const float* lse, const int32_t* seg, void* dq, void* dk, void* dv, float* ws, int B, int Hq,
+                              int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t do_strides[3],
+                              const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                              const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                              const int64_t dv_strides[3], float sm_scale, int causal, int dtype, void* stream,
+                              void* const* events) {
   TP_REQUIRE(dout && q && k && v && out && lse && dq && dk && dv && ws, TP_ERR_BAD_ARG, "tp_attn_bwd: null pointer");
   TP_REQUIRE(do_strides && q_strides && k_strides && v_strides && o_strides && dq_strides && dk_strides && dv_strides,
              TP_ERR_BAD_ARG, "tp_attn_bwd: null stride array");
@@ -697,7 +708,7 @@ extern "C" int tp_attn_bwd(const void* dout, const void* q, const void* k, const
   a.scale_log2 = sm_scale * LOG2E;
   a.sm_scale = sm_scale;
   hipStream_t st = (hipStream_t)stream;
-#define TP_BWD(T, DQ, DVV) return dispatch_bwd<T, DQ, DVV>(a, causal, st)
+#define TP_BWD(T, DQ, DVV) return dispatch_bwd<T, DQ, DVV>(a, causal, st, events)
   if (dtype == TP_BF16) {
     if (Dqk == 128 && Dv == 128) TP_BWD(bf16_t, 128, 128);
     if (Dqk == 64 && Dv == 64) TP_BWD(bf16_t, 64, 64);
@@ -709,4 +720,15 @@ extern "C" int tp_attn_bwd(const void* dout, const void* q, const void* k, const
   }
 #undef TP_BWD
   TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_attn_bwd: head dims (qk=%d, v=%d) not built", Dqk, Dv);
+}
+
+extern "C" int tp_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                           const float* lse, const int32_t* seg, void* dq, void* dk, void* dv, float* ws, int B, int Hq,
+                           int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t do_strides[3],
+                           const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                           const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                           const int64_t dv_strides[3], float sm_scale, int causal, int dtype, void* stream) {
+  return tp_attn_bwd_ex(dout, q, k, v, out, lse, seg, dq, dk, dv, ws, B, Hq, Hkv, Sq, Skv, Dqk, Dv, do_strides, q_strides,
+                        k_strides, v_strides, o_strides, dq_strides, dk_strides, dv_strides, sm_scale, causal, dtype, stream,
+                        nullptr);
 }
