@@ -121,6 +121,7 @@ rmsnorm_fwd.register_autograd(_rmsnorm_backward, setup_context=_rmsnorm_setup)
 
 def rmsnorm(x: Tensor, weight: Tensor, eps: float) -> Tensor:
   """``weight * (x.float() * rsqrt(mean(x.float()**2, -1) + eps)).to(x.dtype)`` in one pass."""
+  _lib.require_gpu(x, weight)
   return rmsnorm_fwd(x, weight, eps)[0]
 
 
@@ -237,6 +238,7 @@ rope_apply_op.register_autograd(_rope_backward, setup_context=_rope_setup)
 
 def rope_apply(q: Tensor, k: Tensor, cos: Tensor, sin: Tensor, pos: Tensor | None = None, interleaved: bool = False):
   """``(q*cos + rotate_half(q)*sin, k*cos + rotate_half(k)*sin)`` for (B,H,S,D) q and k in one launch."""
+  _lib.require_gpu(q, k, cos, sin, pos)
   return rope_apply_op(q, k, cos, sin, pos, interleaved, False)
 
 
@@ -356,6 +358,7 @@ def attention(
 
   ``sm_scale=None`` means ``1/sqrt(v.shape[-1])``, the scale AttentionModule uses
   (torchprime/torch_xla_models/attention.py:54-58, 107, 143, 154)."""
+  _lib.require_gpu(q, k, v, segment_ids)
   if sm_scale is None:
     sm_scale = 1.0 / math.sqrt(v.shape[-1])
   return attn_fwd(q, k, v, segment_ids, sm_scale, causal)[0]

@@ -17,7 +17,7 @@ from __future__ import annotations
 import torch
 from torch import nn
 
-from . import ops
+from . import _lib, ops
 from .rope import RopeScaling, deepseek_v3_rope_init_fn, llama3_rope_frequencies
 
 
@@ -32,6 +32,7 @@ class LlamaRotaryEmbedding(nn.Module):
   @torch.no_grad()
   def forward(self, x, position_ids):
     # x: [bs, num_attention_heads, seq_len, head_size]; position_ids: (bs or 1, seq_len), float in the models
+    _lib.require_gpu(x, position_ids)
     return ops.rope_table(self.inv_freq, position_ids, 1.0, x.dtype)
 
 
@@ -47,6 +48,7 @@ class DeepseekV3RotaryEmbedding(nn.Module):
 
   @torch.no_grad()
   def forward(self, x: torch.Tensor, position_ids: torch.Tensor):
+    _lib.require_gpu(x, position_ids)
     return ops.rope_table(self.inv_freq, position_ids, float(self.attention_scaling), x.dtype)
 
 
@@ -74,6 +76,7 @@ class MixtralRotaryEmbedding(nn.Module):
 
   def forward(self, x, seq_len=None):
     # x: [bs, num_attention_heads, seq_len, head_size]
+    _lib.require_gpu(x)
     if self.max_seq_len_cached == 0 or self.cos_cached.device != x.device:
       # the reference fills the cache in __init__ on the construction device; the table kernel is
       # GPU-only, so the first call on the GPU fills it (same values, same dtype)
