@@ -96,7 +96,7 @@ def test_segment_equals_block_diagonal_decomposition():
   for L in lengths[0]:
     sl = slice(pos, pos + L)
     part = tpa.ops.attention(q[:, :, sl].to(DEV), k[:, :, sl].to(DEV), v[:, :, sl].to(DEV), None, None, True)
-    assert_close(full[:, :, sl], part.float().cpu(), f"doc@{pos}", max_abs=8e-3, rel_l2=4e-3)
+    assert_close(full[:, :, sl], part.float().cpu(), f"doc@{pos}")  # two bf16 results: within one output ulp
     pos += L
 
 

@@ -261,6 +261,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     load_tile(0);
     store_tile(0);
   }
+  // all earlier loads (the K/V fragments) have landed: keeps per-iteration MFMAs from waiting on the
+  // in-order vector-memory counter for that iteration's own prefetch
+  __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 
   for (int it = 0; it < n_iter; it++) {
@@ -312,24 +315,31 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       v8 pfr[BMQ / 16], dsf[BMQ / 16];
       const int kvcol = wkv0 + ln;
 #pragma unroll
+      for (int qb = 0; qb < QB; qb++)
+#pragma unroll
+        for (int vq = 0; vq < 4; vq++) {
+          const f32x4 l4 = *(const f32x4*)(lsel + qb * 32 + 8 * vq + 4 * g);
+#pragma unroll
+          for (int e = 0; e < 4; e++) sacc[qb][4 * vq + e] = fast_exp2(__builtin_fmaf(sacc[qb][4 * vq + e], c, -l4[e]));
+        }
+      if (need_mask) {  // separate pass: the common unmasked tile carries no per-element branches
+#pragma unroll
+        for (int qb = 0; qb < QB; qb++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) {
+            const int r = qb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
+            const int qrow = qi0 + r;
+            const bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || segl[r] == segk);
+            sacc[qb][v] = ok ? sacc[qb][v] : 0.f;
+          }
+      }
+#pragma unroll
       for (int qb = 0; qb < QB; qb++) {
 #pragma unroll
         for (int vq = 0; vq < 4; vq++) {
-          const int r0 = qb * 32 + 8 * vq + 4 * g;
-          const f32x4 l4 = *(const f32x4*)(lsel + r0);
-          const f32x4 d4 = *(const f32x4*)(deltal + r0);
+          const f32x4 d4 = *(const f32x4*)(deltal + qb * 32 + 8 * vq + 4 * g);
 #pragma unroll
-          for (int e = 0; e < 4; e++) {
-            const int v = 4 * vq + e;
-            float p = fast_exp2(__builtin_fmaf(sacc[qb][v], c, -l4[e]));
-            if (need_mask) {
-              const int qrow = qi0 + r0 + e;
-              const bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || segl[r0 + e] == segk);
-              p = ok ? p : 0.f;
-            }
-            sacc[qb][v] = p;
-            dpacc[qb][v] = p * (dpacc[qb][v] - d4[e]);
-          }
+          for (int e = 0; e < 4; e++) dpacc[qb][4 * vq + e] = sacc[qb][4 * vq + e] * (dpacc[qb][4 * vq + e] - d4[e]);
         }
 #pragma unroll
         for (int hh = 0; hh < 2; hh++) {
@@ -501,6 +511,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
     load_tile(SEG ? active[0] : 0);
     store_tile(0);
   }
+  __builtin_amdgcn_s_waitcnt(0);  // Q / dO fragments, LSE and delta have landed (see the dK/dV kernel)
   __syncthreads();
 
   for (int it = 0; it < nact; it++) {
@@ -544,18 +555,24 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
         }
       v8 dsf[BN / 16];
 #pragma unroll
-      for (int nb = 0; nb < NB; nb++) {
+      for (int nb = 0; nb < NB; nb++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-          float p = fast_exp2(__builtin_fmaf(sacc[nb][v], c, -lse_s));
-          if (need_mask) {
+        for (int v = 0; v < 16; v++) sacc[nb][v] = fast_exp2(__builtin_fmaf(sacc[nb][v], c, -lse_s));
+      if (need_mask) {  // separate pass: the common unmasked tile carries no per-element branches
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) {
             const int kvl = nb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
             const int kv = kv0 + kvl;
             const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
-            p = ok ? p : 0.f;
+            sacc[nb][v] = ok ? sacc[nb][v] : 0.f;
           }
-          dpacc[nb][v] = p * (dpacc[nb][v] - delta_s);
-        }
+      }
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) dpacc[nb][v] = sacc[nb][v] * (dpacc[nb][v] - delta_s);
 #pragma unroll
         for (int hh = 0; hh < 2; hh++) {
           const f32x16& d = dpacc[nb];

@@ -187,6 +187,11 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
     load_tile(SEG ? active[0] : 0);
     store_tile(0);
   }
+  // Everything loaded so far (the Q fragments above all) has landed before the loop starts.  Without
+  // this the compiler must assume those loads may still be in flight at the loop head and, the vector
+  // memory counter being in-order, makes the first MFMA of EVERY iteration wait for that iteration's
+  // own prefetch loads.
+  __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 
   for (int it = 0; it < nact; it++) {
@@ -252,9 +257,14 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
 #pragma unroll
           for (int v = 0; v < 16; v++) mx = fmaxf(mx, sacc[nb][mr][v]);
         mx = half_max(mx);
-        const float m_new = fmaxf(m_run[mr], mx * c);
+        // Lazy rescale: the running max only moves when the tile max exceeds it by more than 2^8, so
+        // p stays <= 256 (harmless in fp32 sums and in the 16-bit P operand) and on most tiles no lane of
+        // the wave needs its accumulators rescaled.  O and l always share the same reference max.
+        const float mxs = mx * c;
+        const bool grow = mxs > m_run[mr] + 8.0f;
+        const float m_new = grow ? mxs : m_run[mr];
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = fast_exp2(m_run[mr] - m_use);
+        const float alpha = grow ? fast_exp2(m_run[mr] - m_use) : 1.0f;
         m_run[mr] = m_new;
         float rs = 0.f;
 #pragma unroll
@@ -266,10 +276,12 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
             rs += p;
           }
         l_run[mr] = l_run[mr] * alpha + rs;
+        if (__builtin_amdgcn_ballot_w64(grow) != 0) {
 #pragma unroll
-        for (int d = 0; d < DVB; d++)
+          for (int d = 0; d < DVB; d++)
 #pragma unroll
-          for (int v = 0; v < 16; v++) oacc[d][mr][v] *= alpha;
+            for (int v = 0; v < 16; v++) oacc[d][mr][v] *= alpha;
+        }
 #pragma unroll
         for (int nb = 0; nb < NB; nb++)
 #pragma unroll
