@@ -77,19 +77,24 @@ struct Stage64 {
   static constexpr int TOT = (D / 8) * 16;       // 4x8 blocks in the tile
   static constexpr int ITEMS = (TOT + 255) / 256;
   u32x4 r[ITEMS][4];
+  unsigned vo[ITEMS][4];  // byte offsets of this thread's 16-byte pieces inside a tile
 
-  template <typename T>
-  __device__ __forceinline__ void load(const T* base, int64_t row_stride, int row0, int row_max, int tid) {
+  __device__ __forceinline__ void init(int64_t row_stride, int tid) {
 #pragma unroll
     for (int i = 0; i < ITEMS; i++) {
       const int item = tid + 256 * i;
-      if (item < TOT) {
-        const int c8 = item % (D / 8), rq = item / (D / 8);
+      const int c8 = item % (D / 8), rq = item / (D / 8);
 #pragma unroll
-        for (int ii = 0; ii < 4; ii++) {
-          const int row = min(row0 + 4 * rq + ii, row_max);
-          r[i][ii] = *(const u32x4*)(base + row * row_stride + c8 * 8);
-        }
+      for (int ii = 0; ii < 4; ii++) vo[i][ii] = (unsigned)(((4 * rq + ii) * row_stride + c8 * 8) * 2);
+    }
+  }
+  // rows past the end of the tensor (offset >= the resource's size) read as zero
+  __device__ __forceinline__ void load(rsrc_t rs, unsigned tile_byte_offset, int tid) {
+#pragma unroll
+    for (int i = 0; i < ITEMS; i++) {
+      if (tid + 256 * i < TOT) {
+#pragma unroll
+        for (int ii = 0; ii < 4; ii++) r[i][ii] = buf_load16(rs, vo[i][ii], tile_byte_offset);
       }
     }
   }
@@ -208,21 +213,27 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   }
   const int n_iter = nact * a.n_rep;
 
-  // ---- staging
+  // ---- staging: Q / dO tiles by buffer loads (offsets inside a tile precomputed, tile offset scalar)
   Stage64<DQK> qst;
   Stage64<DV> dost;
+  qst.init(a.qs[2], tid);
+  dost.init(a.dos[2], tid);
+  const unsigned q_span = span_bytes(Sq, a.qs[2], DQK), do_span = span_bytes(Sq, a.dos[2], DV);
+  const unsigned q_tile_bytes = (unsigned)(BMQ * a.qs[2] * 2), do_tile_bytes = (unsigned)(BMQ * a.dos[2] * 2);
   float lse_r = 0.f, delta_r = 0.f;
   int segq_r = 0;
-  auto tile_of = [&](int it, int& hq, int& qi0) {
-    const int hl = it / nact, idx = it - hl * nact;
-    hq = hk * a.n_rep + hl;
-    qi0 = (qt_first + (SEG ? active[idx] : idx)) * BMQ;
-  };
-  auto load_tile = [&](int it) {
-    int hq, qi0;
-    tile_of(it, hq, qi0);
-    qst.load((const T*)a.q + b * a.qs[0] + hq * a.qs[1], a.qs[2], qi0, Sq - 1, tid);
-    dost.load((const T*)a.dout + b * a.dos[0] + hq * a.dos[1], a.dos[2], qi0, Sq - 1, tid);
+  // iteration -> (query head of the group, query tile): heads outer, tiles inner, no division in the loop
+  int cur_hl = 0, cur_idx = 0;  // position of the tile being computed
+  int nxt_hl = 0, nxt_idx = 0;  // position of the tile being prefetched
+  auto qtile_of = [&](int idx) { return qt_first + (SEG ? active[idx] : idx); };
+  auto load_tile = [&](int hl, int idx) {
+    const int hq = hk * a.n_rep + hl;
+    const int qt = qtile_of(idx);
+    const int qi0 = qt * BMQ;
+    const rsrc_t qrs = make_rsrc((const T*)a.q + b * a.qs[0] + hq * a.qs[1], q_span);
+    const rsrc_t dors = make_rsrc((const T*)a.dout + b * a.dos[0] + hq * a.dos[1], do_span);
+    qst.load(qrs, (unsigned)qt * q_tile_bytes, tid);
+    dost.load(dors, (unsigned)qt * do_tile_bytes, tid);
     if (tid < BMQ) {
       const int row = min(qi0 + tid, Sq - 1);
       const int64_t ro = ((int64_t)b * a.Hq + hq) * Sq + row;
@@ -258,7 +269,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   const float c = a.scale_log2;
 
   if (n_iter > 0) {
-    load_tile(0);
+    load_tile(0, 0);
     store_tile(0);
   }
   // all earlier loads (the K/V fragments) have landed: keeps per-iteration MFMAs from waiting on the
@@ -268,9 +279,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
 
   for (int it = 0; it < n_iter; it++) {
     const int buf = NBUF == 2 ? (it & 1) : 0;
-    int hq, qi0;
-    tile_of(it, hq, qi0);
-    if (it + 1 < n_iter) load_tile(it + 1);
+    const int qi0 = qtile_of(cur_idx) * BMQ;
+    nxt_idx = cur_idx + 1;
+    nxt_hl = cur_hl;
+    if (nxt_idx == nact) { nxt_idx = 0; nxt_hl++; }
+    if (it + 1 < n_iter) load_tile(nxt_hl, nxt_idx);
 
     const unsigned char* ql = smem + buf * BUF_BYTES;
     const unsigned char* dol = ql + Q_BYTES;
@@ -284,8 +297,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     bool skip = (CAUSAL && qi0 + BMQ - 1 < wkv0) || wkv0 >= Skv;
     bool need_mask = (qi0 + BMQ > Sq) || (wkv0 + 32 > Skv) || (CAUSAL && qi0 < wkv0 + 31);
     if (SEG) {
-      const int idx = it % nact;
-      const int lo = qmin[active[idx]], hi = qmax[active[idx]];
+      const int lo = qmin[active[cur_idx]], hi = qmax[active[cur_idx]];
       skip = skip || hi < wkmin || lo > wkmax;
       need_mask = need_mask || !(lo == hi && wkmin == wkmax && lo == wkmin);
     }
@@ -369,6 +381,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     if (NBUF == 1) __syncthreads();
     if (it + 1 < n_iter) store_tile(NBUF == 2 ? (buf ^ 1) : 0);
     __syncthreads();
+    cur_idx = nxt_idx;
+    cur_hl = nxt_hl;
   }
 
   // ---- epilogue: lane = kv row, 4 consecutive head-dim values per store
@@ -473,18 +487,23 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
   }
 
   Stage64<DQK> kst;
+  kst.init(a.ks[2], tid);
+  const rsrc_t krs = make_rsrc(kb, span_bytes(Skv, a.ks[2], DQK));
+  const rsrc_t vrs = make_rsrc(vb, span_bytes(Skv, a.vs[2], DV));
+  const unsigned k_tile_bytes = (unsigned)(BN * a.ks[2] * 2), v_tile_bytes = (unsigned)(BN * a.vs[2] * 2);
   u32x4 vreg[V_ITEMS];
+  unsigned vvo[V_ITEMS];
+#pragma unroll
+  for (int i = 0; i < V_ITEMS; i++) {
+    const int item = tid + 256 * i;
+    vvo[i] = (unsigned)(((item / VCH) * a.vs[2] + (item % VCH) * 8) * 2);
+  }
   int sreg = 0;
   auto load_tile = [&](int t) {
-    const int kv0 = t * BN;
-    kst.load(kb, a.ks[2], kv0, Skv - 1, tid);
+    kst.load(krs, (unsigned)t * k_tile_bytes, tid);
 #pragma unroll
-    for (int i = 0; i < V_ITEMS; i++) {
-      const int item = tid + 256 * i;
-      const int row = min(kv0 + item / VCH, Skv - 1), ch = item % VCH;
-      vreg[i] = *(const u32x4*)(vb + row * a.vs[2] + ch * 8);
-    }
-    if (SEG && tid < BN) sreg = segb[min(kv0 + tid, Skv - 1)];
+    for (int i = 0; i < V_ITEMS; i++) vreg[i] = buf_load16(vrs, vvo[i], (unsigned)t * v_tile_bytes);
+    if (SEG && tid < BN) sreg = segb[min(t * BN + tid, Skv - 1)];
   };
   auto store_tile = [&](int buf) {
     unsigned char* base = smem + buf * BUF_BYTES;
@@ -722,6 +741,14 @@ extern "C" int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, co
          do_strides[i] % 8 == 0 && dq_strides[i] % 4 == 0 && dk_strides[i] % 4 == 0 && dv_strides[i] % 4 == 0;
   }
   TP_REQUIRE(ok, TP_ERR_BAD_ARG, "tp_attn_bwd: pointers and strides must keep rows 16-byte aligned");
+  {
+    // tiles are addressed with 32-bit byte offsets inside one (batch, head) slice
+    const int64_t lim = 1ll << 31;
+    const bool fits = ((int64_t)Sq * q_strides[2] + Dqk) * 2 < lim && ((int64_t)Sq * do_strides[2] + Dv) * 2 < lim &&
+                      ((int64_t)Skv * k_strides[2] + Dqk) * 2 < lim && ((int64_t)Skv * v_strides[2] + Dv) * 2 < lim &&
+                      q_strides[2] > 0 && do_strides[2] > 0 && k_strides[2] > 0 && v_strides[2] > 0;
+    TP_REQUIRE(fits, TP_ERR_UNSUPPORTED, "tp_attn_bwd: one (batch, head) slice of q, dO, k or v spans 2 GiB or more");
+  }
   a.scale_log2 = sm_scale * LOG2E;
   a.sm_scale = sm_scale;
   hipStream_t st = (hipStream_t)stream;

@@ -77,6 +77,22 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
 
+// ---- buffer loads ---------------------------------------------------------------------------------
+// K/V/Q/dO tiles are fetched with raw buffer loads: the per-thread byte offset inside a tile is computed
+// once, the tile's offset is a scalar, so the per-tile address arithmetic is free, and rows past the end
+// of the tensor (offset >= num_records) read as zero instead of needing a clamp per row.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ u32x4 buf_load16(rsrc_t r, unsigned voffset, unsigned soffset) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, (int)voffset, (int)soffset, 0);
+}
+// bytes spanned by `rows` rows of `row_elems` 16-bit elements at a row stride of `stride` elements
+__device__ __forceinline__ unsigned span_bytes(int rows, int64_t stride, int row_elems) {
+  return (unsigned)(((int64_t)(rows - 1) * stride + row_elems) * 2);
+}
+
 // ---- LDS layouts ---------------------------------------------------------------------------------
 // Row-major tile [rows][D] of 16-bit elements: rows padded by 16 bytes so that 16-byte reads by lanes
 // in consecutive rows land in different banks.

@@ -122,31 +122,38 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
     __syncthreads();
   }
 
-  // ---- global -> register staging of one K/V tile, register -> LDS
+  // ---- global -> register staging of one K/V tile (buffer loads, rows past Skv read as zero)
+  const rsrc_t krs = make_rsrc(kb, span_bytes(Skv, a.ks[2], DQK));
+  const rsrc_t vrs = make_rsrc(vb, span_bytes(Skv, a.vs[2], DV));
+  const unsigned k_tile_bytes = (unsigned)(BN * a.ks[2] * 2), v_tile_bytes = (unsigned)(BN * a.vs[2] * 2);
+  unsigned kvo[K_ITEMS], vvo[V_ITEMS][4];
+#pragma unroll
+  for (int i = 0; i < K_ITEMS; i++) {
+    const int item = tid + 256 * i;
+    kvo[i] = (unsigned)(((item / KCH) * a.ks[2] + (item % KCH) * 8) * 2);
+  }
+#pragma unroll
+  for (int i = 0; i < V_ITEMS; i++) {
+    const int item = tid + 256 * i;
+    const int c8 = item % (DV / 8), rq = item / (DV / 8);
+#pragma unroll
+    for (int ii = 0; ii < 4; ii++) vvo[i][ii] = (unsigned)(((4 * rq + ii) * a.vs[2] + c8 * 8) * 2);
+  }
   u32x4 kreg[K_ITEMS];
   u32x4 vreg[V_ITEMS][4];
   int sreg = 0;
   auto load_tile = [&](int t) {
-    const int kv0 = t * BN;
+    const unsigned kso = (unsigned)t * k_tile_bytes, vso = (unsigned)t * v_tile_bytes;
 #pragma unroll
-    for (int i = 0; i < K_ITEMS; i++) {
-      const int item = tid + 256 * i;
-      const int row = min(kv0 + item / KCH, Skv - 1), ch = item % KCH;
-      kreg[i] = *(const u32x4*)(kb + row * a.ks[2] + ch * 8);
-    }
+    for (int i = 0; i < K_ITEMS; i++) kreg[i] = buf_load16(krs, kvo[i], kso);
 #pragma unroll
     for (int i = 0; i < V_ITEMS; i++) {
-      const int item = tid + 256 * i;
-      if (item < V_TOT) {
-        const int c8 = item % (DV / 8), rq = item / (DV / 8);
+      if (tid + 256 * i < V_TOT) {
 #pragma unroll
-        for (int ii = 0; ii < 4; ii++) {
-          const int row = min(kv0 + 4 * rq + ii, Skv - 1);
-          vreg[i][ii] = *(const u32x4*)(vb + row * a.vs[2] + c8 * 8);
-        }
+        for (int ii = 0; ii < 4; ii++) vreg[i][ii] = buf_load16(vrs, vvo[i][ii], vso);
       }
     }
-    if (SEG && tid < BN) sreg = segb[min(kv0 + tid, Skv - 1)];
+    if (SEG && tid < BN) sreg = segb[min(t * BN + tid, Skv - 1)];
   };
   auto store_tile = [&](int buf) {
     unsigned char* kl = smem + buf * BUF_BYTES;
@@ -387,6 +394,10 @@ extern "C" int tp_attn_fwd(const void* q, const void* k, const void* v, const in
     ok = ok && q_strides[i] % 8 == 0 && k_strides[i] % 8 == 0 && v_strides[i] % 8 == 0 && o_strides[i] % 4 == 0;
   }
   TP_REQUIRE(ok, TP_ERR_BAD_ARG, "tp_attn_fwd: pointers and strides must keep rows 16-byte aligned");
+  // tiles are addressed with 32-bit byte offsets inside one (batch, head) slice
+  TP_REQUIRE(((int64_t)Skv * k_strides[2] + Dqk) * 2 < (1ll << 31) && ((int64_t)Skv * v_strides[2] + Dv) * 2 < (1ll << 31) &&
+                 k_strides[2] > 0 && v_strides[2] > 0,
+             TP_ERR_UNSUPPORTED, "tp_attn_fwd: one (batch, head) slice of k or v spans 2 GiB or more");
   a.scale_log2 = sm_scale * LOG2E;
   hipStream_t st = (hipStream_t)stream;
 #define TP_FWD(T, DQ, DVV) return dispatch_fwd<T, DQ, DVV>(a, B, causal, st)
