@@ -36,7 +36,7 @@ def _check(B, Hq, Hkv, S, Dqk, Dv, dtype, causal, seg=None, layout="bshd", seed=
   _, lse_ref = orc.attention_ref(q, k, v, seg, causal, sm_scale, torch.float64)
   assert out.shape == (B, Hq, S, Dv) and out.dtype == dtype
   assert_close(out, o_ref, "out")
-  assert_close(lse, lse_ref, "lse", max_abs=2e-3, rel_l2=1e-3)
+  assert_close(lse, lse_ref, "lse", max_abs=5e-3, rel_l2=1e-3)  # row sums add the 16-bit-rounded p the PV product uses
   # gradients reach |x| > 4 with N(0,1) inputs, where one bf16 rounding alone is up to 1.6e-2:
   # the max-abs bound is taken relative to the tensor's scale there (tests/util.py)
   assert_close(dq, dq_ref, "dq", scale_abs=True)
@@ -66,6 +66,14 @@ def test_causal_fwd_bwd(dtype, B, Hq, Hkv, S, Dqk, Dv):
 def test_full_attention_fwd_bwd(B, Hq, Hkv, S, Skv, Dqk, Dv):
   # the eager branch without a mask (attention.py:151-170 with attention_mask=None)
   _check(B, Hq, Hkv, S, Dqk, Dv, torch.bfloat16, False, Skv=Skv)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_running_max_moves_often(seed):
+  # large score spread: the row maximum keeps growing by more than the lazy-rescale threshold, in either
+  # half of a KV tile, so the rescale paths (including the one deferred past the first half's P V) run
+  _check(1, 4, 2, 512, 128, 128, torch.bfloat16, True, seed=10 * seed, std=2.5)
+  _check(1, 2, 2, 300, 64, 64, torch.bfloat16, False, seed=10 * seed + 5, std=3.0)
 
 
 def test_contiguous_bhsd_layout_and_scale():
@@ -231,7 +239,7 @@ def _slice_check(B, Hq, Hkv, S, Dqk, Dv, seg, seed, b_sel, g_sel, sm_scale=None)
   assert_close(dk[b_sel : b_sel + 1, g_sel : g_sel + 1], dk_ref, "dk", scale_abs=True)
   assert_close(dv[b_sel : b_sel + 1, g_sel : g_sel + 1], dv_ref, "dv", scale_abs=True)
   # every row is a convex combination of V rows: bounded by max |v|
-  assert out.abs().max().item() <= v.abs().max().item() + 1e-2
+  assert out.abs().max().item() <= v.abs().max().item() * (1 + 2.0**-7) + 1e-2  # P is rounded to bf16 for PV
   assert torch.isfinite(lse).all() and torch.isfinite(dq.float()).all()
 
 

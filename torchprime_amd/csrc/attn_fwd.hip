@@ -3,7 +3,7 @@
 // Replaces AttentionModule.forward's three branches (torchprime/torch_xla_models/attention.py:70-170)
 // and the segment-id path of torchprime/utils/kernel_utils.py:215-220, 259-263.
 //
-// Structure (one workgroup = 4 waves = 128*MR query rows of one (batch, head); KV tiles of 64):
+// Structure (one workgroup = 4 waves = 128 query rows of one (batch, head); KV tiles of 64):
 //   * the scores are computed TRANSPOSED, S^T = K Q^T, so that in the MFMA result layout a lane owns
 //     one query column and 16 key rows per 32x32 block: row max / sum / rescale are per-lane scalars
 //     (one half-wave exchange per tile), and exp(S^T) converted to 16 bit is already the B operand of
@@ -15,6 +15,8 @@
 //   * causal: the KV loop ends at the diagonal, element masks only on tiles that straddle it;
 //     segments: per-tile [min,max] of the ids is computed once per workgroup, tiles whose id range
 //     misses the query rows' range are skipped, element compares only where ranges are not one id.
+#include <type_traits>
+
 #include "attn_common.hpp"
 
 namespace tp {
@@ -31,12 +33,11 @@ struct FwdArgs {
   float scale_log2;  // sm_scale * log2(e)
 };
 
-template <typename T, int DQK, int DV, int MR, bool CAUSAL, bool SEG>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
+template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
+__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
   typedef typename MT<T>::v8 v8;
-  constexpr int BN = 64;              // kv rows per tile
-  constexpr int BM = 128 * MR;        // q rows per workgroup
-  constexpr int NB = BN / 32;         // 32-row kv blocks per tile
+  constexpr int BN = 64;              // kv rows per LDS tile, processed as two halves of 32
+  constexpr int BM = 128;             // q rows per workgroup, 32 per wave
   constexpr int KSTEPS = DQK / 16;    // MFMA k-steps over the qk head dim
   constexpr int DVB = DV / 32;        // 32-column blocks of the v head dim
   typedef RowTile<DQK> KT;
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
   const int qt = gridDim.x - 1 - blockIdx.x;  // longest (latest) query tiles are scheduled first
   const int h = blockIdx.y, b = blockIdx.z, hk = h / a.n_rep;
   const int q0 = qt * BM;
-  const int wq0 = q0 + wave * 32 * MR;
+  const int wq0 = q0 + wave * 32;
   const int Sq = a.Sq, Skv = a.Skv;
 
   const T* qb = (const T*)a.q + b * a.qs[0] + h * a.qs[1];
@@ -68,16 +69,14 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
   const int ntiles = (kv_end + BN - 1) / BN;
 
   // ---- Q fragments (B operand of S^T = K Q^T): lane = query column, 8 head-dim values per k-step
-  v8 qf[MR][KSTEPS];
-  int segq[MR];
+  v8 qf[KSTEPS];
+  const int qrow = wq0 + ln;
+  {
+    const T* qp = qb + min(qrow, Sq - 1) * a.qs[2] + 8 * g;
 #pragma unroll
-  for (int mr = 0; mr < MR; mr++) {
-    const int row = min(wq0 + mr * 32 + ln, Sq - 1);
-    const T* qp = qb + row * a.qs[2] + 8 * g;
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) qf[mr][ks] = *(const v8*)(qp + 16 * ks);
-    segq[mr] = SEG ? segb[row] : 0;
+    for (int ks = 0; ks < KSTEPS; ks++) qf[ks] = *(const v8*)(qp + 16 * ks);
   }
+  const int segq = SEG ? segb[min(qrow, Sq - 1)] : 0;
 
   // ---- segment bookkeeping: per-tile id ranges, list of tiles that can contain an allowed pair
   int* kvmin = (int*)(smem + 2 * BUF_BYTES);
@@ -87,14 +86,14 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
   int nact = ntiles;
   int wqmin = 0, wqmax = 0;
   if (SEG) {
-    wqmin = segq[0]; wqmax = segq[0];
-#pragma unroll
-    for (int mr = 1; mr < MR; mr++) { wqmin = min(wqmin, segq[mr]); wqmax = max(wqmax, segq[mr]); }
+    wqmin = segq; wqmax = segq;
 #pragma unroll
     for (int o = 16; o > 0; o >>= 1) {
       wqmin = min(wqmin, __shfl_xor(wqmin, o, 64));
       wqmax = max(wqmax, __shfl_xor(wqmax, o, 64));
     }
+    wqmin = __builtin_amdgcn_readfirstlane(wqmin);
+    wqmax = __builtin_amdgcn_readfirstlane(wqmax);
     if (lane == 0) { bq[2 * wave] = wqmin; bq[2 * wave + 1] = wqmax; }
     for (int t = wave; t < ntiles; t += 4) {
       const int idx = min(t * BN + lane, Skv - 1);
@@ -175,20 +174,127 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
     if (SEG && tid < BN) ((int*)(vl + V_BYTES))[tid] = sreg;
   };
 
-  // ---- accumulators: O^T blocks [DVB][MR], running max (log2 units) and per-lane partial row sums
-  f32x16 oacc[DVB][MR];
-  float m_run[MR], l_run[MR];
+  // ---- accumulators: O^T blocks, running max (log2 units), per-lane partial row sum
+  f32x16 oacc[DVB];
 #pragma unroll
-  for (int mr = 0; mr < MR; mr++) {
-    m_run[mr] = -INFINITY;
-    l_run[mr] = 0.f;
+  for (int d = 0; d < DVB; d++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) oacc[d][v] = 0.f;
+  float m_run = -INFINITY;  // reference max of the row (stale by at most 8: lazy rescale)
+  float m_use = 0.f;        // m_run, or 0 while the row has seen no allowed key
+  float l_run = 0.f;
+  const float c = a.scale_log2;
+
+  // Online softmax of one 32-row half of S^T held in `s` (lane = query column, 16 key rows):
+  // updates the row state and returns exp2(s*c - m) in place.  The running max only moves when the
+  // half's max exceeds it by more than 2^8, so p stays <= 256 (harmless in fp32 sums and in the 16-bit
+  // P operand) and the rescale of O, a wave-uniform branch, is off the common path.
+  // Returns true (wave-uniform) when some lane moved its reference max; `alpha` is then the factor its
+  // O accumulators must be multiplied by (1 for lanes that kept theirs).  m_run, m_use and l_run are
+  // updated here; rescaling O is left to the caller, who knows which P V products are already in O.
+  auto row_max_update = [&](const f32x16& s, float& alpha) -> bool {
+    float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
+#pragma unroll
+    for (int v = 3; v < 15; v += 2) mx = fmaxf(fmaxf(mx, s[v]), s[v + 1]);
+    mx = fmaxf(mx, s[15]);
+    mx = half_max(mx);
+    const float mxs = mx * c;
+    const bool grow = mxs > m_run + 8.0f;
+    alpha = 1.0f;
+    const bool any = __builtin_amdgcn_ballot_w64(grow) != 0;
+    if (any) {
+      const float m_new = grow ? mxs : m_run;
+      const float m_new_use = (m_new == -INFINITY) ? 0.f : m_new;
+      alpha = grow ? fast_exp2(m_run - m_new_use) : 1.0f;
+      m_run = m_new;
+      m_use = m_new_use;
+      l_run *= alpha;
+    }
+    return any;
+  };
+  auto rescale_o = [&](float alpha) {
 #pragma unroll
     for (int d = 0; d < DVB; d++)
 #pragma unroll
-      for (int v = 0; v < 16; v++) oacc[d][mr][v] = 0.f;
-  }
-  const float c = a.scale_log2;
-  const int wq_last = wq0 + 32 * MR - 1;
+      for (int v = 0; v < 16; v++) oacc[d][v] *= alpha;
+  };
+  auto exp_half = [&](f32x16& s, v8 (&pf)[2]) {
+    // (plain adds for the row sum: v_dot2 shares the matrix pipe and would serialise with the MFMAs)
+    float rs0 = 0.f, rs1 = 0.f;
+#pragma unroll
+    for (int v = 0; v < 16; v += 2) {
+      s[v] = fast_exp2(__builtin_fmaf(s[v], c, -m_use));
+      s[v + 1] = fast_exp2(__builtin_fmaf(s[v + 1], c, -m_use));
+      rs0 += s[v];
+      rs1 += s[v + 1];
+    }
+    l_run += rs0 + rs1;
+#pragma unroll
+    for (int hh = 0; hh < 2; hh++)
+      pf[hh] = pack8<T>(s[8 * hh + 0], s[8 * hh + 1], s[8 * hh + 2], s[8 * hh + 3], s[8 * hh + 4], s[8 * hh + 5],
+                        s[8 * hh + 6], s[8 * hh + 7]);
+  };
+
+  // One LDS tile.  Source order = intended overlap (each line is MFMA work next to independent VALU work):
+  //   S0 = K[0:32] Q^T                       | -
+  //   S1 = K[32:64] Q^T                      | exp(S0)
+  //   O += V[0:32]^T P0                      | exp(S1)
+  //   O += V[32:64]^T P1                     | transpose + LDS store of the next tile
+  // Fragments are read from LDS one phase ahead of their use.
+  auto tile_body = [&](auto masked_c, int t, int buf, bool has_next) {
+    constexpr bool MASKED = decltype(masked_c)::value;
+    const int kv0 = t * BN;
+    const unsigned char* kl = smem + buf * BUF_BYTES;
+    const unsigned char* vl = kl + K_BYTES;
+    const int* sl = (const int*)(vl + V_BYTES);
+    auto kfrag = [&](int hf, int ks) { return *(const v8*)(kl + KT::off(hf * 32 + ln, 16 * ks + 8 * g)); };
+    auto vfrag = [&](int hf, int kk, int d) { return *(const v8*)(vl + TrTile64::chunk_off(d * 32 + ln, 2 * hf + kk, g)); };
+    auto mask_half = [&](f32x16& s, int hf) {
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int kvl = hf * 32 + 8 * (v / 4) + 4 * g + (v % 4);
+        const int kv = kv0 + kvl;
+        const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
+        s[v] = ok ? s[v] : -INFINITY;
+      }
+    };
+
+    v8 fr[KSTEPS > 2 * DVB ? KSTEPS : 2 * DVB];  // fragments of the current phase
+    f32x16 s0, s1;
+#pragma unroll
+    for (int v = 0; v < 16; v++) { s0[v] = 0.f; s1[v] = 0.f; }
+    // phase 1
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) fr[ks] = kfrag(0, ks);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) s0 = MT<T>::mfma32(fr[ks], qf[ks], s0);
+    if (MASKED) mask_half(s0, 0);
+    float alpha0, alpha1;
+    if (row_max_update(s0, alpha0)) rescale_o(alpha0);
+    // phase 2: S1 MFMAs next to exp(S0)
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) fr[ks] = kfrag(1, ks);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) s1 = MT<T>::mfma32(fr[ks], qf[ks], s1);
+    v8 p0[2], p1[2];
+    exp_half(s0, p0);
+    if (MASKED) mask_half(s1, 1);
+    // P0 is relative to the reference max before this update: O is rescaled only after V0^T P0 is in it
+    const bool moved1 = row_max_update(s1, alpha1);
+    // phase 3: O += V0^T P0 next to exp(S1)
+#pragma unroll
+    for (int i = 0; i < 2 * DVB; i++) fr[i] = vfrag(0, i / DVB, i % DVB);
+#pragma unroll
+    for (int i = 0; i < 2 * DVB; i++) oacc[i % DVB] = MT<T>::mfma32(fr[i], p0[i / DVB], oacc[i % DVB]);
+    exp_half(s1, p1);
+    if (moved1) rescale_o(alpha1);
+    // phase 4: O += V1^T P1 next to the LDS store of the prefetched tile
+#pragma unroll
+    for (int i = 0; i < 2 * DVB; i++) fr[i] = vfrag(1, i / DVB, i % DVB);
+#pragma unroll
+    for (int i = 0; i < 2 * DVB; i++) oacc[i % DVB] = MT<T>::mfma32(fr[i], p1[i / DVB], oacc[i % DVB]);
+    if (has_next) store_tile(buf ^ 1);
+  };
 
   if (nact > 0) {
     load_tile(SEG ? active[0] : 0);
@@ -201,16 +307,16 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 
+  const int wq_last = wq0 + 31;
   for (int it = 0; it < nact; it++) {
     const int t = SEG ? active[it] : it;
     const int kv0 = t * BN;
     const int buf = it & 1;
-    if (it + 1 < nact) load_tile(SEG ? active[it + 1] : it + 1);
+    const bool has_next = it + 1 < nact;
+    if (has_next) load_tile(SEG ? active[it + 1] : it + 1);
 
-    const unsigned char* kl = smem + buf * BUF_BYTES;
-    const unsigned char* vl = kl + K_BYTES;
-    const int* sl = (const int*)(vl + V_BYTES);
-
+    // wave-uniform decisions: nothing to do above the diagonal or outside the rows' segments; element
+    // masks only on tiles that straddle the diagonal, the tail, or a segment boundary
     bool skip = CAUSAL && kv0 > wq_last;
     bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0);
     if (SEG) {
@@ -218,117 +324,30 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
       skip = skip || hi < wqmin || lo > wqmax;
       need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
     }
-    if (!skip) {
-      // ---- S^T = K Q^T
-      f32x16 sacc[NB][MR];
-#pragma unroll
-      for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-        for (int mr = 0; mr < MR; mr++)
-#pragma unroll
-          for (int v = 0; v < 16; v++) sacc[nb][mr][v] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ks++) {
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-          const v8 kf = *(const v8*)(kl + KT::off(nb * 32 + ln, 16 * ks + 8 * g));
-#pragma unroll
-          for (int mr = 0; mr < MR; mr++) sacc[nb][mr] = MT<T>::mfma32(kf, qf[mr][ks], sacc[nb][mr]);
-        }
-      }
-      // ---- mask (only tiles that straddle the diagonal, the tail, or a segment boundary)
-      if (need_mask) {
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
-#pragma unroll
-          for (int v = 0; v < 16; v++) {
-            const int kvl = nb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
-            const int kv = kv0 + kvl;
-            const int sk = SEG ? sl[kvl] : 0;
-#pragma unroll
-            for (int mr = 0; mr < MR; mr++) {
-              const int qrow = wq0 + mr * 32 + ln;
-              const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sk == segq[mr]);
-              sacc[nb][mr][v] = ok ? sacc[nb][mr][v] : -INFINITY;
-            }
-          }
-        }
-      }
-      // ---- online softmax, per lane = per query column
-      v8 pf[MR][BN / 16];
-#pragma unroll
-      for (int mr = 0; mr < MR; mr++) {
-        float mx = -INFINITY;
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-          for (int v = 0; v < 16; v++) mx = fmaxf(mx, sacc[nb][mr][v]);
-        mx = half_max(mx);
-        // Lazy rescale: the running max only moves when the tile max exceeds it by more than 2^8, so
-        // p stays <= 256 (harmless in fp32 sums and in the 16-bit P operand) and on most tiles no lane of
-        // the wave needs its accumulators rescaled.  O and l always share the same reference max.
-        const float mxs = mx * c;
-        const bool grow = mxs > m_run[mr] + 8.0f;
-        const float m_new = grow ? mxs : m_run[mr];
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = grow ? fast_exp2(m_run[mr] - m_use) : 1.0f;
-        m_run[mr] = m_new;
-        float rs = 0.f;
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-          for (int v = 0; v < 16; v++) {
-            const float p = fast_exp2(__builtin_fmaf(sacc[nb][mr][v], c, -m_use));
-            sacc[nb][mr][v] = p;
-            rs += p;
-          }
-        l_run[mr] = l_run[mr] * alpha + rs;
-        if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-#pragma unroll
-          for (int d = 0; d < DVB; d++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) oacc[d][mr][v] *= alpha;
-        }
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-          for (int hh = 0; hh < 2; hh++) {
-            const f32x16& s = sacc[nb][mr];
-            pf[mr][nb * 2 + hh] = pack8<T>(s[8 * hh + 0], s[8 * hh + 1], s[8 * hh + 2], s[8 * hh + 3], s[8 * hh + 4],
-                                           s[8 * hh + 5], s[8 * hh + 6], s[8 * hh + 7]);
-          }
-      }
-      // ---- O^T += V^T P^T
-#pragma unroll
-      for (int ks = 0; ks < BN / 16; ks++) {
-#pragma unroll
-        for (int d = 0; d < DVB; d++) {
-          const v8 vf = *(const v8*)(vl + TrTile64::chunk_off(d * 32 + ln, ks, g));
-#pragma unroll
-          for (int mr = 0; mr < MR; mr++) oacc[d][mr] = MT<T>::mfma32(vf, pf[mr][ks], oacc[d][mr]);
-        }
-      }
+    if (skip) {
+      if (has_next) store_tile(buf ^ 1);
+    } else if (need_mask) {
+      tile_body(std::true_type{}, t, buf, has_next);
+    } else {
+      tile_body(std::false_type{}, t, buf, has_next);
     }
-    if (it + 1 < nact) store_tile(buf ^ 1);
     __syncthreads();
   }
 
   // ---- epilogue: normalise, write O (row = query, 4 consecutive v-dims per store) and LSE
   T* ob = (T*)a.out + b * a.os[0] + h * a.os[1];
   float* lb = a.lse + ((int64_t)b * a.Hq + h) * Sq;
-#pragma unroll
-  for (int mr = 0; mr < MR; mr++) {
-    const int row = wq0 + mr * 32 + ln;
-    const float l = half_sum(l_run[mr]);
+  {
+    const float l = half_sum(l_run);
     const float inv = l > 0.f ? 1.f / l : 0.f;
-    if (row < Sq) {
-      if (g == 0) lb[row] = l > 0.f ? (m_run[mr] + log2f(l)) * LN2 : -INFINITY;
-      T* op = ob + row * a.os[2];
+    if (qrow < Sq) {
+      if (g == 0) lb[qrow] = l > 0.f ? (m_run + log2f(l)) * LN2 : -INFINITY;
+      T* op = ob + qrow * a.os[2];
 #pragma unroll
       for (int d = 0; d < DVB; d++)
 #pragma unroll
         for (int vq = 0; vq < 4; vq++) {
-          const f32x16& o = oacc[d][mr];
+          const f32x16& o = oacc[d];
           *(u32x2*)(op + d * 32 + 8 * vq + 4 * g) =
               pack4<T>(o[4 * vq] * inv, o[4 * vq + 1] * inv, o[4 * vq + 2] * inv, o[4 * vq + 3] * inv);
         }
@@ -339,14 +358,14 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
 // ------------------------------------------------------------------------------------------------
 // host dispatch
 // ------------------------------------------------------------------------------------------------
-template <typename T, int DQK, int DV, int MR, bool CAUSAL, bool SEG>
+template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
 static int launch_fwd(const FwdArgs& a, int B, hipStream_t st) {
-  constexpr int BN = 64, BM = 128 * MR;
+  constexpr int BN = 64, BM = 128;
   constexpr int BUF = BN * RowTile<DQK>::STRIDE + DV * TrTile64::ROW_BYTES + (SEG ? BN * 4 : 0);
   const int ntiles_max = (a.Skv + BN - 1) / BN;
   const size_t smem = 2 * (size_t)BUF + (SEG ? (size_t)(3 * ntiles_max + 8) * 4 : 0);
   TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_fwd: Skv=%d needs %zu bytes of LDS (max 163840)", a.Skv, smem);
-  auto kern = attn_fwd_kernel<T, DQK, DV, MR, CAUSAL, SEG>;
+  auto kern = attn_fwd_kernel<T, DQK, DV, CAUSAL, SEG>;
   static bool attr_set = false;  // benign race: every thread sets the same value
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -360,13 +379,12 @@ static int launch_fwd(const FwdArgs& a, int B, hipStream_t st) {
 
 template <typename T, int DQK, int DV>
 static int dispatch_fwd(const FwdArgs& a, int B, int causal, hipStream_t st) {
-  constexpr int MR = 1;
   if (causal) {
-    if (a.seg) return launch_fwd<T, DQK, DV, MR, true, true>(a, B, st);
-    return launch_fwd<T, DQK, DV, MR, true, false>(a, B, st);
+    if (a.seg) return launch_fwd<T, DQK, DV, true, true>(a, B, st);
+    return launch_fwd<T, DQK, DV, true, false>(a, B, st);
   }
-  if (a.seg) return launch_fwd<T, DQK, DV, MR, false, true>(a, B, st);
-  return launch_fwd<T, DQK, DV, MR, false, false>(a, B, st);
+  if (a.seg) return launch_fwd<T, DQK, DV, false, true>(a, B, st);
+  return launch_fwd<T, DQK, DV, false, false>(a, B, st);
 }
 
 }  // namespace tp
