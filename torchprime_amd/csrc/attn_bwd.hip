@@ -20,6 +20,8 @@
 //                         and delta are per-lane scalars) and dS^T feeds dQ^T += K^T dS^T.
 // Splitting dQ from dK/dV recomputes S and dP once more but needs no atomics: fp32 atomic adds reach
 // about 1.3 TB/s on this part, an order of magnitude short of what accumulating dQ tiles would need.
+#include <type_traits>
+
 #include "attn_common.hpp"
 
 namespace tp {
@@ -144,7 +146,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   typedef typename MT<T>::v8 v8;
   constexpr int BMQ = 64;   // query rows per streamed tile
   constexpr int BNK = 128;  // kv rows per workgroup, 32 per wave
-  constexpr int QB = BMQ / 32;
   constexpr int KS_QK = DQK / 16, KS_DV = DV / 16;
   constexpr int DKB = DQK / 32, DVB = DV / 32;
   typedef RowTile<DQK> QT;
@@ -301,80 +302,167 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       skip = skip || hi < wkmin || lo > wkmax;
       need_mask = need_mask || !(lo == hi && wkmin == wkmax && lo == wkmin);
     }
-    if (!skip) {
-      f32x16 sacc[QB], dpacc[QB];
-#pragma unroll
-      for (int qb = 0; qb < QB; qb++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) { sacc[qb][v] = 0.f; dpacc[qb][v] = 0.f; }
-      // S = Q K^T  (rows = queries, columns = this wave's kv rows)
-#pragma unroll
-      for (int ks = 0; ks < KS_QK; ks++)
-#pragma unroll
-        for (int qb = 0; qb < QB; qb++) {
-          const v8 qf = *(const v8*)(ql + QT::off(qb * 32 + ln, 16 * ks + 8 * g));
-          sacc[qb] = MT<T>::mfma32(qf, kf[ks], sacc[qb]);
-        }
-      // dP = dO V^T
-#pragma unroll
-      for (int ks = 0; ks < KS_DV; ks++)
-#pragma unroll
-        for (int qb = 0; qb < QB; qb++) {
-          const v8 dof = *(const v8*)(dol + OT::off(qb * 32 + ln, 16 * ks + 8 * g));
-          dpacc[qb] = MT<T>::mfma32(dof, vf[ks], dpacc[qb]);
-        }
-      // P = exp2(S*c - lse), dS = P o (dP - delta); rows of the C tile are queries
-      v8 pfr[BMQ / 16], dsf[BMQ / 16];
+    // The two 32-row query blocks of the tile are staggered so that every group of MFMAs has
+    // independent VALU work next to it (source order = intended overlap):
+    //   S0 = Q0 K^T, dP0 = dO0 V^T               |
+    //   S1 = Q1 K^T, dP1 = dO1 V^T               | P0 = exp2(S0 c - lse), dS0 = P0 o (dP0 - delta)
+    //   dV^T += dO0^T P0, dK^T += Q0^T dS0       | P1, dS1
+    //   dV^T += dO1^T P1, dK^T += Q1^T dS1       | (transpose + LDS store of the next tile)
+    auto body = [&](auto masked_c) {
+      constexpr bool MASKED = decltype(masked_c)::value;
       const int kvcol = wkv0 + ln;
+      auto s_dp = [&](int qb, f32x16& sa, f32x16& dp) {
 #pragma unroll
-      for (int qb = 0; qb < QB; qb++)
+        for (int v = 0; v < 16; v++) { sa[v] = 0.f; dp[v] = 0.f; }
 #pragma unroll
-        for (int vq = 0; vq < 4; vq++) {
-          const f32x4 l4 = *(const f32x4*)(lsel + qb * 32 + 8 * vq + 4 * g);
-#pragma unroll
-          for (int e = 0; e < 4; e++) sacc[qb][4 * vq + e] = fast_exp2(__builtin_fmaf(sacc[qb][4 * vq + e], c, -l4[e]));
+        for (int ks = 0; ks < KS_QK; ks++) {
+          const v8 f = *(const v8*)(ql + QT::off(qb * 32 + ln, 16 * ks + 8 * g));
+          sa = MT<T>::mfma32(f, kf[ks], sa);
         }
-      if (need_mask) {  // separate pass: the common unmasked tile carries no per-element branches
 #pragma unroll
-        for (int qb = 0; qb < QB; qb++)
-#pragma unroll
-          for (int v = 0; v < 16; v++) {
-            const int r = qb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
-            const int qrow = qi0 + r;
-            const bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || segl[r] == segk);
-            sacc[qb][v] = ok ? sacc[qb][v] : 0.f;
-          }
-      }
-#pragma unroll
-      for (int qb = 0; qb < QB; qb++) {
+        for (int ks = 0; ks < KS_DV; ks++) {
+          const v8 f = *(const v8*)(dol + OT::off(qb * 32 + ln, 16 * ks + 8 * g));
+          dp = MT<T>::mfma32(f, vf[ks], dp);
+        }
+      };
+      // P and dS of one query block, converted to the B operands of the accumulating products
+      auto p_ds = [&](int qb, f32x16& sa, f32x16& dp, v8 (&pf)[2], v8 (&df)[2]) {
 #pragma unroll
         for (int vq = 0; vq < 4; vq++) {
-          const f32x4 d4 = *(const f32x4*)(deltal + qb * 32 + 8 * vq + 4 * g);
+          const int r0 = qb * 32 + 8 * vq + 4 * g;
+          const f32x4 l4 = *(const f32x4*)(lsel + r0);
+          const f32x4 d4 = *(const f32x4*)(deltal + r0);
 #pragma unroll
-          for (int e = 0; e < 4; e++) dpacc[qb][4 * vq + e] = sacc[qb][4 * vq + e] * (dpacc[qb][4 * vq + e] - d4[e]);
+          for (int e = 0; e < 4; e++) {
+            const int v = 4 * vq + e;
+            float pv = fast_exp2(__builtin_fmaf(sa[v], c, -l4[e]));
+            if (MASKED) {
+              const int qrow = qi0 + r0 + e;
+              const bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || segl[r0 + e] == segk);
+              pv = ok ? pv : 0.f;
+            }
+            sa[v] = pv;
+            dp[v] = pv * (dp[v] - d4[e]);
+          }
         }
 #pragma unroll
         for (int hh = 0; hh < 2; hh++) {
-          const f32x16& s = sacc[qb];
-          const f32x16& d = dpacc[qb];
-          pfr[qb * 2 + hh] = pack8<T>(s[8 * hh + 0], s[8 * hh + 1], s[8 * hh + 2], s[8 * hh + 3], s[8 * hh + 4],
-                                      s[8 * hh + 5], s[8 * hh + 6], s[8 * hh + 7]);
-          dsf[qb * 2 + hh] = pack8<T>(d[8 * hh + 0], d[8 * hh + 1], d[8 * hh + 2], d[8 * hh + 3], d[8 * hh + 4],
-                                      d[8 * hh + 5], d[8 * hh + 6], d[8 * hh + 7]);
+          pf[hh] = pack8<T>(sa[8 * hh + 0], sa[8 * hh + 1], sa[8 * hh + 2], sa[8 * hh + 3], sa[8 * hh + 4],
+                            sa[8 * hh + 5], sa[8 * hh + 6], sa[8 * hh + 7]);
+          df[hh] = pack8<T>(dp[8 * hh + 0], dp[8 * hh + 1], dp[8 * hh + 2], dp[8 * hh + 3], dp[8 * hh + 4],
+                            dp[8 * hh + 5], dp[8 * hh + 6], dp[8 * hh + 7]);
         }
+      };
+      // dV^T += dO^T P, dK^T += Q^T dS over the 32 query rows of block qb (two k-steps of 16)
+      auto accumulate = [&](int qb, const v8 (&pf)[2], const v8 (&df)[2]) {
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++) {
+          const int ks = 2 * qb + hh;
+#pragma unroll
+          for (int d = 0; d < DVB; d++) {
+            const v8 f = *(const v8*)(dotl + TrTile64::chunk_off(d * 32 + ln, ks, g));
+            dvacc[d] = MT<T>::mfma32(f, pf[hh], dvacc[d]);
+          }
+#pragma unroll
+          for (int d = 0; d < DKB; d++) {
+            const v8 f = *(const v8*)(qtl + TrTile64::chunk_off(d * 32 + ln, ks, g));
+            dkacc[d] = MT<T>::mfma32(f, df[hh], dkacc[d]);
+          }
+        }
+      };
+      f32x16 s0, dp0, s1, dp1;
+      v8 pf0[2], df0[2], pf1[2], df1[2];
+      s_dp(0, s0, dp0);
+      s_dp(1, s1, dp1);
+      p_ds(0, s0, dp0, pf0, df0);
+      accumulate(0, pf0, df0);
+      p_ds(1, s1, dp1, pf1, df1);
+      accumulate(1, pf1, df1);
+    };
+    if constexpr (DQK <= 128) {
+      if (!skip) {
+        if (need_mask) body(std::true_type{});
+        else body(std::false_type{});
       }
-      // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 64 query rows)
-#pragma unroll
-      for (int ks = 0; ks < BMQ / 16; ks++) {
-#pragma unroll
-        for (int d = 0; d < DVB; d++) {
-          const v8 f = *(const v8*)(dotl + TrTile64::chunk_off(d * 32 + ln, ks, g));
-          dvacc[d] = MT<T>::mfma32(f, pfr[ks], dvacc[d]);
+    } else {
+      // Wider heads do not fit the staggered schedule in the register file: both query blocks go
+      // through each step together.
+      constexpr int QB = BMQ / 32;
+    if (!skip) {
+        f32x16 sacc[QB], dpacc[QB];
+  #pragma unroll
+        for (int qb = 0; qb < QB; qb++)
+  #pragma unroll
+          for (int v = 0; v < 16; v++) { sacc[qb][v] = 0.f; dpacc[qb][v] = 0.f; }
+        // S = Q K^T  (rows = queries, columns = this wave's kv rows)
+  #pragma unroll
+        for (int ks = 0; ks < KS_QK; ks++)
+  #pragma unroll
+          for (int qb = 0; qb < QB; qb++) {
+            const v8 qf = *(const v8*)(ql + QT::off(qb * 32 + ln, 16 * ks + 8 * g));
+            sacc[qb] = MT<T>::mfma32(qf, kf[ks], sacc[qb]);
+          }
+        // dP = dO V^T
+  #pragma unroll
+        for (int ks = 0; ks < KS_DV; ks++)
+  #pragma unroll
+          for (int qb = 0; qb < QB; qb++) {
+            const v8 dof = *(const v8*)(dol + OT::off(qb * 32 + ln, 16 * ks + 8 * g));
+            dpacc[qb] = MT<T>::mfma32(dof, vf[ks], dpacc[qb]);
+          }
+        // P = exp2(S*c - lse), dS = P o (dP - delta); rows of the C tile are queries
+        v8 pfr[BMQ / 16], dsf[BMQ / 16];
+        const int kvcol = wkv0 + ln;
+  #pragma unroll
+        for (int qb = 0; qb < QB; qb++)
+  #pragma unroll
+          for (int vq = 0; vq < 4; vq++) {
+            const f32x4 l4 = *(const f32x4*)(lsel + qb * 32 + 8 * vq + 4 * g);
+  #pragma unroll
+            for (int e = 0; e < 4; e++) sacc[qb][4 * vq + e] = fast_exp2(__builtin_fmaf(sacc[qb][4 * vq + e], c, -l4[e]));
+          }
+        if (need_mask) {  // separate pass: the common unmasked tile carries no per-element branches
+  #pragma unroll
+          for (int qb = 0; qb < QB; qb++)
+  #pragma unroll
+            for (int v = 0; v < 16; v++) {
+              const int r = qb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
+              const int qrow = qi0 + r;
+              const bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || segl[r] == segk);
+              sacc[qb][v] = ok ? sacc[qb][v] : 0.f;
+            }
         }
-#pragma unroll
-        for (int d = 0; d < DKB; d++) {
-          const v8 f = *(const v8*)(qtl + TrTile64::chunk_off(d * 32 + ln, ks, g));
-          dkacc[d] = MT<T>::mfma32(f, dsf[ks], dkacc[d]);
+  #pragma unroll
+        for (int qb = 0; qb < QB; qb++) {
+  #pragma unroll
+          for (int vq = 0; vq < 4; vq++) {
+            const f32x4 d4 = *(const f32x4*)(deltal + qb * 32 + 8 * vq + 4 * g);
+  #pragma unroll
+            for (int e = 0; e < 4; e++) dpacc[qb][4 * vq + e] = sacc[qb][4 * vq + e] * (dpacc[qb][4 * vq + e] - d4[e]);
+          }
+  #pragma unroll
+          for (int hh = 0; hh < 2; hh++) {
+            const f32x16& s = sacc[qb];
+            const f32x16& d = dpacc[qb];
+            pfr[qb * 2 + hh] = pack8<T>(s[8 * hh + 0], s[8 * hh + 1], s[8 * hh + 2], s[8 * hh + 3], s[8 * hh + 4],
+                                        s[8 * hh + 5], s[8 * hh + 6], s[8 * hh + 7]);
+            dsf[qb * 2 + hh] = pack8<T>(d[8 * hh + 0], d[8 * hh + 1], d[8 * hh + 2], d[8 * hh + 3], d[8 * hh + 4],
+                                        d[8 * hh + 5], d[8 * hh + 6], d[8 * hh + 7]);
+          }
+        }
+        // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 64 query rows)
+  #pragma unroll
+        for (int ks = 0; ks < BMQ / 16; ks++) {
+  #pragma unroll
+          for (int d = 0; d < DVB; d++) {
+            const v8 f = *(const v8*)(dotl + TrTile64::chunk_off(d * 32 + ln, ks, g));
+            dvacc[d] = MT<T>::mfma32(f, pfr[ks], dvacc[d]);
+          }
+  #pragma unroll
+          for (int d = 0; d < DKB; d++) {
+            const v8 f = *(const v8*)(qtl + TrTile64::chunk_off(d * 32 + ln, ks, g));
+            dkacc[d] = MT<T>::mfma32(f, dsf[ks], dkacc[d]);
+          }
         }
       }
     }
