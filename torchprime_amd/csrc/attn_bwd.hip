@@ -503,7 +503,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
 template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
 __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
   typedef typename MT<T>::v8 v8;
-  constexpr int BN = 64, BM = 128, NB = BN / 32;
+  constexpr int BN = 64, BM = 128;
   constexpr int KS_QK = DQK / 16, KS_DV = DV / 16, DKB = DQK / 32;
   typedef RowTile<DQK> KT;
   typedef RowTile<DV> VT;
@@ -639,62 +639,65 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
       skip = skip || hi < wqmin || lo > wqmax;
       need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
     }
-    if (!skip) {
-      f32x16 sacc[NB], dpacc[NB];
+    // The two 32-row kv blocks of the tile are staggered (source order = intended overlap):
+    //   S0^T = K0 Q^T, dP0^T = V0 dO^T          |
+    //   S1^T = K1 Q^T, dP1^T = V1 dO^T          | dS0^T = exp2(S0^T c - lse) o (dP0^T - delta)
+    //   dQ^T += K0^T dS0^T                      | dS1^T
+    //   dQ^T += K1^T dS1^T                      | (transpose + LDS store of the next tile)
+    auto body = [&](auto masked_c) {
+      constexpr bool MASKED = decltype(masked_c)::value;
+      auto s_dp = [&](int nb, f32x16& sa, f32x16& dp) {
 #pragma unroll
-      for (int nb = 0; nb < NB; nb++)
+        for (int v = 0; v < 16; v++) { sa[v] = 0.f; dp[v] = 0.f; }
 #pragma unroll
-        for (int v = 0; v < 16; v++) { sacc[nb][v] = 0.f; dpacc[nb][v] = 0.f; }
-      // S^T = K Q^T, dP^T = V dO^T  (rows = kv, columns = this wave's queries)
-#pragma unroll
-      for (int ks = 0; ks < KS_QK; ks++)
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
+        for (int ks = 0; ks < KS_QK; ks++) {
           const v8 f = *(const v8*)(kl + KT::off(nb * 32 + ln, 16 * ks + 8 * g));
-          sacc[nb] = MT<T>::mfma32(f, qf[ks], sacc[nb]);
+          sa = MT<T>::mfma32(f, qf[ks], sa);
         }
 #pragma unroll
-      for (int ks = 0; ks < KS_DV; ks++)
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++) {
+        for (int ks = 0; ks < KS_DV; ks++) {
           const v8 f = *(const v8*)(vl + VT::off(nb * 32 + ln, 16 * ks + 8 * g));
-          dpacc[nb] = MT<T>::mfma32(f, dof[ks], dpacc[nb]);
+          dp = MT<T>::mfma32(f, dof[ks], dp);
         }
-      v8 dsf[BN / 16];
+      };
+      auto ds_of = [&](int nb, f32x16& sa, f32x16& dp, v8 (&df)[2]) {
 #pragma unroll
-      for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) sacc[nb][v] = fast_exp2(__builtin_fmaf(sacc[nb][v], c, -lse_s));
-      if (need_mask) {  // separate pass: the common unmasked tile carries no per-element branches
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-          for (int v = 0; v < 16; v++) {
+        for (int v = 0; v < 16; v++) {
+          float pv = fast_exp2(__builtin_fmaf(sa[v], c, -lse_s));
+          if (MASKED) {
             const int kvl = nb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
             const int kv = kv0 + kvl;
             const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
-            sacc[nb][v] = ok ? sacc[nb][v] : 0.f;
+            pv = ok ? pv : 0.f;
           }
-      }
-#pragma unroll
-      for (int nb = 0; nb < NB; nb++) {
-#pragma unroll
-        for (int v = 0; v < 16; v++) dpacc[nb][v] = sacc[nb][v] * (dpacc[nb][v] - delta_s);
-#pragma unroll
-        for (int hh = 0; hh < 2; hh++) {
-          const f32x16& d = dpacc[nb];
-          dsf[nb * 2 + hh] = pack8<T>(d[8 * hh + 0], d[8 * hh + 1], d[8 * hh + 2], d[8 * hh + 3], d[8 * hh + 4],
-                                      d[8 * hh + 5], d[8 * hh + 6], d[8 * hh + 7]);
+          dp[v] = pv * (dp[v] - delta_s);
         }
-      }
-      // dQ^T += K^T dS^T  (contraction over the 64 kv rows)
 #pragma unroll
-      for (int ks = 0; ks < BN / 16; ks++)
+        for (int hh = 0; hh < 2; hh++)
+          df[hh] = pack8<T>(dp[8 * hh + 0], dp[8 * hh + 1], dp[8 * hh + 2], dp[8 * hh + 3], dp[8 * hh + 4],
+                            dp[8 * hh + 5], dp[8 * hh + 6], dp[8 * hh + 7]);
+      };
+      auto accumulate = [&](int nb, const v8 (&df)[2]) {
 #pragma unroll
-        for (int d = 0; d < DKB; d++) {
-          const v8 f = *(const v8*)(ktl + TrTile64::chunk_off(d * 32 + ln, ks, g));
-          dqacc[d] = MT<T>::mfma32(f, dsf[ks], dqacc[d]);
-        }
+        for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+          for (int d = 0; d < DKB; d++) {
+            const v8 f = *(const v8*)(ktl + TrTile64::chunk_off(d * 32 + ln, 2 * nb + hh, g));
+            dqacc[d] = MT<T>::mfma32(f, df[hh], dqacc[d]);
+          }
+      };
+      f32x16 s0, dp0, s1, dp1;
+      v8 df0[2], df1[2];
+      s_dp(0, s0, dp0);
+      s_dp(1, s1, dp1);
+      ds_of(0, s0, dp0, df0);
+      accumulate(0, df0);
+      ds_of(1, s1, dp1, df1);
+      accumulate(1, df1);
+    };
+    if (!skip) {
+      if (need_mask) body(std::true_type{});
+      else body(std::false_type{});
     }
     if (it + 1 < nact) store_tile(buf ^ 1);
     __syncthreads();
