@@ -158,8 +158,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, ln = lane & 31;
-  const int hk = blockIdx.y, b = blockIdx.z;
-  const int kv0 = blockIdx.x * BNK;
+  int tile, inner, group;
+  if (!xcd_map((a.Skv + BNK - 1) / BNK, 1, a.B * a.Hkv, tile, inner, group)) return;
+  const int b = group / a.Hkv, hk = group - b * a.Hkv;
+  const int kv0 = tile * BNK;  // low kv tiles see the most queries: they start first
   const int wkv0 = kv0 + wave * 32;
   const int Sq = a.Sq, Skv = a.Skv;
   const int32_t* segb = SEG ? a.seg + (int64_t)b * Skv : nullptr;
@@ -514,8 +516,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, ln = lane & 31;
-  const int qt = gridDim.x - 1 - blockIdx.x;
-  const int h = blockIdx.y, b = blockIdx.z, hk = h / a.n_rep;
+  const int n_qt = (a.Sq + BM - 1) / BM;
+  int tile, inner, group;
+  if (!xcd_map(n_qt, a.n_rep, a.B * a.Hkv, tile, inner, group)) return;
+  const int qt = n_qt - 1 - tile;
+  const int b = group / a.Hkv, hk = group - b * a.Hkv, h = hk * a.n_rep + inner;
   const int q0 = qt * BM, wq0 = q0 + wave * 32;
   const int Sq = a.Sq, Skv = a.Skv;
   const T* kb = (const T*)a.k + b * a.ks[0] + hk * a.ks[1];
@@ -757,7 +762,7 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
       if (rc) return rc;
       attr_set = true;
     }
-    kern<<<dim3((a.Skv + BNK - 1) / BNK, a.Hkv, a.B), dim3(256), smem, st>>>(a);
+    kern<<<dim3(xcd_grid((a.Skv + BNK - 1) / BNK, 1, a.B * a.Hkv)), dim3(256), smem, st>>>(a);
     int rc = check_launch("tp_attn_bwd(dkdv)");
     if (rc) return rc;
   }
@@ -776,7 +781,7 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
       if (rc) return rc;
       attr_set = true;
     }
-    kern<<<dim3((a.Sq + BM - 1) / BM, a.Hq, a.B), dim3(256), smem, st>>>(a);
+    kern<<<dim3(xcd_grid((a.Sq + BM - 1) / BM, a.n_rep, a.B * a.Hkv)), dim3(256), smem, st>>>(a);
     int rc = check_launch("tp_attn_bwd(dq)");
     if (rc) return rc;
   }
@@ -818,7 +823,7 @@ extern "C" int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, co
   TP_REQUIRE(!seg || Sq == Skv, TP_ERR_BAD_ARG, "tp_attn_bwd: segment ids need Sq == Skv (got %d, %d)", Sq, Skv);
   TP_REQUIRE(sm_scale > 0.f, TP_ERR_BAD_ARG, "tp_attn_bwd: sm_scale must be positive");
   TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F16, TP_ERR_UNSUPPORTED, "tp_attn_bwd: dtype %d (bf16 and fp16 only)", dtype);
-  TP_REQUIRE(B <= 65535 && Hq <= 65535, TP_ERR_UNSUPPORTED, "tp_attn_bwd: batch and heads are limited to 65535");
+  TP_REQUIRE((int64_t)(B + 8) * Hq * ((Sq + 127) / 128 + (Skv + 127) / 128) < (1ll << 31), TP_ERR_UNSUPPORTED, "tp_attn_bwd: too many workgroups");
   BwdArgs a;
   a.q = q; a.k = k; a.v = v; a.out = out; a.dout = dout; a.lse = lse; a.seg = seg;
   a.dq = dq; a.dk = dk; a.dv = dv; a.delta = ws;

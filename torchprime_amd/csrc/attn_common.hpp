@@ -93,6 +93,28 @@ __device__ __forceinline__ unsigned span_bytes(int rows, int64_t stride, int row
   return (unsigned)(((int64_t)(rows - 1) * stride + row_elems) * 2);
 }
 
+// ---- workgroup -> work mapping ---------------------------------------------------------------------
+// The 256 CUs sit in 8 XCDs with one L2 each, and workgroups of a 1-D grid are handed to the XCDs round
+// robin by linear id.  Work is therefore numbered so that every workgroup that streams the same K/V (or
+// Q/dO) slice - one (batch, kv head) "group" - lands on the same XCD and runs at about the same time:
+//     id = (group_local * per_group + r) * 8 + xcd,   group = group_local * 8 + xcd,
+//     r  = tile * n_inner + inner   (tiles outer so the heaviest tiles start first).
+// Returns false for the padding ids of a group count that is not a multiple of 8.
+constexpr int NUM_XCD = 8;
+__device__ __forceinline__ bool xcd_map(int n_tiles, int n_inner, int n_groups, int& tile, int& inner, int& group) {
+  const int n = blockIdx.x;
+  const int xcd = n % NUM_XCD, slot = n / NUM_XCD;
+  const int per_group = n_tiles * n_inner;
+  const int gl = slot / per_group, r = slot - gl * per_group;
+  group = gl * NUM_XCD + xcd;
+  tile = r / n_inner;
+  inner = r - tile * n_inner;
+  return group < n_groups;
+}
+inline unsigned xcd_grid(int n_tiles, int n_inner, int n_groups) {
+  return (unsigned)(NUM_XCD * ((n_groups + NUM_XCD - 1) / NUM_XCD) * n_tiles * n_inner);
+}
+
 // ---- LDS layouts ---------------------------------------------------------------------------------
 // Row-major tile [rows][D] of 16-bit elements: rows padded by 16 bytes so that 16-byte reads by lanes
 // in consecutive rows land in different banks.

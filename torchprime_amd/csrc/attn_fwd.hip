@@ -28,7 +28,7 @@ struct FwdArgs {
   const int32_t* seg;
   void* out;
   float* lse;
-  int Hq, Hkv, Sq, Skv, n_rep;
+  int B, Hq, Hkv, Sq, Skv, n_rep;
   int64_t qs[3], ks[3], vs[3], os[3];
   float scale_log2;  // sm_scale * log2(e)
 };
@@ -54,8 +54,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, ln = lane & 31;
-  const int qt = gridDim.x - 1 - blockIdx.x;  // longest (latest) query tiles are scheduled first
-  const int h = blockIdx.y, b = blockIdx.z, hk = h / a.n_rep;
+  const int n_qt = (a.Sq + BM - 1) / BM;
+  int tile, inner, group;
+  if (!xcd_map(n_qt, a.n_rep, a.B * a.Hkv, tile, inner, group)) return;
+  const int qt = n_qt - 1 - tile;  // longest (latest) query tiles are scheduled first
+  const int b = group / a.Hkv, hk = group - b * a.Hkv, h = hk * a.n_rep + inner;
   const int q0 = qt * BM;
   const int wq0 = q0 + wave * 32;
   const int Sq = a.Sq, Skv = a.Skv;
@@ -372,7 +375,7 @@ static int launch_fwd(const FwdArgs& a, int B, hipStream_t st) {
     TP_REQUIRE(e == hipSuccess, TP_ERR_LAUNCH, "tp_attn_fwd: hipFuncSetAttribute failed: %s", hipGetErrorString(e));
     attr_set = true;
   }
-  const dim3 grid((a.Sq + BM - 1) / BM, a.Hq, B), block(256);
+  const dim3 grid(xcd_grid((a.Sq + BM - 1) / BM, a.n_rep, B * a.Hkv)), block(256);
   kern<<<grid, block, smem, st>>>(a);
   return check_launch("tp_attn_fwd");
 }
@@ -402,10 +405,10 @@ extern "C" int tp_attn_fwd(const void* q, const void* k, const void* v, const in
   TP_REQUIRE(!seg || Sq == Skv, TP_ERR_BAD_ARG, "tp_attn_fwd: segment ids need Sq == Skv (got %d, %d)", Sq, Skv);
   TP_REQUIRE(sm_scale > 0.f, TP_ERR_BAD_ARG, "tp_attn_fwd: sm_scale must be positive");
   TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F16, TP_ERR_UNSUPPORTED, "tp_attn_fwd: dtype %d (bf16 and fp16 only)", dtype);
-  TP_REQUIRE(B <= 65535 && Hq <= 65535, TP_ERR_UNSUPPORTED, "tp_attn_fwd: batch and heads are limited to 65535");
+  TP_REQUIRE((int64_t)(B + 8) * Hq * ((Sq + 127) / 128) < (1ll << 31), TP_ERR_UNSUPPORTED, "tp_attn_fwd: too many workgroups");
   FwdArgs a;
   a.q = q; a.k = k; a.v = v; a.seg = seg; a.out = out; a.lse = lse;
-  a.Hq = Hq; a.Hkv = Hkv; a.Sq = Sq; a.Skv = Skv; a.n_rep = Hq / Hkv;
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.Sq = Sq; a.Skv = Skv; a.n_rep = Hq / Hkv;
   bool ok = aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out);
   for (int i = 0; i < 3; i++) {
     a.qs[i] = q_strides[i]; a.ks[i] = k_strides[i]; a.vs[i] = v_strides[i]; a.os[i] = o_strides[i];
