@@ -45,15 +45,16 @@ def test_c_abi_validates_arguments_before_launching():
   assert lib.tp_rmsnorm_fwd(p, p, p, p, 4, 8, 4, 8, 1e-6, 0, 0, None) == -1  # stride < hidden
   assert lib.tp_rmsnorm_fwd(p, p, p, p, 4, 8, 8, 8, 1e-6, 2, 0, None) == -2  # fp32 x with bf16 weight
   assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 3, 2, 8, 8, 128, 128, z3, z3, z3, z3, 0.1, 1, 0, None) == -1  # Hq % Hkv
-  assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 96, 96, z3, z3, z3, z3, 0.1, 1, 0, None) == -2  # head dim
+  s96 = _lib._I64x3(8 * 2 * 96, 96, 2 * 96)
+  assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 96, 96, s96, s96, s96, s96, 0.1, 1, 0, None) == -2  # head dim
   assert b"not built" in lib.tp_last_error()
   assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 128, 128, z3, z3, z3, z3, 0.1, 1, 2, None) == -2  # fp32
   assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 128, 128, z3, z3, z3, z3, -1.0, 1, 0, None) == -1  # scale
   assert lib.tp_attn_fwd(p, p, p, p, p, p, 1, 2, 2, 8, 16, 128, 128, z3, z3, z3, z3, 0.1, 1, 0, None) == -1  # seg, Sq != Skv
   assert lib.tp_rope_apply(p, None, p, p, None, p, None, 1, 2, 0, 8, 24, z3, z3, z3, z3, 0, 24, 0, 0, 0, 0, None) == -2  # D % 16
   assert lib.tp_rope_apply(p + 2, None, p, p, None, p, None, 1, 2, 0, 8, 32, z3, z3, z3, z3, 0, 32, 0, 0, 0, 0, None) == -1  # alignment
-  assert lib.tp_rmsnorm_bwd_workspace_bytes(32768, 4096) == 1024 * 4096 * 4
-  assert lib.tp_rmsnorm_bwd_workspace_bytes(10, 64) == 3 * 64 * 4
+  assert lib.tp_rmsnorm_bwd_workspace_bytes(32768, 4096) == 2048 * 4096 * 4
+  assert lib.tp_rmsnorm_bwd_workspace_bytes(10, 64) == 12 * 64 * 4
   assert lib.tp_attn_bwd_workspace_bytes(4, 32, 8192) == 4 * 32 * 8192 * 4
 
 

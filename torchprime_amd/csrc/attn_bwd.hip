@@ -841,8 +841,9 @@ extern "C" int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, co
     // tiles are addressed with 32-bit byte offsets inside one (batch, head) slice
     const int64_t lim = 1ll << 31;
     const bool fits = ((int64_t)Sq * q_strides[2] + Dqk) * 2 < lim && ((int64_t)Sq * do_strides[2] + Dv) * 2 < lim &&
-                      ((int64_t)Skv * k_strides[2] + Dqk) * 2 < lim && ((int64_t)Skv * v_strides[2] + Dv) * 2 < lim &&
-                      q_strides[2] > 0 && do_strides[2] > 0 && k_strides[2] > 0 && v_strides[2] > 0;
+                      ((int64_t)Skv * k_strides[2] + Dqk) * 2 < lim && ((int64_t)Skv * v_strides[2] + Dv) * 2 < lim;
+    TP_REQUIRE(q_strides[2] > 0 && do_strides[2] > 0 && k_strides[2] > 0 && v_strides[2] > 0, TP_ERR_BAD_ARG,
+               "tp_attn_bwd: sequence strides must be positive");
     TP_REQUIRE(fits, TP_ERR_UNSUPPORTED, "tp_attn_bwd: one (batch, head) slice of q, dO, k or v spans 2 GiB or more");
   }
   a.scale_log2 = sm_scale * LOG2E;

@@ -416,8 +416,8 @@ extern "C" int tp_attn_fwd(const void* q, const void* k, const void* v, const in
   }
   TP_REQUIRE(ok, TP_ERR_BAD_ARG, "tp_attn_fwd: pointers and strides must keep rows 16-byte aligned");
   // tiles are addressed with 32-bit byte offsets inside one (batch, head) slice
-  TP_REQUIRE(((int64_t)Skv * k_strides[2] + Dqk) * 2 < (1ll << 31) && ((int64_t)Skv * v_strides[2] + Dv) * 2 < (1ll << 31) &&
-                 k_strides[2] > 0 && v_strides[2] > 0,
+  TP_REQUIRE(k_strides[2] > 0 && v_strides[2] > 0, TP_ERR_BAD_ARG, "tp_attn_fwd: k / v sequence strides must be positive");
+  TP_REQUIRE(((int64_t)Skv * k_strides[2] + Dqk) * 2 < (1ll << 31) && ((int64_t)Skv * v_strides[2] + Dv) * 2 < (1ll << 31),
              TP_ERR_UNSUPPORTED, "tp_attn_fwd: one (batch, head) slice of k or v spans 2 GiB or more");
   a.scale_log2 = sm_scale * LOG2E;
   hipStream_t st = (hipStream_t)stream;

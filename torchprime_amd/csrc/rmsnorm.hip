@@ -9,25 +9,40 @@
 
 namespace tp {
 
-constexpr int RMS_MAX_PARTS = 1024;  // partial dw rows written by the backward
+constexpr int RMS_MAX_PARTS = 2048;  // partial dw rows written by the backward (multiple of 4)
 
 static inline int rms_parts(int64_t rows) {
-  int64_t p = (rows + 3) / 4;
+  int64_t p = (rows + 3) / 4 * 4;
   return (int)(p < RMS_MAX_PARTS ? p : RMS_MAX_PARTS);
 }
 
+// sum over the WAVES waves that share a row (fixed order); `red` holds 4 floats per buffer
+template <int WAVES>
+__device__ __forceinline__ float row_sum(float v, float* red, int wave) {
+  v = wave_sum(v);
+  if (WAVES == 1) return v;
+  if ((threadIdx.x & 63) == 0) red[wave] = v;
+  __syncthreads();
+  return ((red[0] + red[1]) + red[2]) + red[3];
+}
+
 // ------------------------------------------------------------------------------------------------
-// forward, vector path: NV 16-byte vectors of x per lane
+// forward, vector path.  A row is shared by WAVES waves (1 for short rows, else the whole 256-thread
+// block), each thread holding NV 16-byte vectors: few bytes per thread and many waves in flight is what
+// streams fastest on this part.  x and y are non-temporal (touched once), the weight is not.
 // ------------------------------------------------------------------------------------------------
-template <typename XT, typename WT, typename OT, int NV>
+template <typename XT, typename WT, typename OT, int NV, int WAVES>
 __global__ __launch_bounds__(256) void rmsnorm_fwd_vec(const XT* __restrict__ x, const WT* __restrict__ w,
                                                        OT* __restrict__ y, float* __restrict__ rstd,
                                                        int64_t rows, int hidden, int64_t xs, int64_t ys,
                                                        float eps) {
   constexpr int E = 16 / sizeof(XT);
-  const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= rows) return;
+  constexpr int RPB = 4 / WAVES, TPR = 64 * WAVES;
+  __shared__ float red[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row = (int64_t)blockIdx.x * RPB + wave / WAVES;
+  const int t = (wave % WAVES) * 64 + lane;
+  if (row >= rows) return;  // uniform per block when WAVES == 4
   const int nvec = hidden / E;
   const XT* xr = x + row * xs;
   OT* yr = y + row * ys;
@@ -36,25 +51,25 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_vec(const XT* __restrict__ x,
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < NV; i++) {
-    const int v = lane + 64 * i;
+    const int v = t + TPR * i;
     if (v < nvec) {
-      load_f<XT, E>(xr + (int64_t)v * E, xv[i]);
+      load_f_nt<XT, E>(xr + (int64_t)v * E, xv[i]);
 #pragma unroll
       for (int e = 0; e < E; e++) ss += xv[i][e] * xv[i][e];
     }
   }
-  ss = wave_sum(ss);
+  ss = row_sum<WAVES>(ss, red, wave);
   const float r = rsqrtf(ss / (float)hidden + eps);
-  if (lane == 0) rstd[row] = r;
+  if (t == 0) rstd[row] = r;
 #pragma unroll
   for (int i = 0; i < NV; i++) {
-    const int v = lane + 64 * i;
+    const int v = t + TPR * i;
     if (v < nvec) {
       float wv[E], o[E];
       load_f<WT, E>(w + (int64_t)v * E, wv);
 #pragma unroll
       for (int e = 0; e < E; e++) o[e] = wv[e] * round_to<XT>(xv[i][e] * r);
-      store_f<OT, E>(yr + (int64_t)v * E, o);
+      store_f_nt<OT, E>(yr + (int64_t)v * E, o);
     }
   }
 }
@@ -83,30 +98,36 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_generic(const XT* __restrict_
 }
 
 // ------------------------------------------------------------------------------------------------
-// backward, vector path.  Each wave walks rows gw, gw+nw, ...; dw partial sums stay in registers
-// and are folded over the block's four waves through LDS, one partial row per block.
+// backward, vector path.  Same thread layout as the forward; a block walks rows r, r + gridDim.x*RPB, ...
+// Each thread owns fixed columns, so its dw partial sums stay in registers over all the rows it sees and
+// go straight to one partial row per (block, row slot): no atomics, no cross-thread fold.
 // ------------------------------------------------------------------------------------------------
-template <typename XT, typename WT, typename OT, int NV>
+template <typename XT, typename WT, typename OT, int NV, int WAVES>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_vec(const OT* __restrict__ dy, const XT* __restrict__ x,
                                                        const WT* __restrict__ w, const float* __restrict__ rstd,
                                                        XT* __restrict__ dx, float* __restrict__ ws, int64_t rows,
                                                        int hidden, int64_t dys, int64_t xs, int64_t dxs) {
   constexpr int E = 16 / sizeof(XT);
-  extern __shared__ float red[];  // hidden floats
+  constexpr int RPB = 4 / WAVES, TPR = 64 * WAVES;
+  __shared__ float red[2][4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int slot = wave / WAVES;
+  const int t = (wave % WAVES) * 64 + lane;
   const int nvec = hidden / E;
-  const int64_t gw = (int64_t)blockIdx.x * 4 + wave, nw = (int64_t)gridDim.x * 4;
   const float inv_h = 1.f / (float)hidden;
+  const int64_t step = (int64_t)gridDim.x * RPB;
 
   float wv[NV][E], wacc[NV][E];
 #pragma unroll
   for (int i = 0; i < NV; i++) {
-    const int v = lane + 64 * i;
+    const int v = t + TPR * i;
 #pragma unroll
     for (int e = 0; e < E; e++) { wacc[i][e] = 0.f; wv[i][e] = 0.f; }
     if (v < nvec) load_f<WT, E>(w + (int64_t)v * E, wv[i]);
   }
-  for (int64_t row = gw; row < rows; row += nw) {
+  int it = 0;
+  // with WAVES == 4 all waves of the block share the row, so the loop bound is uniform for the barrier
+  for (int64_t row = (int64_t)blockIdx.x * RPB + slot; row < rows; row += step, it++) {
     const float r = rstd[row];
     const XT* xr = x + row * xs;
     const OT* gr = dy + row * dys;
@@ -115,11 +136,11 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_vec(const OT* __restrict__ dy
     float c = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-      const int v = lane + 64 * i;
+      const int v = t + TPR * i;
       if (v < nvec) {
         float dyv[E];
-        load_f<XT, E>(xr + (int64_t)v * E, n[i]);
-        load_f<OT, E>(gr + (int64_t)v * E, dyv);
+        load_f_nt<XT, E>(xr + (int64_t)v * E, n[i]);
+        load_f_nt<OT, E>(gr + (int64_t)v * E, dyv);
 #pragma unroll
         for (int e = 0; e < E; e++) {
           n[i][e] *= r;
@@ -129,37 +150,24 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_vec(const OT* __restrict__ dy
         }
       }
     }
-    c = wave_sum(c) * inv_h;
+    c = row_sum<WAVES>(c, red[it & 1], wave) * inv_h;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-      const int v = lane + 64 * i;
+      const int v = t + TPR * i;
       if (v < nvec) {
         float o[E];
 #pragma unroll
         for (int e = 0; e < E; e++) o[e] = r * (g[i][e] - n[i][e] * c);
-        store_f<XT, E>(dr + (int64_t)v * E, o);
+        store_f_nt<XT, E>(dr + (int64_t)v * E, o);
       }
     }
   }
-  // fold the four waves in a fixed order
-  for (int k = 0; k < 4; k++) {
-    if (wave == k) {
+  float* out = ws + ((int64_t)blockIdx.x * RPB + slot) * hidden;
 #pragma unroll
-      for (int i = 0; i < NV; i++) {
-        const int v = lane + 64 * i;
-        if (v < nvec) {
-#pragma unroll
-          for (int e = 0; e < E; e++) {
-            if (k == 0) red[v * E + e] = wacc[i][e];
-            else red[v * E + e] += wacc[i][e];
-          }
-        }
-      }
-    }
-    __syncthreads();
+  for (int i = 0; i < NV; i++) {
+    const int v = t + TPR * i;
+    if (v < nvec) store_f<float, E>(out + (int64_t)v * E, wacc[i]);
   }
-  float* out = ws + (int64_t)blockIdx.x * hidden;
-  for (int c = threadIdx.x; c < hidden; c += 256) out[c] = red[c];
 }
 
 // backward dx, any hidden / alignment
@@ -198,22 +206,24 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_dw_generic(const OT* __restri
   ws[(int64_t)blockIdx.y * hidden + c] = acc;
 }
 
-// dw[c] = sum_p ws[p, c], fixed order
+// dw[c] = sum_p ws[p, c], fixed order: 32 columns per block, 8 row groups folded through LDS
 template <typename WT>
 __global__ __launch_bounds__(256) void rmsnorm_dw_reduce(const float* __restrict__ ws, WT* __restrict__ dw, int parts,
                                                          int hidden) {
   __shared__ float red[256];
-  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
-  const int g = threadIdx.x >> 6;
+  const int c = blockIdx.x * 32 + (threadIdx.x & 31);
+  const int g = threadIdx.x >> 5;
   float acc = 0.f;
   if (c < hidden) {
 #pragma unroll 8
-    for (int p = g; p < parts; p += 4) acc += ws[(int64_t)p * hidden + c];
+    for (int p = g; p < parts; p += 8) acc += ws[(int64_t)p * hidden + c];
   }
   red[threadIdx.x] = acc;
   __syncthreads();
   if (g == 0 && c < hidden) {
-    const float s = ((red[threadIdx.x] + red[threadIdx.x + 64]) + red[threadIdx.x + 128]) + red[threadIdx.x + 192];
+    float s = red[threadIdx.x];
+#pragma unroll
+    for (int k = 1; k < 8; k++) s += red[threadIdx.x + 32 * k];
     dw[c] = Elem<WT>::from_f(s);
   }
 }
@@ -228,16 +238,18 @@ static int fwd_typed(const void* x, const void* w, void* y, float* rstd, int64_t
   const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
   const XT* xp = (const XT*)x; const WT* wp = (const WT*)w; OT* yp = (OT*)y;
   const bool vec = hidden % E == 0 && aligned16(x) && aligned16(w) && aligned16(y) && (xs * sizeof(XT)) % 16 == 0 &&
-                   (ys * sizeof(OT)) % 16 == 0 && hidden / E <= 64 * 32;
+                   (ys * sizeof(OT)) % 16 == 0 && hidden / E <= 256 * 8;
   if (vec) {
-    const int per = (hidden / E + 63) / 64;
-#define TP_RMS_FWD(NV) rmsnorm_fwd_vec<XT, WT, OT, NV><<<grid, block, 0, st>>>(xp, wp, yp, rstd, rows, hidden, xs, ys, eps)
-    if (per <= 1) TP_RMS_FWD(1);
-    else if (per <= 2) TP_RMS_FWD(2);
-    else if (per <= 4) TP_RMS_FWD(4);
-    else if (per <= 8) TP_RMS_FWD(8);
-    else if (per <= 16) TP_RMS_FWD(16);
-    else TP_RMS_FWD(32);
+    const int nvec = hidden / E;
+#define TP_RMS_FWD(NV, WAVES)                                                                                  \
+  rmsnorm_fwd_vec<XT, WT, OT, NV, WAVES><<<dim3((unsigned)((rows + 4 / WAVES - 1) / (4 / WAVES))), block, 0, st>>>( \
+      xp, wp, yp, rstd, rows, hidden, xs, ys, eps)
+    if (nvec <= 64) TP_RMS_FWD(1, 1);
+    else if (nvec <= 128) TP_RMS_FWD(2, 1);
+    else if (nvec <= 256) TP_RMS_FWD(1, 4);
+    else if (nvec <= 512) TP_RMS_FWD(2, 4);
+    else if (nvec <= 1024) TP_RMS_FWD(4, 4);
+    else TP_RMS_FWD(8, 4);
 #undef TP_RMS_FWD
   } else {
     rmsnorm_fwd_generic<XT, WT, OT><<<grid, block, 0, st>>>(xp, wp, yp, rstd, rows, hidden, xs, ys, eps);
@@ -251,20 +263,21 @@ static int bwd_typed(const void* dy, const void* x, const void* w, const float* 
   constexpr int E = 16 / sizeof(XT);
   const OT* gp = (const OT*)dy; const XT* xp = (const XT*)x; const WT* wp = (const WT*)w; XT* dxp = (XT*)dx;
   const int parts = rms_parts(rows);
-  const int per = (hidden / E + 63) / 64;
+  const int nvec = hidden / E;
   const bool vec = hidden % E == 0 && aligned16(dy) && aligned16(x) && aligned16(w) && aligned16(dx) &&
                    (dys * sizeof(OT)) % 16 == 0 && (xs * sizeof(XT)) % 16 == 0 && (dxs * sizeof(XT)) % 16 == 0 &&
-                   per * E <= 128 && (size_t)hidden * 4 <= 64 * 1024;
+                   nvec <= 256 * 8;
   if (vec) {
-    const dim3 grid(parts), block(256);
-    const size_t sh = (size_t)hidden * sizeof(float);
-#define TP_RMS_BWD(NV) rmsnorm_bwd_vec<XT, WT, OT, NV><<<grid, block, sh, st>>>(gp, xp, wp, rstd, dxp, ws, rows, hidden, dys, xs, dxs)
-    if (per <= 1) TP_RMS_BWD(1);
-    else if (per <= 2) TP_RMS_BWD(2);
-    else if (per <= 4) TP_RMS_BWD(4);
-    else if (per <= 8) TP_RMS_BWD(8);
-    else if (per <= 16) TP_RMS_BWD(16);
-    else TP_RMS_BWD(32);
+    const dim3 block(256);
+#define TP_RMS_BWD(NV, WAVES)                                                                             \
+  rmsnorm_bwd_vec<XT, WT, OT, NV, WAVES><<<dim3(parts / (4 / WAVES)), block, 0, st>>>(gp, xp, wp, rstd, dxp, ws, rows, \
+                                                                                     hidden, dys, xs, dxs)
+    if (nvec <= 64) TP_RMS_BWD(1, 1);
+    else if (nvec <= 128) TP_RMS_BWD(2, 1);
+    else if (nvec <= 256) TP_RMS_BWD(1, 4);
+    else if (nvec <= 512) TP_RMS_BWD(2, 4);
+    else if (nvec <= 1024) TP_RMS_BWD(4, 4);
+    else TP_RMS_BWD(8, 4);
 #undef TP_RMS_BWD
   } else {
     rmsnorm_bwd_dx_generic<XT, WT, OT><<<dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st>>>(gp, xp, wp, rstd, dxp, rows,
@@ -272,7 +285,7 @@ static int bwd_typed(const void* dy, const void* x, const void* w, const float* 
     rmsnorm_bwd_dw_generic<XT, OT><<<dim3((hidden + 255) / 256, parts), dim3(256), 0, st>>>(gp, xp, rstd, ws, rows, hidden,
                                                                                           dys, xs);
   }
-  rmsnorm_dw_reduce<WT><<<dim3((hidden + 63) / 64), dim3(256), 0, st>>>(ws, (WT*)dw, parts, hidden);
+  rmsnorm_dw_reduce<WT><<<dim3((hidden + 31) / 32), dim3(256), 0, st>>>(ws, (WT*)dw, parts, hidden);
   return check_launch("tp_rmsnorm_bwd");
 }
 

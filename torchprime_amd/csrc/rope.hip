@@ -57,12 +57,23 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
   const int64_t total = (int64_t)a.B * a.S * Htot * VH;
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= total) return;
-  const int j = (int)(idx % VH);
-  int64_t t = idx / VH;
-  int h = (int)(t % Htot);
-  t /= Htot;
-  const int s = (int)(t % a.S);
-  const int b = (int)(t / a.S);
+  int j, h, s, b;
+  if (total <= 0xffffffffll) {  // the usual case: 32-bit divisions are several times cheaper
+    const unsigned i32 = (unsigned)idx;
+    const unsigned t1 = i32 / (unsigned)VH;
+    j = (int)(i32 - t1 * (unsigned)VH);
+    const unsigned t2 = t1 / (unsigned)Htot;
+    h = (int)(t1 - t2 * (unsigned)Htot);
+    b = (int)(t2 / (unsigned)a.S);
+    s = (int)(t2 - (unsigned)b * (unsigned)a.S);
+  } else {
+    j = (int)(idx % VH);
+    int64_t t = idx / VH;
+    h = (int)(t % Htot);
+    t /= Htot;
+    s = (int)(t % a.S);
+    b = (int)(t / a.S);
+  }
   const int which = h >= a.H[0] ? 1 : 0;
   h -= which ? a.H[0] : 0;
 
@@ -82,13 +93,13 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
 
   float x1[E], x2[E], o1[E], o2[E];
   if (!INTERLEAVED || BACKWARD) {
-    load_f<T, E>(xp + j * E, x1);
-    load_f<T, E>(xp + half + j * E, x2);
+    load_f_nt<T, E>(xp + j * E, x1);
+    load_f_nt<T, E>(xp + half + j * E, x2);
   } else {
     // permuted input: first-half element i is x[2i], second-half element i is x[2i+1]
     float lo[E], hi[E];
-    load_f<T, E>(xp + 2 * j * E, lo);
-    load_f<T, E>(xp + 2 * j * E + E, hi);
+    load_f_nt<T, E>(xp + 2 * j * E, lo);
+    load_f_nt<T, E>(xp + 2 * j * E + E, hi);
 #pragma unroll
     for (int e = 0; e < E / 2; e++) {
       x1[e] = lo[2 * e];
@@ -111,8 +122,8 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
     }
   }
   if (!INTERLEAVED || !BACKWARD) {
-    store_f<T, E>(yp + j * E, o1);
-    store_f<T, E>(yp + half + j * E, o2);
+    store_f_nt<T, E>(yp + j * E, o1);
+    store_f_nt<T, E>(yp + half + j * E, o2);
   } else {
     // inverse permutation: dx[2i] = d_first[i], dx[2i+1] = d_second[i]
     float lo[E], hi[E];
@@ -123,8 +134,8 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
       hi[2 * e] = o1[E / 2 + e];
       hi[2 * e + 1] = o2[E / 2 + e];
     }
-    store_f<T, E>(yp + 2 * j * E, lo);
-    store_f<T, E>(yp + 2 * j * E + E, hi);
+    store_f_nt<T, E>(yp + 2 * j * E, lo);
+    store_f_nt<T, E>(yp + 2 * j * E + E, hi);
   }
 }
 
