@@ -9,21 +9,24 @@
 
 namespace tp {
 
-constexpr int RMS_MAX_PARTS = 2048;  // partial dw rows written by the backward (multiple of 4)
+constexpr int RMS_MAX_PARTS = 1024;  // partial dw rows written by the backward (multiple of 4)
 
 static inline int rms_parts(int64_t rows) {
   int64_t p = (rows + 3) / 4 * 4;
   return (int)(p < RMS_MAX_PARTS ? p : RMS_MAX_PARTS);
 }
 
-// sum over the WAVES waves that share a row (fixed order); `red` holds 4 floats per buffer
+// sum over the WAVES waves that share a row (fixed order); `red` holds one float per wave of the block
 template <int WAVES>
 __device__ __forceinline__ float row_sum(float v, float* red, int wave) {
   v = wave_sum(v);
   if (WAVES == 1) return v;
   if ((threadIdx.x & 63) == 0) red[wave] = v;
   __syncthreads();
-  return ((red[0] + red[1]) + red[2]) + red[3];
+  float s = red[0];
+#pragma unroll
+  for (int i = 1; i < WAVES; i++) s += red[i];
+  return s;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -47,13 +50,18 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_vec(const XT* __restrict__ x,
   const XT* xr = x + row * xs;
   OT* yr = y + row * ys;
 
+  // every load is issued before the first use: out-of-range vectors re-read the row's last one, so no
+  // branch sits between the loads and they all travel together
   float xv[NV][E];
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < NV; i++) {
     const int v = t + TPR * i;
-    if (v < nvec) {
-      load_f_nt<XT, E>(xr + (int64_t)v * E, xv[i]);
+    load_f_nt<XT, E>(xr + (int64_t)(v < nvec ? v : nvec - 1) * E, xv[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    if (t + TPR * i < nvec) {
 #pragma unroll
       for (int e = 0; e < E; e++) ss += xv[i][e] * xv[i][e];
     }
@@ -134,19 +142,24 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_vec(const OT* __restrict__ dy
     XT* dr = dx + row * dxs;
     float n[NV][E], g[NV][E];
     float c = 0.f;
+    // all loads first (out-of-range vectors re-read the row's last one), then the arithmetic
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       const int v = t + TPR * i;
-      if (v < nvec) {
-        float dyv[E];
-        load_f_nt<XT, E>(xr + (int64_t)v * E, n[i]);
-        load_f_nt<OT, E>(gr + (int64_t)v * E, dyv);
+      const int64_t o = (int64_t)(v < nvec ? v : nvec - 1) * E;
+      load_f_nt<XT, E>(xr + o, n[i]);
+      load_f_nt<OT, E>(gr + o, g[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      if (t + TPR * i < nvec) {
 #pragma unroll
         for (int e = 0; e < E; e++) {
+          const float dyv = g[i][e];
           n[i][e] *= r;
-          g[i][e] = dyv[e] * wv[i][e];
+          g[i][e] = dyv * wv[i][e];
           c += g[i][e] * n[i][e];
-          wacc[i][e] += dyv[e] * round_to<XT>(n[i][e]);
+          wacc[i][e] += dyv * round_to<XT>(n[i][e]);
         }
       }
     }
@@ -206,24 +219,25 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_dw_generic(const OT* __restri
   ws[(int64_t)blockIdx.y * hidden + c] = acc;
 }
 
-// dw[c] = sum_p ws[p, c], fixed order: 32 columns per block, 8 row groups folded through LDS
+// dw[c] = sum_p ws[p, c], fixed order: 16 columns per block, 16 row groups folded through LDS (the
+// partial rows were just written and mostly still sit in cache, so many small blocks beat few wide ones)
 template <typename WT>
 __global__ __launch_bounds__(256) void rmsnorm_dw_reduce(const float* __restrict__ ws, WT* __restrict__ dw, int parts,
                                                          int hidden) {
   __shared__ float red[256];
-  const int c = blockIdx.x * 32 + (threadIdx.x & 31);
-  const int g = threadIdx.x >> 5;
+  const int c = blockIdx.x * 16 + (threadIdx.x & 15);
+  const int g = threadIdx.x >> 4;
   float acc = 0.f;
   if (c < hidden) {
 #pragma unroll 8
-    for (int p = g; p < parts; p += 8) acc += ws[(int64_t)p * hidden + c];
+    for (int p = g; p < parts; p += 16) acc += ws[(int64_t)p * hidden + c];
   }
   red[threadIdx.x] = acc;
   __syncthreads();
   if (g == 0 && c < hidden) {
     float s = red[threadIdx.x];
 #pragma unroll
-    for (int k = 1; k < 8; k++) s += red[threadIdx.x + 32 * k];
+    for (int k = 1; k < 16; k++) s += red[threadIdx.x + 16 * k];
     dw[c] = Elem<WT>::from_f(s);
   }
 }
@@ -244,6 +258,8 @@ static int fwd_typed(const void* x, const void* w, void* y, float* rstd, int64_t
 #define TP_RMS_FWD(NV, WAVES)                                                                                  \
   rmsnorm_fwd_vec<XT, WT, OT, NV, WAVES><<<dim3((unsigned)((rows + 4 / WAVES - 1) / (4 / WAVES))), block, 0, st>>>( \
       xp, wp, yp, rstd, rows, hidden, xs, ys, eps)
+    // two vectors per thread over a whole block measured fastest at hidden 4096 (against one vector over
+    // 512 threads, or a wave per row)
     if (nvec <= 64) TP_RMS_FWD(1, 1);
     else if (nvec <= 128) TP_RMS_FWD(2, 1);
     else if (nvec <= 256) TP_RMS_FWD(1, 4);
@@ -285,7 +301,7 @@ static int bwd_typed(const void* dy, const void* x, const void* w, const float* 
     rmsnorm_bwd_dw_generic<XT, OT><<<dim3((hidden + 255) / 256, parts), dim3(256), 0, st>>>(gp, xp, rstd, ws, rows, hidden,
                                                                                           dys, xs);
   }
-  rmsnorm_dw_reduce<WT><<<dim3((hidden + 31) / 32), dim3(256), 0, st>>>(ws, (WT*)dw, parts, hidden);
+  rmsnorm_dw_reduce<WT><<<dim3((hidden + 15) / 16), dim3(256), 0, st>>>(ws, (WT*)dw, parts, hidden);
   return check_launch("tp_rmsnorm_bwd");
 }
 

@@ -10,6 +10,8 @@
 // The eager expression `(x * cos) + (rotate_half(x) * sin)` rounds each product and the sum to the
 // tensor dtype; the kernel reproduces those three roundings so bf16 results match it bit for bit.
 // The file is compiled with -ffp-contract=off so the fp32 path does not fuse mul+add either.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace tp {
@@ -32,12 +34,34 @@ __global__ __launch_bounds__(256) void rope_table_kernel(const float* __restrict
   sin_o[o + half] = Elem<T>::from_f(s);
 }
 
+// n / d for n < 2^31 with a multiplier computed on the host: q = mulhi(n, ceil(2^(31+l) / d)) >> (l - 1),
+// l = ceil(log2 d).  One quarter-rate multiply instead of the two dozen instructions of a runtime divide;
+// this kernel is close enough to the VALU limit for that to show.
+struct FastDiv {
+  unsigned d, m, sh;
+};
+static inline FastDiv fast_div(unsigned d) {
+  FastDiv f = {d, 0u, 0u};
+  if (d > 1) {
+    unsigned l = 0;
+    while ((1ull << l) < d) l++;
+    f.m = (unsigned)(((1ull << (31 + l)) + d - 1) / d);
+    f.sh = l - 1;
+  }
+  return f;
+}
+__device__ __forceinline__ unsigned div_by(unsigned n, const FastDiv& f) {
+  return f.d == 1 ? n : (__umulhi(n, f.m) >> f.sh);
+}
+
 struct RopeArgs {
   const void* x[2];
   void* y[2];
   int64_t xs[2][3];  // element strides (b, h, s)
   int64_t ys[2][3];
   int H[2];
+  unsigned nblk0;    // blocks that work on x[0]; the rest work on x[1]
+  FastDiv dH[2], dVH;
   const void* cos;
   const void* sin;
   const int64_t* pos;
@@ -45,45 +69,40 @@ struct RopeArgs {
   int B, S, D;
 };
 
-// One thread = one 16-byte vector of the first half and its partner in the second half
-// (E elements each), i.e. E rotation pairs.  Work item order: ((b*S + s) * Htot + h) * VH + j so a
-// wave sweeps the heads of one token, which are contiguous in (B,S,H,D) memory.
-template <typename T, bool INTERLEAVED, bool BACKWARD>
+// One thread = one 16-byte vector of the first half and its partner in the second half (E rotation
+// pairs).  A block works on one tensor (q or k) of one batch element (blockIdx.y); inside it the work
+// items are numbered (s * H + h) * VH + j so a wave sweeps the heads of one token, which are contiguous
+// in (B,S,H,D) memory.  Which tensor, the batch offset and all strides are wave-uniform, so they stay
+// on the scalar unit; WIDE = false keeps the per-lane offsets in 32 bits (every offset inside a batch
+// element below 2^31 elements, checked on the host).
+template <typename T, bool INTERLEAVED, bool BACKWARD, bool WIDE>
 __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
   constexpr int E = 16 / sizeof(T);
+  typedef typename std::conditional<WIDE, int64_t, unsigned>::type off_t;
   const int half = a.D / 2;
-  const int VH = half / E;  // vectors per half
-  const int Htot = a.H[0] + a.H[1];
-  const int64_t total = (int64_t)a.B * a.S * Htot * VH;
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= total) return;
-  int j, h, s, b;
-  if (total <= 0xffffffffll) {  // the usual case: 32-bit divisions are several times cheaper
-    const unsigned i32 = (unsigned)idx;
-    const unsigned t1 = i32 / (unsigned)VH;
-    j = (int)(i32 - t1 * (unsigned)VH);
-    const unsigned t2 = t1 / (unsigned)Htot;
-    h = (int)(t1 - t2 * (unsigned)Htot);
-    b = (int)(t2 / (unsigned)a.S);
-    s = (int)(t2 - (unsigned)b * (unsigned)a.S);
-  } else {
-    j = (int)(idx % VH);
-    int64_t t = idx / VH;
-    h = (int)(t % Htot);
-    t /= Htot;
-    s = (int)(t % a.S);
-    b = (int)(t / a.S);
-  }
-  const int which = h >= a.H[0] ? 1 : 0;
-  h -= which ? a.H[0] : 0;
+  const int which = blockIdx.x >= a.nblk0 ? 1 : 0;
+  const unsigned blk = blockIdx.x - (which ? a.nblk0 : 0u);
+  const int b = blockIdx.y;
+  const int H = a.H[which];
+  const unsigned lin = blk * 256u + threadIdx.x;
+  const unsigned u = div_by(lin, a.dVH);
+  const int j = (int)(lin - u * a.dVH.d);
+  const unsigned s = div_by(u, a.dH[which]);
+  const unsigned h = u - s * (unsigned)H;
+  if (s >= (unsigned)a.S) return;
 
-  const T* xp = (const T*)a.x[which] + b * a.xs[which][0] + h * a.xs[which][1] + s * a.xs[which][2];
-  T* yp = (T*)a.y[which] + b * a.ys[which][0] + h * a.ys[which][1] + s * a.ys[which][2];
-  int64_t crow;
-  if (a.pos) crow = a.cs_s * a.pos[b * a.pos_b + s];
-  else crow = a.cs_b * b + a.cs_s * s;
-  const T* cp = (const T*)a.cos + crow;
-  const T* sp = (const T*)a.sin + crow;
+  const T* xp = (const T*)a.x[which] + b * a.xs[which][0] + (off_t)h * (off_t)a.xs[which][1] + (off_t)s * (off_t)a.xs[which][2];
+  T* yp = (T*)a.y[which] + b * a.ys[which][0] + (off_t)h * (off_t)a.ys[which][1] + (off_t)s * (off_t)a.ys[which][2];
+  const T *cp, *sp;
+  if (a.pos) {
+    const int64_t crow = a.cs_s * a.pos[b * a.pos_b + s];
+    cp = (const T*)a.cos + crow;
+    sp = (const T*)a.sin + crow;
+  } else {
+    const off_t crow = (off_t)s * (off_t)a.cs_s;
+    cp = (const T*)a.cos + a.cs_b * b + crow;
+    sp = (const T*)a.sin + a.cs_b * b + crow;
+  }
 
   float c1[E], c2[E], s1[E], s2[E];
   load_f<T, E>(cp + j * E, c1);
@@ -139,16 +158,38 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
   }
 }
 
+template <typename T, bool WIDE>
+static void rope_launch(const RopeArgs& a, int interleaved, int backward, dim3 grid, hipStream_t st) {
+  const dim3 block(256);
+  if (!interleaved && !backward) rope_apply_kernel<T, false, false, WIDE><<<grid, block, 0, st>>>(a);
+  else if (!interleaved && backward) rope_apply_kernel<T, false, true, WIDE><<<grid, block, 0, st>>>(a);
+  else if (interleaved && !backward) rope_apply_kernel<T, true, false, WIDE><<<grid, block, 0, st>>>(a);
+  else rope_apply_kernel<T, true, true, WIDE><<<grid, block, 0, st>>>(a);
+}
+
 template <typename T>
-static int rope_typed(const RopeArgs& a, int interleaved, int backward, hipStream_t st) {
+static int rope_typed(RopeArgs& a, int interleaved, int backward, hipStream_t st) {
   constexpr int E = 16 / sizeof(T);
-  const int64_t total = (int64_t)a.B * a.S * (a.H[0] + a.H[1]) * (a.D / 2 / E);
-  if (total == 0) return TP_OK;
-  const dim3 grid((unsigned)((total + 255) / 256)), block(256);
-  if (!interleaved && !backward) rope_apply_kernel<T, false, false><<<grid, block, 0, st>>>(a);
-  else if (!interleaved && backward) rope_apply_kernel<T, false, true><<<grid, block, 0, st>>>(a);
-  else if (interleaved && !backward) rope_apply_kernel<T, true, false><<<grid, block, 0, st>>>(a);
-  else rope_apply_kernel<T, true, true><<<grid, block, 0, st>>>(a);
+  const int VH = a.D / 2 / E;
+  if (a.B == 0 || a.S == 0) return TP_OK;
+  const int64_t lim = 1ll << 31;
+  const int64_t items0 = (int64_t)a.S * a.H[0] * VH, items1 = (int64_t)a.S * a.H[1] * VH;
+  TP_REQUIRE(items0 < lim - 256 && items1 < lim - 256 && a.B <= 65535, TP_ERR_UNSUPPORTED,
+             "tp_rope_apply: more than 2^31 16-byte vectors per batch element, or batch > 65535");
+  const unsigned nb0 = (unsigned)((items0 + 255) / 256), nb1 = (unsigned)((items1 + 255) / 256);
+  a.nblk0 = nb0;
+  a.dVH = fast_div((unsigned)VH);
+  a.dH[0] = fast_div((unsigned)a.H[0]);
+  a.dH[1] = fast_div((unsigned)(a.H[1] > 0 ? a.H[1] : 1));
+  // 32-bit per-lane offsets when every offset inside one batch element stays below 2^31 elements
+  bool narrow = a.cs_s >= 0 && (int64_t)a.S * a.cs_s < lim;
+  for (int w = 0; w < 2; w++)
+    for (int i = 1; i < 3; i++) narrow = narrow && a.xs[w][i] >= 0 && a.ys[w][i] >= 0;
+  for (int w = 0; w < 2 && narrow; w++)
+    narrow = a.H[w] * a.xs[w][1] + a.S * a.xs[w][2] < lim && a.H[w] * a.ys[w][1] + a.S * a.ys[w][2] < lim;
+  const dim3 grid(nb0 + nb1, (unsigned)a.B);
+  if (narrow) rope_launch<T, false>(a, interleaved, backward, grid, st);
+  else rope_launch<T, true>(a, interleaved, backward, grid, st);
   return check_launch("tp_rope_apply");
 }
 
