@@ -26,6 +26,14 @@
 
 namespace tp {
 
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
 struct BwdArgs {
   const void* q;
   const void* k;
@@ -124,6 +132,76 @@ struct Stage64 {
   }
 };
 
+// ------------------------------------------------------------------------------------------------
+// row-major tiles filled by buffer loads that write LDS directly (no staging registers)
+// ------------------------------------------------------------------------------------------------
+// One such load moves 16 bytes per lane to LDS address  base + 16 * lane: where a chunk lands is fixed by
+// the lane, which global chunk it carries is free.  A tile of 64 rows x D 16-bit elements is stored
+// densely (row r at r * D*2) with the 16-byte chunks of a row XOR-swizzled by the row, so that the MFMA
+// fragment reads (lanes = consecutive rows, same logical chunk) fall into different banks.
+template <int D>
+struct DmaTile {
+  static constexpr int CPR = D / 8;              // 16-byte chunks per row
+  static constexpr int ROWB = D * 2;             // bytes per row
+  static constexpr int BYTES = 64 * ROWB;
+  static constexpr int PER_WAVE = CPR / 4;       // load instructions per wave for one tile (4 waves)
+  static_assert(CPR % 8 == 0, "head dim must be a multiple of 64");
+  static __device__ __forceinline__ int swz(int row) { return (CPR % 16 == 0) ? (row & 15) : ((row >> 1) & 7); }
+  // byte offset of logical chunk c of a row
+  static __device__ __forceinline__ int off(int row, int c) { return row * ROWB + ((c ^ swz(row)) << 4); }
+
+  unsigned vo[PER_WAVE];  // global byte offset (inside a tile) of the chunk this lane carries, per instruction
+
+  __device__ __forceinline__ void init(int64_t row_stride, int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; i++) {
+      const int slot = (wave * PER_WAVE + i) * 64 + lane;  // 16-byte slot inside the LDS tile
+      const int row = slot / CPR, c = (slot % CPR) ^ swz(row);
+      vo[i] = (unsigned)((row * row_stride + c * 8) * 2);
+    }
+  }
+  // Issue this wave's share of the tile.  The loads are written as assembly on purpose: the compiler
+  // orders every later LDS read behind an LDS-writing load it knows of, which would stall the tile being
+  // computed on the one in flight; the caller waits (s_waitcnt 0 + barrier) before the tile is read.
+  // Rows past the end of the tensor (offset >= rs.z) arrive as zeros.
+  __device__ __forceinline__ void issue(u32x4 rs, unsigned tile_byte_offset, unsigned char* lds_tile, int wave) const {
+    tile_byte_offset = __builtin_amdgcn_readfirstlane(tile_byte_offset);
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; i++) {
+      const unsigned dst = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lds_tile + (wave * PER_WAVE + i) * 1024));
+      asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                   :: "s"(dst), "v"(vo[i]), "s"(rs), "s"(tile_byte_offset) : "memory");
+    }
+  }
+};
+// buffer resource words for the assembly loads: base, stride 0, size in bytes, raw-buffer flags
+__device__ __forceinline__ u32x4 make_rsrc_words(const void* base, unsigned bytes) {
+  const unsigned long long p = (unsigned long long)base;
+  u32x4 r;
+  r.x = __builtin_amdgcn_readfirstlane((unsigned)p);
+  r.y = __builtin_amdgcn_readfirstlane((unsigned)(p >> 32));
+  r.z = __builtin_amdgcn_readfirstlane(bytes);
+  r.w = 0x00020000u;
+  return r;
+}
+// transposed copy of a DmaTile: every thread turns 4-row x 8-column blocks into 8-byte column pieces
+template <int D>
+__device__ __forceinline__ void transpose_tile(const unsigned char* src, unsigned char* dst, int tid) {
+  constexpr int CPR = D / 8, TOT = CPR * 16, ITEMS = (TOT + 255) / 256;
+#pragma unroll
+  for (int i = 0; i < ITEMS; i++) {
+    const int item = tid + 256 * i;
+    if (item < TOT) {
+      const int c8 = item % CPR, rq = item / CPR;
+      u32x4 r[4];
+#pragma unroll
+      for (int ii = 0; ii < 4; ii++) r[ii] = *(const u32x4*)(src + DmaTile<D>::off(4 * rq + ii, c8));
+#pragma unroll
+      for (int j = 0; j < 8; j++) *(u32x2*)(dst + TrTile64::quad_off(c8 * 8 + j, rq)) = transpose_col(r, j);
+    }
+  }
+}
+
 // per-tile [min,max] of segment ids for 64-row tiles t0..t1-1 into LDS (lane = row of the tile)
 __device__ __forceinline__ void seg_tile_ranges(const int32_t* segb, int S, int t0, int t1, int* tmin, int* tmax,
                                                 int wave, int lane) {
@@ -148,9 +226,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   constexpr int BNK = 128;  // kv rows per workgroup, 32 per wave
   constexpr int KS_QK = DQK / 16, KS_DV = DV / 16;
   constexpr int DKB = DQK / 32, DVB = DV / 32;
-  typedef RowTile<DQK> QT;
-  typedef RowTile<DV> OT;
-  constexpr int Q_BYTES = BMQ * QT::STRIDE, DO_BYTES = BMQ * OT::STRIDE;
+  typedef DmaTile<DQK> QT;
+  typedef DmaTile<DV> OT;
+  constexpr int Q_BYTES = QT::BYTES, DO_BYTES = OT::BYTES;
   constexpr int QTR_BYTES = DQK * TrTile64::ROW_BYTES, DOTR_BYTES = DV * TrTile64::ROW_BYTES;
   constexpr int ROW_BYTES = BMQ * 4 * 3;  // lse (log2 units), delta, segment id per query row
   constexpr int BUF_BYTES = Q_BYTES + DO_BYTES + QTR_BYTES + DOTR_BYTES + ROW_BYTES;
@@ -216,11 +294,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   }
   const int n_iter = nact * a.n_rep;
 
-  // ---- staging: Q / dO tiles by buffer loads (offsets inside a tile precomputed, tile offset scalar)
-  Stage64<DQK> qst;
-  Stage64<DV> dost;
-  qst.init(a.qs[2], tid);
-  dost.init(a.dos[2], tid);
+  // ---- staging: row-major Q / dO tiles by loads that write LDS directly; the transposed copies are made
+  // from LDS once a tile has landed; LSE, delta and segment id of the tile's rows go through registers
+  QT qdma;
+  OT dodma;
+  qdma.init(a.qs[2], wave, lane);
+  dodma.init(a.dos[2], wave, lane);
   const unsigned q_span = span_bytes(Sq, a.qs[2], DQK), do_span = span_bytes(Sq, a.dos[2], DV);
   const unsigned q_tile_bytes = (unsigned)(BMQ * a.qs[2] * 2), do_tile_bytes = (unsigned)(BMQ * a.dos[2] * 2);
   float lse_r = 0.f, delta_r = 0.f;
@@ -229,14 +308,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   int cur_hl = 0, cur_idx = 0;  // position of the tile being computed
   int nxt_hl = 0, nxt_idx = 0;  // position of the tile being prefetched
   auto qtile_of = [&](int idx) { return qt_first + (SEG ? active[idx] : idx); };
-  auto load_tile = [&](int hl, int idx) {
+  auto load_tile = [&](int hl, int idx, int buf) {
     const int hq = hk * a.n_rep + hl;
     const int qt = qtile_of(idx);
     const int qi0 = qt * BMQ;
-    const rsrc_t qrs = make_rsrc((const T*)a.q + b * a.qs[0] + hq * a.qs[1], q_span);
-    const rsrc_t dors = make_rsrc((const T*)a.dout + b * a.dos[0] + hq * a.dos[1], do_span);
-    qst.load(qrs, (unsigned)qt * q_tile_bytes, tid);
-    dost.load(dors, (unsigned)qt * do_tile_bytes, tid);
+    unsigned char* base = smem + buf * BUF_BYTES;
+    qdma.issue(make_rsrc_words((const T*)a.q + b * a.qs[0] + hq * a.qs[1], q_span), (unsigned)qt * q_tile_bytes, base, wave);
+    dodma.issue(make_rsrc_words((const T*)a.dout + b * a.dos[0] + hq * a.dos[1], do_span), (unsigned)qt * do_tile_bytes,
+                base + Q_BYTES, wave);
     if (tid < BMQ) {
       const int row = min(qi0 + tid, Sq - 1);
       const int64_t ro = ((int64_t)b * a.Hq + hq) * Sq + row;
@@ -246,12 +325,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       if (SEG) segq_r = segb[row];
     }
   };
-  auto store_tile = [&](int buf) {
+  // second half of the staging, after the tile's loads have landed (s_waitcnt 0 + barrier by the caller)
+  auto finish_tile = [&](int buf) {
     unsigned char* base = smem + buf * BUF_BYTES;
-    qst.store_rowmajor(base, tid);
-    dost.store_rowmajor(base + Q_BYTES, tid);
-    qst.store_transposed(base + Q_BYTES + DO_BYTES, tid);
-    dost.store_transposed(base + Q_BYTES + DO_BYTES + QTR_BYTES, tid);
+    transpose_tile<DQK>(base, base + Q_BYTES + DO_BYTES, tid);
+    transpose_tile<DV>(base + Q_BYTES, base + Q_BYTES + DO_BYTES + QTR_BYTES, tid);
     if (tid < BMQ) {
       float* rf = (float*)(base + Q_BYTES + DO_BYTES + QTR_BYTES + DOTR_BYTES);
       rf[tid] = lse_r;
@@ -259,6 +337,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       ((int*)rf)[2 * BMQ + tid] = segq_r;
     }
   };
+
+  // per-lane byte offsets of the MFMA fragments inside a tile (the swizzles are resolved once, here)
+  unsigned faq[KS_QK], fao[KS_DV], ta[4];
+#pragma unroll
+  for (int ks = 0; ks < KS_QK; ks++) faq[ks] = (unsigned)QT::off(ln, 2 * ks + g);
+#pragma unroll
+  for (int ks = 0; ks < KS_DV; ks++) fao[ks] = (unsigned)OT::off(ln, 2 * ks + g);
+#pragma unroll
+  for (int m = 0; m < 4; m++) ta[m] = (unsigned)TrTile64::chunk_off(ln, m, g);
 
   f32x16 dkacc[DKB], dvacc[DVB];
 #pragma unroll
@@ -271,13 +358,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     for (int v = 0; v < 16; v++) dvacc[d][v] = 0.f;
   const float c = a.scale_log2;
 
-  if (n_iter > 0) {
-    load_tile(0, 0);
-    store_tile(0);
-  }
-  // all earlier loads (the K/V fragments) have landed: keeps per-iteration MFMAs from waiting on the
-  // in-order vector-memory counter for that iteration's own prefetch
+  if (n_iter > 0) load_tile(0, 0, 0);
+  // all earlier loads (the K/V fragments, the first tile) have landed: also keeps per-iteration MFMAs
+  // from waiting on the in-order vector-memory counter for that iteration's own prefetch
   __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (n_iter > 0) finish_tile(0);
   __syncthreads();
 
   for (int it = 0; it < n_iter; it++) {
@@ -286,7 +372,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     nxt_idx = cur_idx + 1;
     nxt_hl = cur_hl;
     if (nxt_idx == nact) { nxt_idx = 0; nxt_hl++; }
-    if (it + 1 < n_iter) load_tile(nxt_hl, nxt_idx);
+    if (NBUF == 2 && it + 1 < n_iter) load_tile(nxt_hl, nxt_idx, buf ^ 1);
 
     const unsigned char* ql = smem + buf * BUF_BYTES;
     const unsigned char* dol = ql + Q_BYTES;
@@ -304,82 +390,112 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       skip = skip || hi < wkmin || lo > wkmax;
       need_mask = need_mask || !(lo == hi && wkmin == wkmax && lo == wkmin);
     }
-    // The two 32-row query blocks of the tile are staggered so that every group of MFMAs has
-    // independent VALU work next to it (source order = intended overlap):
-    //   S0 = Q0 K^T, dP0 = dO0 V^T               |
-    //   S1 = Q1 K^T, dP1 = dO1 V^T               | P0 = exp2(S0 c - lse), dS0 = P0 o (dP0 - delta)
-    //   dV^T += dO0^T P0, dK^T += Q0^T dS0       | P1, dS1
-    //   dV^T += dO1^T P1, dK^T += Q1^T dS1       | (transpose + LDS store of the next tile)
+    // The tile body is laid out by hand as a sequence of slots, one MFMA each, with a scheduling barrier
+    // after every slot: the LDS fragment a slot needs was requested AHEAD slots earlier, and the
+    // exponentials / products that turn S, dP into the 16-bit operands P, dS are spread two elements per
+    // slot under the MFMAs of the other query block.  (Left to itself the compiler reads each fragment
+    // right before its MFMA and the matrix unit waits out every LDS round trip.)
+    //   slots   A0: S0 = Q0 K^T   A1: S1 = Q1 K^T   B0: dP0 = dO0 V^T   B1: dP1 = dO1 V^T
+    //           C0, C1: dV^T += dO^T P   D0, D1: dK^T += Q^T dS
+    //   VALU    P0 under A1, P1 under B0, dS0 under B1, dS1 under C0
     auto body = [&](auto masked_c) {
       constexpr bool MASKED = decltype(masked_c)::value;
+      constexpr int A0 = 0, A1 = A0 + KS_QK, B0 = A1 + KS_QK, B1 = B0 + KS_DV, C0 = B1 + KS_DV, C1 = C0 + 2 * DVB,
+                    D0 = C1 + 2 * DVB, D1 = D0 + 2 * DKB, NS = D1 + 2 * DKB;
+      constexpr int AHEAD = 3, NF = 4;                        // fragment read-ahead, fragment ring size
+      constexpr int VP0 = A1, VP1 = B0, VS0 = B1, VS1 = C0;   // first slot of each 8-slot VALU group
+      static_assert(VP0 + 8 <= C0 && VP1 + 8 <= C1 && VS0 + 8 <= D0 && VS1 + 8 <= D1, "operands ready too late");
       const int kvcol = wkv0 + ln;
-      auto s_dp = [&](int qb, f32x16& sa, f32x16& dp) {
-#pragma unroll
-        for (int v = 0; v < 16; v++) { sa[v] = 0.f; dp[v] = 0.f; }
-#pragma unroll
-        for (int ks = 0; ks < KS_QK; ks++) {
-          const v8 f = *(const v8*)(ql + QT::off(qb * 32 + ln, 16 * ks + 8 * g));
-          sa = MT<T>::mfma32(f, kf[ks], sa);
-        }
-#pragma unroll
-        for (int ks = 0; ks < KS_DV; ks++) {
-          const v8 f = *(const v8*)(dol + OT::off(qb * 32 + ln, 16 * ks + 8 * g));
-          dp = MT<T>::mfma32(f, vf[ks], dp);
+      v8 fr[NF];
+      f32x16 s[2], dp[2];
+      v8 pf[2][2], df[2][2];
+      f32x4 rowv[4][2];  // per VALU group: LSE or delta of four query rows, requested two slots before use
+
+      auto frag = [&](auto I) -> v8 {
+        constexpr int i = decltype(I)::value;
+        if constexpr (i < A1) return *(const v8*)(ql + faq[i - A0]);
+        else if constexpr (i < B0) return *(const v8*)(ql + faq[i - A1] + 32 * QT::ROWB);
+        else if constexpr (i < B1) return *(const v8*)(dol + fao[i - B0]);
+        else if constexpr (i < C0) return *(const v8*)(dol + fao[i - B1] + 32 * OT::ROWB);
+        else if constexpr (i < D0) {
+          constexpr int qb = (i - C0) / (2 * DVB), j = (i - C0) % (2 * DVB), hh = j / DVB, d = j % DVB;
+          return *(const v8*)(dotl + ta[(2 * qb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+        } else {
+          constexpr int qb = (i - D0) / (2 * DKB), j = (i - D0) % (2 * DKB), hh = j / DKB, d = j % DKB;
+          return *(const v8*)(qtl + ta[(2 * qb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
         }
       };
-      // P and dS of one query block, converted to the B operands of the accumulating products
-      auto p_ds = [&](int qb, f32x16& sa, f32x16& dp, v8 (&pf)[2], v8 (&df)[2]) {
+      auto mma = [&](auto I, const v8& f) {
+        constexpr int i = decltype(I)::value;
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if constexpr (i < B0) {
+          constexpr int qb = (i - A0) / KS_QK, ks = (i - A0) % KS_QK;
+          s[qb] = MT<T>::mfma32(f, kf[ks], ks == 0 ? zero : s[qb]);
+        } else if constexpr (i < C0) {
+          constexpr int qb = (i - B0) / KS_DV, ks = (i - B0) % KS_DV;
+          dp[qb] = MT<T>::mfma32(f, vf[ks], ks == 0 ? zero : dp[qb]);
+        } else if constexpr (i < D0) {
+          constexpr int qb = (i - C0) / (2 * DVB), j = (i - C0) % (2 * DVB), hh = j / DVB, d = j % DVB;
+          dvacc[d] = MT<T>::mfma32(f, pf[qb][hh], dvacc[d]);
+        } else {
+          constexpr int qb = (i - D0) / (2 * DKB), j = (i - D0) % (2 * DKB), hh = j / DKB, d = j % DKB;
+          dkacc[d] = MT<T>::mfma32(f, df[qb][hh], dkacc[d]);
+        }
+      };
+      // VALU group of query block QB starting at slot START: two elements per slot for 8 slots.
+      // IS_P: s <- exp2(s c - lse) (masked), else dp <- s (dp - delta); the 16-bit operands are packed as
+      // soon as the eight values of a half are done.
+      auto valu = [&](auto I, auto START, auto QBc, auto IS_Pc) {
+        constexpr int i = decltype(I)::value, st = decltype(START)::value, qb = decltype(QBc)::value;
+        constexpr bool IS_P = decltype(IS_Pc)::value;
+        constexpr int GI = (IS_P ? 0 : 2) + qb;
+        // request the row values of quad vq two slots before its first element (slot st + 2 vq)
+        if constexpr (i + 2 >= st && i + 2 < st + 8 && (i + 2 - st) % 2 == 0) {
+          constexpr int vq = (i + 2 - st) / 2;
+          rowv[GI][vq & 1] = *(const f32x4*)((IS_P ? lsel : deltal) + qb * 32 + 8 * vq + 4 * g);
+        }
+        if constexpr (i >= st && i < st + 8) {
+          constexpr int k = i - st, vq = k / 2;
+          const f32x4 r4 = rowv[GI][vq & 1];
 #pragma unroll
-        for (int vq = 0; vq < 4; vq++) {
-          const int r0 = qb * 32 + 8 * vq + 4 * g;
-          const f32x4 l4 = *(const f32x4*)(lsel + r0);
-          const f32x4 d4 = *(const f32x4*)(deltal + r0);
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            const int v = 4 * vq + e;
-            float pv = fast_exp2(__builtin_fmaf(sa[v], c, -l4[e]));
-            if (MASKED) {
-              const int qrow = qi0 + r0 + e;
-              const bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || segl[r0 + e] == segk);
-              pv = ok ? pv : 0.f;
+          for (int e2 = 0; e2 < 2; e2++) {
+            const int e = 2 * (k % 2) + e2, v = 4 * vq + e;
+            if constexpr (IS_P) {
+              float pv = fast_exp2(__builtin_fmaf(s[qb][v], c, -r4[e]));
+              if (MASKED) {
+                const int r = qb * 32 + 8 * vq + 4 * g + e;
+                const int qrow = qi0 + r;
+                const bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || segl[r] == segk);
+                pv = ok ? pv : 0.f;
+              }
+              s[qb][v] = pv;
+            } else {
+              dp[qb][v] = s[qb][v] * (dp[qb][v] - r4[e]);
             }
-            sa[v] = pv;
-            dp[v] = pv * (dp[v] - d4[e]);
           }
-        }
-#pragma unroll
-        for (int hh = 0; hh < 2; hh++) {
-          pf[hh] = pack8<T>(sa[8 * hh + 0], sa[8 * hh + 1], sa[8 * hh + 2], sa[8 * hh + 3], sa[8 * hh + 4],
-                            sa[8 * hh + 5], sa[8 * hh + 6], sa[8 * hh + 7]);
-          df[hh] = pack8<T>(dp[8 * hh + 0], dp[8 * hh + 1], dp[8 * hh + 2], dp[8 * hh + 3], dp[8 * hh + 4],
-                            dp[8 * hh + 5], dp[8 * hh + 6], dp[8 * hh + 7]);
-        }
-      };
-      // dV^T += dO^T P, dK^T += Q^T dS over the 32 query rows of block qb (two k-steps of 16)
-      auto accumulate = [&](int qb, const v8 (&pf)[2], const v8 (&df)[2]) {
-#pragma unroll
-        for (int hh = 0; hh < 2; hh++) {
-          const int ks = 2 * qb + hh;
-#pragma unroll
-          for (int d = 0; d < DVB; d++) {
-            const v8 f = *(const v8*)(dotl + TrTile64::chunk_off(d * 32 + ln, ks, g));
-            dvacc[d] = MT<T>::mfma32(f, pf[hh], dvacc[d]);
-          }
-#pragma unroll
-          for (int d = 0; d < DKB; d++) {
-            const v8 f = *(const v8*)(qtl + TrTile64::chunk_off(d * 32 + ln, ks, g));
-            dkacc[d] = MT<T>::mfma32(f, df[hh], dkacc[d]);
+          if constexpr (k % 4 == 3) {
+            constexpr int hh = k / 4;
+            const f32x16& x = IS_P ? s[qb] : dp[qb];
+            const v8 packed = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4],
+                                       x[8 * hh + 5], x[8 * hh + 6], x[8 * hh + 7]);
+            if constexpr (IS_P) pf[qb][hh] = packed;
+            else df[qb][hh] = packed;
           }
         }
       };
-      f32x16 s0, dp0, s1, dp1;
-      v8 pf0[2], df0[2], pf1[2], df1[2];
-      s_dp(0, s0, dp0);
-      s_dp(1, s1, dp1);
-      p_ds(0, s0, dp0, pf0, df0);
-      accumulate(0, pf0, df0);
-      p_ds(1, s1, dp1, pf1, df1);
-      accumulate(1, pf1, df1);
+      typedef std::integral_constant<int, 0> I0;
+      typedef std::integral_constant<int, 1> I1;
+      static_for<0, AHEAD>([&](auto I) { fr[decltype(I)::value % NF] = frag(I); });
+      static_for<0, NS>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+        if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
+        mma(I, fr[i % NF]);
+        valu(I, std::integral_constant<int, VP0>{}, I0{}, std::true_type{});
+        valu(I, std::integral_constant<int, VP1>{}, I1{}, std::true_type{});
+        valu(I, std::integral_constant<int, VS0>{}, I0{}, std::false_type{});
+        valu(I, std::integral_constant<int, VS1>{}, I1{}, std::false_type{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
     };
     if constexpr (DQK <= 128) {
       if (!skip) {
@@ -401,7 +517,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         for (int ks = 0; ks < KS_QK; ks++)
   #pragma unroll
           for (int qb = 0; qb < QB; qb++) {
-            const v8 qf = *(const v8*)(ql + QT::off(qb * 32 + ln, 16 * ks + 8 * g));
+            const v8 qf = *(const v8*)(ql + QT::off(qb * 32 + ln, 2 * ks + g));
             sacc[qb] = MT<T>::mfma32(qf, kf[ks], sacc[qb]);
           }
         // dP = dO V^T
@@ -409,7 +525,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         for (int ks = 0; ks < KS_DV; ks++)
   #pragma unroll
           for (int qb = 0; qb < QB; qb++) {
-            const v8 dof = *(const v8*)(dol + OT::off(qb * 32 + ln, 16 * ks + 8 * g));
+            const v8 dof = *(const v8*)(dol + OT::off(qb * 32 + ln, 2 * ks + g));
             dpacc[qb] = MT<T>::mfma32(dof, vf[ks], dpacc[qb]);
           }
         // P = exp2(S*c - lse), dS = P o (dP - delta); rows of the C tile are queries
@@ -468,8 +584,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         }
       }
     }
-    if (NBUF == 1) __syncthreads();
-    if (it + 1 < n_iter) store_tile(NBUF == 2 ? (buf ^ 1) : 0);
+    if (it + 1 < n_iter) {
+      if (NBUF == 1) {  // single buffer: the next tile can only be requested once this one has been used
+        __syncthreads();
+        load_tile(nxt_hl, nxt_idx, 0);
+      }
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();  // the next tile's row-major copies are complete, everyone is done with this tile
+      finish_tile(NBUF == 2 ? (buf ^ 1) : 0);
+    }
     __syncthreads();
     cur_idx = nxt_idx;
     cur_hl = nxt_hl;
@@ -750,7 +873,7 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
   // dK, dV
   {
     constexpr int BMQ = 64, BNK = 128;
-    constexpr int BUF = BMQ * RowTile<DQK>::STRIDE + BMQ * RowTile<DV>::STRIDE + (DQK + DV) * TrTile64::ROW_BYTES + BMQ * 12;
+    constexpr int BUF = DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES + (DQK + DV) * TrTile64::ROW_BYTES + BMQ * 12;
     constexpr int NBUF = (2 * BUF + 4096 <= 160 * 1024) ? 2 : 1;
     const int nqt = (a.Sq + BMQ - 1) / BMQ;
     const size_t smem = (size_t)NBUF * BUF + (SEG ? (size_t)(3 * nqt + 8) * 4 : 0);
