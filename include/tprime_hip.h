@@ -123,7 +123,8 @@ int tp_attn_fwd(const void* q, const void* k, const void* v, const int32_t* seg,
                 const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
                 const int64_t o_strides[3], float sm_scale, int causal, int dtype, void* stream);
 
-/* Bytes of fp32 workspace tp_attn_bwd needs. */
+/* Bytes of fp32 workspace tp_attn_bwd needs (two floats per query row: rowsum(dO o O) and the LSE in
+ * log2 units). */
 size_t tp_attn_bwd_workspace_bytes(int B, int Hq, int Sq);
 
 /* Attention backward (the reference gets it from autograd through attention.py:151-170, or from

@@ -75,7 +75,13 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
   for (int e = 0; e < 8; e++) acc += o[e] * g[e];
 #pragma unroll
   for (int off = TPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-  if (valid && ch == 0) a.delta[rowid] = acc;
+  if (valid && ch == 0) {
+    a.delta[rowid] = acc;
+    // second half of the workspace: LSE in log2 units for the dK/dV kernel; a row with no allowed key
+    // (LSE = -inf) gets +inf so that its P = exp2(s - inf) = 0
+    const float l = a.lse[rowid];
+    a.delta[total + rowid] = (l == -INFINITY) ? INFINITY : l * LOG2E;
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -196,11 +202,70 @@ __device__ __forceinline__ void transpose_tile(const unsigned char* src, unsigne
       u32x4 r[4];
 #pragma unroll
       for (int ii = 0; ii < 4; ii++) r[ii] = *(const u32x4*)(src + DmaTile<D>::off(4 * rq + ii, c8));
+      // odd column blocks take their columns in the order 1,0,3,2,...: at every step half the lanes write
+      // even LDS rows and half odd ones, which spreads the 8-byte stores over all banks
+      const int flip = c8 & 1;
+      const unsigned sel_even = flip ? 0x07060302u : 0x05040100u, sel_odd = flip ? 0x05040100u : 0x07060302u;
 #pragma unroll
-      for (int j = 0; j < 8; j++) *(u32x2*)(dst + TrTile64::quad_off(c8 * 8 + j, rq)) = transpose_col(r, j);
+      for (int j = 0; j < 8; j++) {
+        const unsigned sel = (j & 1) ? sel_odd : sel_even;
+        const int w = j >> 1;
+        u32x2 o;
+        o.x = __builtin_amdgcn_perm(r[1][w], r[0][w], sel);
+        o.y = __builtin_amdgcn_perm(r[3][w], r[2][w], sel);
+        *(u32x2*)(dst + TrTile64::quad_off(c8 * 8 + (j ^ flip), rq)) = o;
+      }
     }
   }
 }
+
+// 4 bytes per lane straight into LDS at dst + 4 * lane (a 64-entry row vector per instruction)
+__device__ __forceinline__ void dma_dword(u32x4 rs, unsigned byte_offset, unsigned char* dst, int lane) {
+  const unsigned d = __builtin_amdgcn_readfirstlane((unsigned)(size_t)dst);
+  byte_offset = __builtin_amdgcn_readfirstlane(byte_offset);
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+               :: "s"(d), "v"((unsigned)lane * 4u), "s"(rs), "s"(byte_offset) : "memory");
+}
+// The same transposition as transpose_tile, cut into steps that can be placed between MFMAs: read() fetches
+// this thread's 4-row x 8-column block, write(J) stores column pair member J (0..7) as 8 bytes.  Threads
+// are assigned to blocks so that the 32 lanes served together write 32 different bank pairs; threads beyond
+// the number of blocks repeat the work of an earlier one (same values to the same addresses).
+template <int D>
+struct TransposeSteps {
+  static constexpr int CPR = D / 8, TOT = CPR * 16;
+  static_assert(TOT <= 256, "one block per thread");
+  u32x4 r[4];
+  unsigned rd, zs, wbase, y, sel_even, sel_odd;
+  __device__ __forceinline__ void init(int tid) {
+    const int item = tid % TOT, c8 = item % CPR, rqi = item / CPR;
+    const int rq = (rqi & ~3) | ((rqi & 1) << 1) | ((rqi >> 1) & 1);
+    rd = (unsigned)(4 * rq * DmaTile<D>::ROWB);
+    zs = (unsigned)((c8 ^ DmaTile<D>::swz(4 * rq)) << 4);
+    const int flip = c8 & 1;
+    const int k = (((c8 & 1) << 2) ^ (c8 >> 1)) & 7, rqc = 2 * (rq >> 2) + (rq & 1);
+    wbase = (unsigned)(c8 * 8 * TrTile64::ROW_BYTES + (((rq >> 1) & 1) << 3));
+    y = (unsigned)((flip << 7) | ((rqc ^ k) << 4));
+    sel_even = flip ? 0x07060302u : 0x05040100u;
+    sel_odd = flip ? 0x05040100u : 0x07060302u;
+  }
+  __device__ __forceinline__ void read(const unsigned char* src) {
+#pragma unroll
+    for (int ii = 0; ii < 4; ii++) {
+      const unsigned sw = (unsigned)((CPR % 16 == 0 ? ii : (ii >> 1)) << 4);
+      r[ii] = *(const u32x4*)(src + rd + (zs ^ sw) + ii * DmaTile<D>::ROWB);
+    }
+  }
+  template <typename J>
+  __device__ __forceinline__ void write(unsigned char* dst, J) const {
+    constexpr int j = J::value, w = j >> 1;
+    constexpr unsigned cj = (unsigned)(((j & 1) << 7) | ((j >> 1) << 4));
+    const unsigned sel = (j & 1) ? sel_odd : sel_even;
+    u32x2 o;
+    o.x = __builtin_amdgcn_perm(r[1][w], r[0][w], sel);
+    o.y = __builtin_amdgcn_perm(r[3][w], r[2][w], sel);
+    *(u32x2*)(dst + wbase + (y ^ cj) + (j >> 1) * 2 * TrTile64::ROW_BYTES) = o;
+  }
+};
 
 // per-tile [min,max] of segment ids for 64-row tiles t0..t1-1 into LDS (lane = row of the tile)
 __device__ __forceinline__ void seg_tile_ranges(const int32_t* segb, int S, int t0, int t1, int* tmin, int* tmax,
@@ -230,8 +295,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   typedef DmaTile<DV> OT;
   constexpr int Q_BYTES = QT::BYTES, DO_BYTES = OT::BYTES;
   constexpr int QTR_BYTES = DQK * TrTile64::ROW_BYTES, DOTR_BYTES = DV * TrTile64::ROW_BYTES;
-  constexpr int ROW_BYTES = BMQ * 4 * 3;  // lse (log2 units), delta, segment id per query row
-  constexpr int BUF_BYTES = Q_BYTES + DO_BYTES + QTR_BYTES + DOTR_BYTES + ROW_BYTES;
+  constexpr int ROW_BYTES = BMQ * 4 * 3;  // lse (log2 units), delta, segment id per query row: 3 slots
+  constexpr int BUF_BYTES = Q_BYTES + DO_BYTES + QTR_BYTES + DOTR_BYTES;
+  constexpr bool PIPE = NBUF == 2 && DQK <= 128 && DV <= 128;
 
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -261,7 +327,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   const int nqt_all = (Sq + BMQ - 1) / BMQ;
   const int qt_first = CAUSAL ? min(kv0 / BMQ, nqt_all) : 0;
   const int nqt = nqt_all - qt_first;
-  int* qmin = (int*)(smem + NBUF * BUF_BYTES);
+  int* qmin = (int*)(smem + NBUF * BUF_BYTES + 3 * ROW_BYTES);
   int* qmax = qmin + nqt;
   int* active = qmax + nqt;
   int* bk = active + nqt;  // 8 ints: per-wave (min,max) of kv ids
@@ -294,48 +360,29 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   }
   const int n_iter = nact * a.n_rep;
 
-  // ---- staging: row-major Q / dO tiles by loads that write LDS directly; the transposed copies are made
-  // from LDS once a tile has landed; LSE, delta and segment id of the tile's rows go through registers
+  // ---- staging: every piece of a query tile (Q, dO row-major; log2-scaled LSE, delta, segment ids of its
+  // rows) is written into LDS by the loads themselves; the transposed copies are made LDS-to-LDS
   QT qdma;
   OT dodma;
   qdma.init(a.qs[2], wave, lane);
   dodma.init(a.dos[2], wave, lane);
   const unsigned q_span = span_bytes(Sq, a.qs[2], DQK), do_span = span_bytes(Sq, a.dos[2], DV);
   const unsigned q_tile_bytes = (unsigned)(BMQ * a.qs[2] * 2), do_tile_bytes = (unsigned)(BMQ * a.dos[2] * 2);
-  float lse_r = 0.f, delta_r = 0.f;
-  int segq_r = 0;
-  // iteration -> (query head of the group, query tile): heads outer, tiles inner, no division in the loop
-  int cur_hl = 0, cur_idx = 0;  // position of the tile being computed
-  int nxt_hl = 0, nxt_idx = 0;  // position of the tile being prefetched
+  const float* lse2 = a.delta + (int64_t)a.B * a.Hq * Sq;  // second half of the workspace (delta kernel)
+  unsigned char* const rows_base = smem + NBUF * BUF_BYTES;
   auto qtile_of = [&](int idx) { return qt_first + (SEG ? active[idx] : idx); };
-  auto load_tile = [&](int hl, int idx, int buf) {
+  auto issue_tile = [&](int hl, int idx, int buf, int rslot) {
     const int hq = hk * a.n_rep + hl;
     const int qt = qtile_of(idx);
-    const int qi0 = qt * BMQ;
     unsigned char* base = smem + buf * BUF_BYTES;
     qdma.issue(make_rsrc_words((const T*)a.q + b * a.qs[0] + hq * a.qs[1], q_span), (unsigned)qt * q_tile_bytes, base, wave);
     dodma.issue(make_rsrc_words((const T*)a.dout + b * a.dos[0] + hq * a.dos[1], do_span), (unsigned)qt * do_tile_bytes,
                 base + Q_BYTES, wave);
-    if (tid < BMQ) {
-      const int row = min(qi0 + tid, Sq - 1);
-      const int64_t ro = ((int64_t)b * a.Hq + hq) * Sq + row;
-      const float l = a.lse[ro];
-      lse_r = (l == -INFINITY) ? INFINITY : l * LOG2E;  // a row with no allowed key gets P = 0
-      delta_r = a.delta[ro];
-      if (SEG) segq_r = segb[row];
-    }
-  };
-  // second half of the staging, after the tile's loads have landed (s_waitcnt 0 + barrier by the caller)
-  auto finish_tile = [&](int buf) {
-    unsigned char* base = smem + buf * BUF_BYTES;
-    transpose_tile<DQK>(base, base + Q_BYTES + DO_BYTES, tid);
-    transpose_tile<DV>(base + Q_BYTES, base + Q_BYTES + DO_BYTES + QTR_BYTES, tid);
-    if (tid < BMQ) {
-      float* rf = (float*)(base + Q_BYTES + DO_BYTES + QTR_BYTES + DOTR_BYTES);
-      rf[tid] = lse_r;
-      rf[BMQ + tid] = delta_r;
-      ((int*)rf)[2 * BMQ + tid] = segq_r;
-    }
+    // waves 0..2 fetch one 64-entry row vector each: 4 bytes per lane, rows past Sq arrive as zeros
+    const int64_t ro = ((int64_t)b * a.Hq + hq) * Sq;
+    const void* src = wave == 0 ? (const void*)(lse2 + ro) : wave == 1 ? (const void*)(a.delta + ro) : (const void*)segb;
+    if (wave < 2 || (SEG && wave == 2))
+      dma_dword(make_rsrc_words(src, (unsigned)Sq * 4u), (unsigned)(qt * BMQ) * 4u, rows_base + rslot * ROW_BYTES + wave * BMQ * 4, lane);
   };
 
   // per-lane byte offsets of the MFMA fragments inside a tile (the swizzles are resolved once, here)
@@ -358,191 +405,280 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     for (int v = 0; v < 16; v++) dvacc[d][v] = 0.f;
   const float c = a.scale_log2;
 
-  if (n_iter > 0) load_tile(0, 0, 0);
-  // all earlier loads (the K/V fragments, the first tile) have landed: also keeps per-iteration MFMAs
-  // from waiting on the in-order vector-memory counter for that iteration's own prefetch
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
-  if (n_iter > 0) finish_tile(0);
-  __syncthreads();
-
-  for (int it = 0; it < n_iter; it++) {
-    const int buf = NBUF == 2 ? (it & 1) : 0;
-    const int qi0 = qtile_of(cur_idx) * BMQ;
-    nxt_idx = cur_idx + 1;
-    nxt_hl = cur_hl;
-    if (nxt_idx == nact) { nxt_idx = 0; nxt_hl++; }
-    if (NBUF == 2 && it + 1 < n_iter) load_tile(nxt_hl, nxt_idx, buf ^ 1);
-
-    const unsigned char* ql = smem + buf * BUF_BYTES;
-    const unsigned char* dol = ql + Q_BYTES;
-    const unsigned char* qtl = dol + DO_BYTES;
-    const unsigned char* dotl = qtl + QTR_BYTES;
-    const float* lsel = (const float*)(dotl + DOTR_BYTES);
-    const float* deltal = lsel + BMQ;
-    const int* segl = (const int*)(deltal + BMQ);
-
-    // wave-level decisions (uniform): nothing to do if every query row precedes every kv row
+  // wave-level decisions for a query tile (uniform): skip if every query row precedes every kv row
+  auto tile_mode = [&](int idx, int qi0) {  // 0 = nothing to compute, 1 = no masking needed, 2 = masked
     bool skip = (CAUSAL && qi0 + BMQ - 1 < wkv0) || wkv0 >= Skv;
     bool need_mask = (qi0 + BMQ > Sq) || (wkv0 + 32 > Skv) || (CAUSAL && qi0 < wkv0 + 31);
     if (SEG) {
-      const int lo = qmin[active[cur_idx]], hi = qmax[active[cur_idx]];
+      const int lo = qmin[active[idx]], hi = qmax[active[idx]];
       skip = skip || hi < wkmin || lo > wkmax;
       need_mask = need_mask || !(lo == hi && wkmin == wkmax && lo == wkmin);
     }
-    // The tile body is laid out by hand as a sequence of slots, one MFMA each, with a scheduling barrier
-    // after every slot: the LDS fragment a slot needs was requested AHEAD slots earlier, and the
-    // exponentials / products that turn S, dP into the 16-bit operands P, dS are spread two elements per
-    // slot under the MFMAs of the other query block.  (Left to itself the compiler reads each fragment
-    // right before its MFMA and the matrix unit waits out every LDS round trip.)
-    //   slots   A0: S0 = Q0 K^T   A1: S1 = Q1 K^T   B0: dP0 = dO0 V^T   B1: dP1 = dO1 V^T
-    //           C0, C1: dV^T += dO^T P   D0, D1: dK^T += Q^T dS
-    //   VALU    P0 under A1, P1 under B0, dS0 under B1, dS1 under C0
-    auto body = [&](auto masked_c) {
-      constexpr bool MASKED = decltype(masked_c)::value;
-      constexpr int A0 = 0, A1 = A0 + KS_QK, B0 = A1 + KS_QK, B1 = B0 + KS_DV, C0 = B1 + KS_DV, C1 = C0 + 2 * DVB,
-                    D0 = C1 + 2 * DVB, D1 = D0 + 2 * DKB, NS = D1 + 2 * DKB;
-      constexpr int AHEAD = 3, NF = 4;                        // fragment read-ahead, fragment ring size
-      constexpr int VP0 = A1, VP1 = B0, VS0 = B1, VS1 = C0;   // first slot of each 8-slot VALU group
-      static_assert(VP0 + 8 <= C0 && VP1 + 8 <= C1 && VS0 + 8 <= D0 && VS1 + 8 <= D1, "operands ready too late");
-      const int kvcol = wkv0 + ln;
-      v8 fr[NF];
-      f32x16 s[2], dp[2];
-      v8 pf[2][2], df[2][2];
-      f32x4 rowv[4][2];  // per VALU group: LSE or delta of four query rows, requested two slots before use
+    return skip ? 0 : (need_mask ? 2 : 1);
+  };
+  // iteration -> (query head of the group, query tile): heads outer, tiles inner, no division in the loop
+  auto advance = [&](int& hl, int& idx) {
+    if (++idx == nact) { idx = 0; hl++; }
+  };
 
-      auto frag = [&](auto I) -> v8 {
-        constexpr int i = decltype(I)::value;
-        if constexpr (i < A1) return *(const v8*)(ql + faq[i - A0]);
-        else if constexpr (i < B0) return *(const v8*)(ql + faq[i - A1] + 32 * QT::ROWB);
-        else if constexpr (i < B1) return *(const v8*)(dol + fao[i - B0]);
-        else if constexpr (i < C0) return *(const v8*)(dol + fao[i - B1] + 32 * OT::ROWB);
-        else if constexpr (i < D0) {
-          constexpr int qb = (i - C0) / (2 * DVB), j = (i - C0) % (2 * DVB), hh = j / DVB, d = j % DVB;
-          return *(const v8*)(dotl + ta[(2 * qb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
-        } else {
-          constexpr int qb = (i - D0) / (2 * DKB), j = (i - D0) % (2 * DKB), hh = j / DKB, d = j % DKB;
-          return *(const v8*)(qtl + ta[(2 * qb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
-        }
-      };
-      auto mma = [&](auto I, const v8& f) {
-        constexpr int i = decltype(I)::value;
-        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        if constexpr (i < B0) {
-          constexpr int qb = (i - A0) / KS_QK, ks = (i - A0) % KS_QK;
-          s[qb] = MT<T>::mfma32(f, kf[ks], ks == 0 ? zero : s[qb]);
-        } else if constexpr (i < C0) {
-          constexpr int qb = (i - B0) / KS_DV, ks = (i - B0) % KS_DV;
-          dp[qb] = MT<T>::mfma32(f, vf[ks], ks == 0 ? zero : dp[qb]);
-        } else if constexpr (i < D0) {
-          constexpr int qb = (i - C0) / (2 * DVB), j = (i - C0) % (2 * DVB), hh = j / DVB, d = j % DVB;
-          dvacc[d] = MT<T>::mfma32(f, pf[qb][hh], dvacc[d]);
-        } else {
-          constexpr int qb = (i - D0) / (2 * DKB), j = (i - D0) % (2 * DKB), hh = j / DKB, d = j % DKB;
-          dkacc[d] = MT<T>::mfma32(f, df[qb][hh], dkacc[d]);
-        }
-      };
-      // VALU group of query block QB starting at slot START: two elements per slot for 8 slots.
-      // IS_P: s <- exp2(s c - lse) (masked), else dp <- s (dp - delta); the 16-bit operands are packed as
-      // soon as the eight values of a half are done.
-      auto valu = [&](auto I, auto START, auto QBc, auto IS_Pc) {
-        constexpr int i = decltype(I)::value, st = decltype(START)::value, qb = decltype(QBc)::value;
-        constexpr bool IS_P = decltype(IS_Pc)::value;
-        constexpr int GI = (IS_P ? 0 : 2) + qb;
-        // request the row values of quad vq two slots before its first element (slot st + 2 vq)
-        if constexpr (i + 2 >= st && i + 2 < st + 8 && (i + 2 - st) % 2 == 0) {
-          constexpr int vq = (i + 2 - st) / 2;
-          rowv[GI][vq & 1] = *(const f32x4*)((IS_P ? lsel : deltal) + qb * 32 + 8 * vq + 4 * g);
-        }
-        if constexpr (i >= st && i < st + 8) {
-          constexpr int k = i - st, vq = k / 2;
-          const f32x4 r4 = rowv[GI][vq & 1];
+  if constexpr (PIPE) {
+    // Software pipeline over query tiles t, two full buffers (row-major + transposed) and three row-vector
+    // slots.  Tile t+1's loads are issued in the middle of tile t-1 and have a whole tile body to land;
+    // its transposed copies are made under the second half of tile t's MFMAs:
+    //   part 1 (S, dP: row-major tiles of buffer t&1)
+    //   wait for this wave's share of tile t+1, barrier      -> buffer t&1's row-major tiles are free,
+    //   issue the loads of tile t+2 into them                   tile t+1 has landed for everybody
+    //   part 2 (dV, dK: transposed tiles of buffer t&1), interleaved with transposing tile t+1
+    //   barrier
+    int c_hl = 0, c_idx = 0, n_hl = 0, n_idx = 0;  // tile being computed, tile whose loads are issued next
+    TransposeSteps<DQK> trq;
+    TransposeSteps<DV> tro;
+    trq.init(tid);
+    tro.init(tid);
+    if (n_iter > 0) { issue_tile(n_hl, n_idx, 0, 0); advance(n_hl, n_idx); }
+    if (n_iter > 1) { issue_tile(n_hl, n_idx, 1, 1); advance(n_hl, n_idx); }
+    // all earlier loads (the K/V fragments, the first tiles) have landed
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (n_iter > 0) {
+      trq.read(smem);
+      tro.read(smem + Q_BYTES);
+      static_for<0, 8>([&](auto J) {
+        trq.write(smem + Q_BYTES + DO_BYTES, J);
+        tro.write(smem + Q_BYTES + DO_BYTES + QTR_BYTES, J);
+      });
+    }
+    __syncthreads();
+
+    int rslot = 0;
+    for (int it = 0; it < n_iter; it++) {
+      const int buf = it & 1;
+      const int qi0 = qtile_of(c_idx) * BMQ;
+      const int mode = tile_mode(c_idx, qi0);
+      const bool issue_next = it + 2 < n_iter;
+      unsigned char* const bl = smem + buf * BUF_BYTES;
+      unsigned char* const bn = smem + (buf ^ 1) * BUF_BYTES;
+      const unsigned char* ql = bl;
+      const unsigned char* dol = ql + Q_BYTES;
+      const unsigned char* qtl = dol + DO_BYTES;
+      const unsigned char* dotl = qtl + QTR_BYTES;
+      const float* lsel = (const float*)(rows_base + rslot * ROW_BYTES);
+      const float* deltal = lsel + BMQ;
+      const int* segl = (const int*)(deltal + BMQ);
+      const int rnext = rslot >= 1 ? rslot - 1 : 2;  // (it + 2) % 3, the slot tile t-1 used
+
+      // The tile body is laid out by hand as a sequence of slots, one MFMA each, with a scheduling barrier
+      // after every slot: the LDS fragment a slot needs was requested AHEAD slots earlier, and the
+      // exponentials / products that turn S, dP into the 16-bit operands P, dS are spread over the slots
+      // under the MFMAs of the other query block.  (Left to itself the compiler reads each fragment right
+      // before its MFMA and the matrix unit waits out every LDS round trip.)
+      //   slots   A0: S0 = Q0 K^T   A1: S1 = Q1 K^T   B0: dP0 = dO0 V^T   B1: dP1 = dO1 V^T
+      //           C0, C1: dV^T += dO^T P   D0, D1: dK^T += Q^T dS
+      //   VALU    P0 ends before C0, P1 before C1, dS0 before D0, dS1 before D1
+      auto body = [&](auto mode_c) {
+        constexpr int MODE = decltype(mode_c)::value;
+        constexpr bool COMPUTE = MODE != 0, MASKED = MODE == 2;
+        constexpr int A0 = 0, A1 = A0 + KS_QK, B0 = A1 + KS_QK, B1 = B0 + KS_DV, C0 = B1 + KS_DV, C1 = C0 + 2 * DVB,
+                      D0 = C1 + 2 * DVB, D1 = D0 + 2 * DKB, NS = D1 + 2 * DKB;
+        constexpr int AHEAD = 3, NF = 4;  // fragment read-ahead, fragment ring size
+        // VALU groups: one element per slot where the tile body is long enough, each group ending right
+        // before the MFMAs that consume its packed operand
+        constexpr int EPS = (C0 - 16 >= A1) ? 1 : 2, VL = 16 / EPS;
+        constexpr int VP0 = C0 - VL, VP1 = C1 - VL, VS0 = D0 - VL, VS1 = D1 - VL;
+        static_assert(VP0 >= A1 && VP1 >= B0 && VS0 >= B1 && VS1 >= C0 && VS0 > VP0 && VS1 > VP1, "operands not ready");
+        // transposing the next tile: reads of a tile in one slot, then WPS column pairs per slot
+        constexpr int WPS = (NS - C0 >= 24) ? 1 : 2, TQ0 = C0, TO0 = TQ0 + 2 + 8 / WPS;
+        static_assert(TO0 + 2 + 8 / WPS <= NS, "second half too short for the transposition");
+        const int kvcol = wkv0 + ln;
+        v8 fr[NF];
+        f32x16 s[2], dp[2];
+        v8 pf[2][2], df[2][2];
+        f32x4 rowv[4][2];  // per VALU group: LSE or delta of four query rows, requested two slots before use
+
+        auto frag = [&](auto I) -> v8 {
+          constexpr int i = decltype(I)::value;
+          if constexpr (i < A1) return *(const v8*)(ql + faq[i - A0]);
+          else if constexpr (i < B0) return *(const v8*)(ql + faq[i - A1] + 32 * QT::ROWB);
+          else if constexpr (i < B1) return *(const v8*)(dol + fao[i - B0]);
+          else if constexpr (i < C0) return *(const v8*)(dol + fao[i - B1] + 32 * OT::ROWB);
+          else if constexpr (i < D0) {
+            constexpr int qb = (i - C0) / (2 * DVB), j = (i - C0) % (2 * DVB), hh = j / DVB, d = j % DVB;
+            return *(const v8*)(dotl + ta[(2 * qb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+          } else {
+            constexpr int qb = (i - D0) / (2 * DKB), j = (i - D0) % (2 * DKB), hh = j / DKB, d = j % DKB;
+            return *(const v8*)(qtl + ta[(2 * qb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+          }
+        };
+        auto mma = [&](auto I, const v8& f) {
+          constexpr int i = decltype(I)::value;
+          const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          if constexpr (i < B0) {
+            constexpr int qb = (i - A0) / KS_QK, ks = (i - A0) % KS_QK;
+            s[qb] = MT<T>::mfma32(f, kf[ks], ks == 0 ? zero : s[qb]);
+          } else if constexpr (i < C0) {
+            constexpr int qb = (i - B0) / KS_DV, ks = (i - B0) % KS_DV;
+            dp[qb] = MT<T>::mfma32(f, vf[ks], ks == 0 ? zero : dp[qb]);
+          } else if constexpr (i < D0) {
+            constexpr int qb = (i - C0) / (2 * DVB), j = (i - C0) % (2 * DVB), hh = j / DVB, d = j % DVB;
+            dvacc[d] = MT<T>::mfma32(f, pf[qb][hh], dvacc[d]);
+          } else {
+            constexpr int qb = (i - D0) / (2 * DKB), j = (i - D0) % (2 * DKB), hh = j / DKB, d = j % DKB;
+            dkacc[d] = MT<T>::mfma32(f, df[qb][hh], dkacc[d]);
+          }
+        };
+        // VALU group of query block QB starting at slot START: EPS elements per slot for VL slots.
+        // IS_P: s <- exp2(s c - lse) (masked), else dp <- s (dp - delta); the 16-bit operands are packed as
+        // soon as the eight values of a half are done.
+        auto valu = [&](auto I, auto START, auto QBc, auto IS_Pc) {
+          constexpr int i = decltype(I)::value, st = decltype(START)::value, qb = decltype(QBc)::value;
+          constexpr bool IS_P = decltype(IS_Pc)::value;
+          constexpr int GI = (IS_P ? 0 : 2) + qb;
+          constexpr int QS = 4 / EPS;  // slots per quad of rows
+          // request the row values of quad vq two slots before its first element (slot st + QS vq)
+          if constexpr (i + 2 >= st && i + 2 < st + VL && (i + 2 - st) % QS == 0) {
+            constexpr int vq = (i + 2 - st) / QS;
+            rowv[GI][vq & 1] = *(const f32x4*)((IS_P ? lsel : deltal) + qb * 32 + 8 * vq + 4 * g);
+          }
+          if constexpr (i >= st && i < st + VL) {
+            constexpr int k = i - st, vq = k / QS;
+            const f32x4 r4 = rowv[GI][vq & 1];
 #pragma unroll
-          for (int e2 = 0; e2 < 2; e2++) {
-            const int e = 2 * (k % 2) + e2, v = 4 * vq + e;
-            if constexpr (IS_P) {
-              float pv = fast_exp2(__builtin_fmaf(s[qb][v], c, -r4[e]));
-              if (MASKED) {
-                const int r = qb * 32 + 8 * vq + 4 * g + e;
-                const int qrow = qi0 + r;
-                const bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || segl[r] == segk);
-                pv = ok ? pv : 0.f;
+            for (int e2 = 0; e2 < EPS; e2++) {
+              const int e = EPS * (k % QS) + e2, v = 4 * vq + e;
+              if constexpr (IS_P) {
+                float pv = fast_exp2(__builtin_fmaf(s[qb][v], c, -r4[e]));
+                if (MASKED) {
+                  const int r = qb * 32 + 8 * vq + 4 * g + e;
+                  const int qrow = qi0 + r;
+                  const bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || segl[r] == segk);
+                  pv = ok ? pv : 0.f;
+                }
+                asm volatile("" : "+v"(pv));  // anchors the computation in this slot (it would sink past the barrier)
+                s[qb][v] = pv;
+              } else {
+                float dsv = s[qb][v] * (dp[qb][v] - r4[e]);
+                asm volatile("" : "+v"(dsv));
+                dp[qb][v] = dsv;
               }
-              s[qb][v] = pv;
-            } else {
-              dp[qb][v] = s[qb][v] * (dp[qb][v] - r4[e]);
+            }
+            if constexpr (((k + 1) * EPS) % 8 == 0) {
+              constexpr int hh = (k + 1) * EPS / 8 - 1;
+              const f32x16& x = IS_P ? s[qb] : dp[qb];
+              const v8 packed = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4],
+                                         x[8 * hh + 5], x[8 * hh + 6], x[8 * hh + 7]);
+              if constexpr (IS_P) pf[qb][hh] = packed;
+              else df[qb][hh] = packed;
             }
           }
-          if constexpr (k % 4 == 3) {
-            constexpr int hh = k / 4;
-            const f32x16& x = IS_P ? s[qb] : dp[qb];
-            const v8 packed = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4],
-                                       x[8 * hh + 5], x[8 * hh + 6], x[8 * hh + 7]);
-            if constexpr (IS_P) pf[qb][hh] = packed;
-            else df[qb][hh] = packed;
+        };
+        // transposition of tile t+1 (buffer bn), one step per slot from slot C0 on
+        auto transpose_step = [&](auto I) {
+          constexpr int i = decltype(I)::value;
+          if constexpr (i == TQ0) trq.read(bn);
+          if constexpr (i == TO0) tro.read(bn + Q_BYTES);
+          if constexpr (i >= TQ0 + 2 && i < TQ0 + 2 + 8 / WPS)
+            static_for<0, WPS>([&](auto W) {
+              trq.write(bn + Q_BYTES + DO_BYTES, std::integral_constant<int, (i - TQ0 - 2) * WPS + decltype(W)::value>{});
+            });
+          if constexpr (i >= TO0 + 2 && i < TO0 + 2 + 8 / WPS)
+            static_for<0, WPS>([&](auto W) {
+              tro.write(bn + Q_BYTES + DO_BYTES + QTR_BYTES, std::integral_constant<int, (i - TO0 - 2) * WPS + decltype(W)::value>{});
+            });
+        };
+        typedef std::integral_constant<int, 0> I0;
+        typedef std::integral_constant<int, 1> I1;
+        if constexpr (COMPUTE) static_for<0, AHEAD>([&](auto I) { fr[decltype(I)::value % NF] = frag(I); });
+        static_for<0, NS>([&](auto I) {
+          constexpr int i = decltype(I)::value;
+          if constexpr (i == C0) {
+            // this wave's loads of tile t+1 were issued a tile ago (vmcnt only: fragment reads stay in flight)
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
+            if (issue_next) issue_tile(n_hl, n_idx, buf, rnext);
+            __builtin_amdgcn_sched_barrier(0);
           }
-        }
+          if constexpr (COMPUTE) {
+            if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
+            mma(I, fr[i % NF]);
+            valu(I, std::integral_constant<int, VP0>{}, I0{}, std::true_type{});
+            valu(I, std::integral_constant<int, VP1>{}, I1{}, std::true_type{});
+            valu(I, std::integral_constant<int, VS0>{}, I0{}, std::false_type{});
+            valu(I, std::integral_constant<int, VS1>{}, I1{}, std::false_type{});
+          }
+          transpose_step(I);
+          __builtin_amdgcn_sched_barrier(0);
+        });
       };
-      typedef std::integral_constant<int, 0> I0;
-      typedef std::integral_constant<int, 1> I1;
-      static_for<0, AHEAD>([&](auto I) { fr[decltype(I)::value % NF] = frag(I); });
-      static_for<0, NS>([&](auto I) {
-        constexpr int i = decltype(I)::value;
-        if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
-        mma(I, fr[i % NF]);
-        valu(I, std::integral_constant<int, VP0>{}, I0{}, std::true_type{});
-        valu(I, std::integral_constant<int, VP1>{}, I1{}, std::true_type{});
-        valu(I, std::integral_constant<int, VS0>{}, I0{}, std::false_type{});
-        valu(I, std::integral_constant<int, VS1>{}, I1{}, std::false_type{});
-        __builtin_amdgcn_sched_barrier(0);
-      });
+      if (mode == 1) body(std::integral_constant<int, 1>{});
+      else if (mode == 2) body(std::integral_constant<int, 2>{});
+      else body(std::integral_constant<int, 0>{});
+      __syncthreads();
+      if (issue_next) advance(n_hl, n_idx);
+      advance(c_hl, c_idx);
+      rslot = rslot == 2 ? 0 : rslot + 1;
+    }
+  } else {
+    // Wide heads: one buffer, and the register file does not hold the staggered schedule: the next tile is
+    // requested once this one has been used, both query blocks go through each step together.
+    int c_hl = 0, c_idx = 0;
+    auto stage = [&](int hl, int idx) {
+      issue_tile(hl, idx, 0, 0);
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();
+      transpose_tile<DQK>(smem, smem + Q_BYTES + DO_BYTES, tid);
+      transpose_tile<DV>(smem + Q_BYTES, smem + Q_BYTES + DO_BYTES + QTR_BYTES, tid);
+      __syncthreads();
     };
-    if constexpr (DQK <= 128) {
-      if (!skip) {
-        if (need_mask) body(std::true_type{});
-        else body(std::false_type{});
-      }
-    } else {
-      // Wider heads do not fit the staggered schedule in the register file: both query blocks go
-      // through each step together.
+    if (n_iter > 0) stage(0, 0);
+    for (int it = 0; it < n_iter; it++) {
+      const int qi0 = qtile_of(c_idx) * BMQ;
+      const int mode = tile_mode(c_idx, qi0);
+      const bool need_mask = mode == 2;
+      const unsigned char* ql = smem;
+      const unsigned char* dol = ql + Q_BYTES;
+      const unsigned char* qtl = dol + DO_BYTES;
+      const unsigned char* dotl = qtl + QTR_BYTES;
+      const float* lsel = (const float*)rows_base;
+      const float* deltal = lsel + BMQ;
+      const int* segl = (const int*)(deltal + BMQ);
       constexpr int QB = BMQ / 32;
-    if (!skip) {
+      if (mode != 0) {
         f32x16 sacc[QB], dpacc[QB];
-  #pragma unroll
+#pragma unroll
         for (int qb = 0; qb < QB; qb++)
-  #pragma unroll
+#pragma unroll
           for (int v = 0; v < 16; v++) { sacc[qb][v] = 0.f; dpacc[qb][v] = 0.f; }
         // S = Q K^T  (rows = queries, columns = this wave's kv rows)
-  #pragma unroll
+#pragma unroll
         for (int ks = 0; ks < KS_QK; ks++)
-  #pragma unroll
+#pragma unroll
           for (int qb = 0; qb < QB; qb++) {
-            const v8 qf = *(const v8*)(ql + QT::off(qb * 32 + ln, 2 * ks + g));
+            const v8 qf = *(const v8*)(ql + faq[ks] + qb * 32 * QT::ROWB);
             sacc[qb] = MT<T>::mfma32(qf, kf[ks], sacc[qb]);
           }
         // dP = dO V^T
-  #pragma unroll
+#pragma unroll
         for (int ks = 0; ks < KS_DV; ks++)
-  #pragma unroll
+#pragma unroll
           for (int qb = 0; qb < QB; qb++) {
-            const v8 dof = *(const v8*)(dol + OT::off(qb * 32 + ln, 2 * ks + g));
+            const v8 dof = *(const v8*)(dol + fao[ks] + qb * 32 * OT::ROWB);
             dpacc[qb] = MT<T>::mfma32(dof, vf[ks], dpacc[qb]);
           }
         // P = exp2(S*c - lse), dS = P o (dP - delta); rows of the C tile are queries
         v8 pfr[BMQ / 16], dsf[BMQ / 16];
         const int kvcol = wkv0 + ln;
-  #pragma unroll
+#pragma unroll
         for (int qb = 0; qb < QB; qb++)
-  #pragma unroll
+#pragma unroll
           for (int vq = 0; vq < 4; vq++) {
             const f32x4 l4 = *(const f32x4*)(lsel + qb * 32 + 8 * vq + 4 * g);
-  #pragma unroll
+#pragma unroll
             for (int e = 0; e < 4; e++) sacc[qb][4 * vq + e] = fast_exp2(__builtin_fmaf(sacc[qb][4 * vq + e], c, -l4[e]));
           }
         if (need_mask) {  // separate pass: the common unmasked tile carries no per-element branches
-  #pragma unroll
+#pragma unroll
           for (int qb = 0; qb < QB; qb++)
-  #pragma unroll
+#pragma unroll
             for (int v = 0; v < 16; v++) {
               const int r = qb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
               const int qrow = qi0 + r;
@@ -550,15 +686,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
               sacc[qb][v] = ok ? sacc[qb][v] : 0.f;
             }
         }
-  #pragma unroll
+#pragma unroll
         for (int qb = 0; qb < QB; qb++) {
-  #pragma unroll
+#pragma unroll
           for (int vq = 0; vq < 4; vq++) {
             const f32x4 d4 = *(const f32x4*)(deltal + qb * 32 + 8 * vq + 4 * g);
-  #pragma unroll
+#pragma unroll
             for (int e = 0; e < 4; e++) dpacc[qb][4 * vq + e] = sacc[qb][4 * vq + e] * (dpacc[qb][4 * vq + e] - d4[e]);
           }
-  #pragma unroll
+#pragma unroll
           for (int hh = 0; hh < 2; hh++) {
             const f32x16& s = sacc[qb];
             const f32x16& d = dpacc[qb];
@@ -569,33 +705,24 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
           }
         }
         // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 64 query rows)
-  #pragma unroll
+#pragma unroll
         for (int ks = 0; ks < BMQ / 16; ks++) {
-  #pragma unroll
+#pragma unroll
           for (int d = 0; d < DVB; d++) {
-            const v8 f = *(const v8*)(dotl + TrTile64::chunk_off(d * 32 + ln, ks, g));
+            const v8 f = *(const v8*)(dotl + ta[ks ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
             dvacc[d] = MT<T>::mfma32(f, pfr[ks], dvacc[d]);
           }
-  #pragma unroll
+#pragma unroll
           for (int d = 0; d < DKB; d++) {
-            const v8 f = *(const v8*)(qtl + TrTile64::chunk_off(d * 32 + ln, ks, g));
+            const v8 f = *(const v8*)(qtl + ta[ks ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
             dkacc[d] = MT<T>::mfma32(f, dsf[ks], dkacc[d]);
           }
         }
       }
+      __syncthreads();  // everyone is done with the tile
+      advance(c_hl, c_idx);
+      if (it + 1 < n_iter) stage(c_hl, c_idx);
     }
-    if (it + 1 < n_iter) {
-      if (NBUF == 1) {  // single buffer: the next tile can only be requested once this one has been used
-        __syncthreads();
-        load_tile(nxt_hl, nxt_idx, 0);
-      }
-      __builtin_amdgcn_s_waitcnt(0);
-      __syncthreads();  // the next tile's row-major copies are complete, everyone is done with this tile
-      finish_tile(NBUF == 2 ? (buf ^ 1) : 0);
-    }
-    __syncthreads();
-    cur_idx = nxt_idx;
-    cur_hl = nxt_hl;
   }
 
   // ---- epilogue: lane = kv row, 4 consecutive head-dim values per store
@@ -873,10 +1000,11 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
   // dK, dV
   {
     constexpr int BMQ = 64, BNK = 128;
-    constexpr int BUF = DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES + (DQK + DV) * TrTile64::ROW_BYTES + BMQ * 12;
-    constexpr int NBUF = (2 * BUF + 4096 <= 160 * 1024) ? 2 : 1;
+    constexpr int BUF = DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES + (DQK + DV) * TrTile64::ROW_BYTES;
+    constexpr int ROWS = 3 * BMQ * 12;
+    constexpr int NBUF = (2 * BUF + ROWS + 4096 <= 160 * 1024) ? 2 : 1;
     const int nqt = (a.Sq + BMQ - 1) / BMQ;
-    const size_t smem = (size_t)NBUF * BUF + (SEG ? (size_t)(3 * nqt + 8) * 4 : 0);
+    const size_t smem = (size_t)NBUF * BUF + ROWS + (SEG ? (size_t)(3 * nqt + 8) * 4 : 0);
     TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_bwd: Sq=%d needs %zu bytes of LDS (max 163840)", a.Sq, smem);
     auto kern = attn_bwd_dkdv_kernel<T, DQK, DV, NBUF, CAUSAL, SEG>;
     static bool attr_set = false;
@@ -928,7 +1056,7 @@ using namespace tp;
 
 extern "C" size_t tp_attn_bwd_workspace_bytes(int B, int Hq, int Sq) {
   if (B <= 0 || Hq <= 0 || Sq <= 0) return 0;
-  return (size_t)B * Hq * Sq * sizeof(float);
+  return 2 * (size_t)B * Hq * Sq * sizeof(float);  // delta and the log2-scaled LSE, one float per query row each
 }
 
 extern "C" int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, const void* v, const void* out,
