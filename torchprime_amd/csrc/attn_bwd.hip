@@ -170,14 +170,21 @@ struct DmaTile {
   // orders every later LDS read behind an LDS-writing load it knows of, which would stall the tile being
   // computed on the one in flight; the caller waits (s_waitcnt 0 + barrier) before the tile is read.
   // Rows past the end of the tensor (offset >= rs.z) arrive as zeros.
+  template <int I>
+  __device__ __forceinline__ void issue_one(u32x4 rs, unsigned tile_byte_offset, unsigned char* lds_tile, int wave) const {
+    const unsigned dst = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lds_tile + (wave * PER_WAVE + I) * 1024));
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(dst), "v"(vo[I]), "s"(rs), "s"(tile_byte_offset) : "memory");
+  }
   __device__ __forceinline__ void issue(u32x4 rs, unsigned tile_byte_offset, unsigned char* lds_tile, int wave) const {
     tile_byte_offset = __builtin_amdgcn_readfirstlane(tile_byte_offset);
-#pragma unroll
-    for (int i = 0; i < PER_WAVE; i++) {
-      const unsigned dst = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lds_tile + (wave * PER_WAVE + i) * 1024));
-      asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                   :: "s"(dst), "v"(vo[i]), "s"(rs), "s"(tile_byte_offset) : "memory");
-    }
+    if constexpr (PER_WAVE > 0) issue_one<0>(rs, tile_byte_offset, lds_tile, wave);
+    if constexpr (PER_WAVE > 1) issue_one<1>(rs, tile_byte_offset, lds_tile, wave);
+    if constexpr (PER_WAVE > 2) issue_one<2>(rs, tile_byte_offset, lds_tile, wave);
+    if constexpr (PER_WAVE > 3) issue_one<3>(rs, tile_byte_offset, lds_tile, wave);
+    if constexpr (PER_WAVE > 4) issue_one<4>(rs, tile_byte_offset, lds_tile, wave);
+    if constexpr (PER_WAVE > 5) issue_one<5>(rs, tile_byte_offset, lds_tile, wave);
+    static_assert(PER_WAVE <= 6, "head dim above 192");
   }
 };
 // buffer resource words for the assembly loads: base, stride 0, size in bytes, raw-buffer flags
@@ -295,9 +302,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   typedef DmaTile<DV> OT;
   constexpr int Q_BYTES = QT::BYTES, DO_BYTES = OT::BYTES;
   constexpr int QTR_BYTES = DQK * TrTile64::ROW_BYTES, DOTR_BYTES = DV * TrTile64::ROW_BYTES;
-  constexpr int ROW_BYTES = BMQ * 4 * 3;  // lse (log2 units), delta, segment id per query row: 3 slots
+  constexpr int ROW_BYTES = BMQ * 4 * 4;  // lse (log2 units), delta, segment id per query row (+1 unused): 3 slots
   constexpr int BUF_BYTES = Q_BYTES + DO_BYTES + QTR_BYTES + DOTR_BYTES;
-  constexpr bool PIPE = NBUF == 2 && DQK <= 128 && DV <= 128;
+  constexpr bool PIPE = NBUF == 2 && DQK == DV && DQK <= 128;
 
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -466,29 +473,50 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       const float* deltal = lsel + BMQ;
       const int* segl = (const int*)(deltal + BMQ);
       const int rnext = rslot >= 1 ? rslot - 1 : 2;  // (it + 2) % 3, the slot tile t-1 used
+      // descriptors of tile t+2's loads (wave-uniform), issued piecewise in part 2
+      struct { u32x4 rq, ro, rr; unsigned offq, offo, offr; } nx;
+      {
+        const int hq = hk * a.n_rep + (issue_next ? n_hl : 0);
+        const int qt = issue_next ? qtile_of(n_idx) : 0;
+        nx.rq = make_rsrc_words((const T*)a.q + b * a.qs[0] + hq * a.qs[1], issue_next ? q_span : 0u);
+        nx.ro = make_rsrc_words((const T*)a.dout + b * a.dos[0] + hq * a.dos[1], issue_next ? do_span : 0u);
+        const int64_t ro = ((int64_t)b * a.Hq + hq) * Sq;
+        const void* src = wave == 0 ? (const void*)(lse2 + ro) : wave == 1 ? (const void*)(a.delta + ro) : (const void*)segb;
+        // wave 3 (and wave 2 without segment ids) fetches nothing: size 0
+        nx.rr = make_rsrc_words(src, (issue_next && (wave < 2 || (SEG && wave == 2))) ? (unsigned)Sq * 4u : 0u);
+        nx.offq = __builtin_amdgcn_readfirstlane((unsigned)qt * q_tile_bytes);
+        nx.offo = __builtin_amdgcn_readfirstlane((unsigned)qt * do_tile_bytes);
+        nx.offr = __builtin_amdgcn_readfirstlane((unsigned)(qt * BMQ) * 4u);
+      }
 
       // The tile body is laid out by hand as a sequence of slots, one MFMA each, with a scheduling barrier
       // after every slot: the LDS fragment a slot needs was requested AHEAD slots earlier, and the
       // exponentials / products that turn S, dP into the 16-bit operands P, dS are spread over the slots
       // under the MFMAs of the other query block.  (Left to itself the compiler reads each fragment right
       // before its MFMA and the matrix unit waits out every LDS round trip.)
-      //   slots   A0: S0 = Q0 K^T   A1: S1 = Q1 K^T   B0: dP0 = dO0 V^T   B1: dP1 = dO1 V^T
-      //           C0, C1: dV^T += dO^T P   D0, D1: dK^T += Q^T dS
-      //   VALU    P0 ends before C0, P1 before C1, dS0 before D0, dS1 before D1
+      //   slots   part 1: S0 = Q0 K^T with dP0 = dO0 V^T, then S1 with dP1
+      //           part 2: dV^T += dO0^T P0, dK^T += Q0^T dS0, dV^T += dO1^T P1, dK^T += Q1^T dS1
+      //   VALU    P0 and dS0 under S1/dP1 and the first of part 2, P1 and dS1 under part 2
       auto body = [&](auto mode_c) {
         constexpr int MODE = decltype(mode_c)::value;
         constexpr bool COMPUTE = MODE != 0, MASKED = MODE == 2;
-        constexpr int A0 = 0, A1 = A0 + KS_QK, B0 = A1 + KS_QK, B1 = B0 + KS_DV, C0 = B1 + KS_DV, C1 = C0 + 2 * DVB,
-                      D0 = C1 + 2 * DVB, D1 = D0 + 2 * DKB, NS = D1 + 2 * DKB;
+        // part 1: S and dP steps of a query block alternate (two independent accumulation chains);
+        // part 2: dV0, dK0, dV1, dK1 (four accumulators each, used round robin)
+        constexpr int K = KS_QK, CL = 2 * DVB;
+        static_assert(KS_QK == KS_DV && DKB == DVB, "the slot plan assumes equal head dims");
+        constexpr int C0 = 4 * K, NS = C0 + 4 * CL;
         constexpr int AHEAD = 3, NF = 4;  // fragment read-ahead, fragment ring size
-        // VALU groups: one element per slot where the tile body is long enough, each group ending right
-        // before the MFMAs that consume its packed operand
-        constexpr int EPS = (C0 - 16 >= A1) ? 1 : 2, VL = 16 / EPS;
-        constexpr int VP0 = C0 - VL, VP1 = C1 - VL, VS0 = D0 - VL, VS1 = D1 - VL;
-        static_assert(VP0 >= A1 && VP1 >= B0 && VS0 >= B1 && VS1 >= C0 && VS0 > VP0 && VS1 > VP1, "operands not ready");
+        // VALU groups: P of a block starts when its S is complete, dS half a group later; each group ends
+        // right before the MFMAs that consume its packed operand
+        constexpr int EPS = K >= 8 ? 1 : 2, VL = 16 / EPS;
+        constexpr int VP0 = 2 * K, VS0 = VP0 + VL / 2, VP1 = 4 * K, VS1 = VP1 + VL / 2;
+        static_assert(VP0 + VL <= C0 && VS0 + VL <= C0 + CL && VP1 + VL <= C0 + 2 * CL && VS1 + VL <= C0 + 3 * CL,
+                      "operands not ready");
         // transposing the next tile: reads of a tile in one slot, then WPS column pairs per slot
         constexpr int WPS = (NS - C0 >= 24) ? 1 : 2, TQ0 = C0, TO0 = TQ0 + 2 + 8 / WPS;
         static_assert(TO0 + 2 + 8 / WPS <= NS, "second half too short for the transposition");
+        constexpr int N_DMA = QT::PER_WAVE + OT::PER_WAVE + 1, DMA_EVERY = (NS - C0) / N_DMA;
+        static_assert(DMA_EVERY >= 1, "second half too short for the loads");
         const int kvcol = wkv0 + ln;
         v8 fr[NF];
         f32x16 s[2], dp[2];
@@ -497,33 +525,27 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
 
         auto frag = [&](auto I) -> v8 {
           constexpr int i = decltype(I)::value;
-          if constexpr (i < A1) return *(const v8*)(ql + faq[i - A0]);
-          else if constexpr (i < B0) return *(const v8*)(ql + faq[i - A1] + 32 * QT::ROWB);
-          else if constexpr (i < B1) return *(const v8*)(dol + fao[i - B0]);
-          else if constexpr (i < C0) return *(const v8*)(dol + fao[i - B1] + 32 * OT::ROWB);
-          else if constexpr (i < D0) {
-            constexpr int qb = (i - C0) / (2 * DVB), j = (i - C0) % (2 * DVB), hh = j / DVB, d = j % DVB;
-            return *(const v8*)(dotl + ta[(2 * qb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+          if constexpr (i < C0) {
+            constexpr int qb = i / (2 * K), ks = (i % (2 * K)) / 2;
+            if constexpr (i % 2 == 0) return *(const v8*)(ql + faq[ks] + qb * 32 * QT::ROWB);
+            else return *(const v8*)(dol + fao[ks] + qb * 32 * OT::ROWB);
           } else {
-            constexpr int qb = (i - D0) / (2 * DKB), j = (i - D0) % (2 * DKB), hh = j / DKB, d = j % DKB;
-            return *(const v8*)(qtl + ta[(2 * qb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+            constexpr int ph = (i - C0) / CL, qb = ph / 2, j = (i - C0) % CL, hh = j / DVB, d = j % DVB;
+            const unsigned char* base = (ph % 2 == 0) ? dotl : qtl;
+            return *(const v8*)(base + ta[(2 * qb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
           }
         };
         auto mma = [&](auto I, const v8& f) {
           constexpr int i = decltype(I)::value;
           const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          if constexpr (i < B0) {
-            constexpr int qb = (i - A0) / KS_QK, ks = (i - A0) % KS_QK;
-            s[qb] = MT<T>::mfma32(f, kf[ks], ks == 0 ? zero : s[qb]);
-          } else if constexpr (i < C0) {
-            constexpr int qb = (i - B0) / KS_DV, ks = (i - B0) % KS_DV;
-            dp[qb] = MT<T>::mfma32(f, vf[ks], ks == 0 ? zero : dp[qb]);
-          } else if constexpr (i < D0) {
-            constexpr int qb = (i - C0) / (2 * DVB), j = (i - C0) % (2 * DVB), hh = j / DVB, d = j % DVB;
-            dvacc[d] = MT<T>::mfma32(f, pf[qb][hh], dvacc[d]);
+          if constexpr (i < C0) {
+            constexpr int qb = i / (2 * K), ks = (i % (2 * K)) / 2;
+            if constexpr (i % 2 == 0) s[qb] = MT<T>::mfma32(f, kf[ks], ks == 0 ? zero : s[qb]);
+            else dp[qb] = MT<T>::mfma32(f, vf[ks], ks == 0 ? zero : dp[qb]);
           } else {
-            constexpr int qb = (i - D0) / (2 * DKB), j = (i - D0) % (2 * DKB), hh = j / DKB, d = j % DKB;
-            dkacc[d] = MT<T>::mfma32(f, df[qb][hh], dkacc[d]);
+            constexpr int ph = (i - C0) / CL, qb = ph / 2, j = (i - C0) % CL, hh = j / DVB, d = j % DVB;
+            if constexpr (ph % 2 == 0) dvacc[d] = MT<T>::mfma32(f, pf[qb][hh], dvacc[d]);
+            else dkacc[d] = MT<T>::mfma32(f, df[qb][hh], dkacc[d]);
           }
         };
         // VALU group of query block QB starting at slot START: EPS elements per slot for VL slots.
@@ -594,8 +616,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
             // this wave's loads of tile t+1 were issued a tile ago (vmcnt only: fragment reads stay in flight)
             __builtin_amdgcn_s_waitcnt(0x0F70);
             __syncthreads();
-            if (issue_next) issue_tile(n_hl, n_idx, buf, rnext);
             __builtin_amdgcn_sched_barrier(0);
+          }
+          // the loads of tile t+2, one instruction every few slots: the texture path takes a kilobyte in
+          // some 25 cycles for the whole CU, and a wave that issues them back to back sits out the queue
+          if constexpr (i >= C0 && (i - C0) % DMA_EVERY == 0 && (i - C0) / DMA_EVERY < N_DMA) {
+            constexpr int m = (i - C0) / DMA_EVERY;
+            // (no branch here: past the last tile the descriptors have size 0 and the loads deliver zeros
+            // into buffers nobody reads any more)
+            if constexpr (m < QT::PER_WAVE) qdma.template issue_one<m>(nx.rq, nx.offq, bl, wave);
+            else if constexpr (m < QT::PER_WAVE + OT::PER_WAVE) dodma.template issue_one<m - QT::PER_WAVE>(nx.ro, nx.offo, bl + Q_BYTES, wave);
+            else dma_dword(nx.rr, nx.offr, rows_base + rnext * ROW_BYTES + wave * BMQ * 4, lane);
           }
           if constexpr (COMPUTE) {
             if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
@@ -1001,7 +1032,7 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
   {
     constexpr int BMQ = 64, BNK = 128;
     constexpr int BUF = DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES + (DQK + DV) * TrTile64::ROW_BYTES;
-    constexpr int ROWS = 3 * BMQ * 12;
+    constexpr int ROWS = 3 * BMQ * 16;
     constexpr int NBUF = (2 * BUF + ROWS + 4096 <= 160 * 1024) ? 2 : 1;
     const int nqt = (a.Sq + BMQ - 1) / BMQ;
     const size_t smem = (size_t)NBUF * BUF + ROWS + (SEG ? (size_t)(3 * nqt + 8) * 4 : 0);
