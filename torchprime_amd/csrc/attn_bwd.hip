@@ -34,6 +34,25 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
+// position j of a sequence that alternates the steps of two accumulation chains of lengths n0 and n1
+struct AbSlot {
+  int kind, k;
+};
+__host__ __device__ constexpr AbSlot ab_slot(int j, int n0, int n1) {
+  int n = 0;
+  for (int k = 0; k < (n0 > n1 ? n0 : n1); k++) {
+    if (k < n0) {
+      if (n == j) return AbSlot{0, k};
+      n++;
+    }
+    if (k < n1) {
+      if (n == j) return AbSlot{1, k};
+      n++;
+    }
+  }
+  return AbSlot{0, 0};
+}
+
 struct BwdArgs {
   const void* q;
   const void* k;
@@ -891,6 +910,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
     if (SEG && tid < BN) ((int*)(base + K_BYTES + V_BYTES + KTR_BYTES))[tid] = sreg;
   };
 
+  unsigned ta[4];  // per-lane byte offsets of the K^T fragments (swizzle resolved once)
+#pragma unroll
+  for (int m = 0; m < 4; m++) ta[m] = (unsigned)TrTile64::chunk_off(ln, m, g);
+
   f32x16 dqacc[DKB];
 #pragma unroll
   for (int d = 0; d < DKB; d++)
@@ -925,61 +948,85 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
       skip = skip || hi < wqmin || lo > wqmax;
       need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
     }
-    // The two 32-row kv blocks of the tile are staggered (source order = intended overlap):
-    //   S0^T = K0 Q^T, dP0^T = V0 dO^T          |
-    //   S1^T = K1 Q^T, dP1^T = V1 dO^T          | dS0^T = exp2(S0^T c - lse) o (dP0^T - delta)
-    //   dQ^T += K0^T dS0^T                      | dS1^T
-    //   dQ^T += K1^T dS1^T                      | (transpose + LDS store of the next tile)
+    // The tile body is laid out slot by slot (one MFMA each, a scheduling barrier after every slot): the
+    // LDS fragment of a slot is requested AHEAD slots earlier, and the element-wise work that turns
+    // S^T, dP^T into the 16-bit operand dS^T is spread under the MFMAs of the following slots.
+    //   slots   S0^T = K0 Q^T alternating with dP0^T = V0 dO^T;  S1^T with dP1^T;
+    //           dQ^T += K0^T dS0^T;  dQ^T += K1^T dS1^T (first the half whose operand is ready first)
+    //   VALU    dS0^T under S1^T/dP1^T; dS1^T under the dQ^T slots that do not need it yet
     auto body = [&](auto masked_c) {
       constexpr bool MASKED = decltype(masked_c)::value;
-      auto s_dp = [&](int nb, f32x16& sa, f32x16& dp) {
-#pragma unroll
-        for (int v = 0; v < 16; v++) { sa[v] = 0.f; dp[v] = 0.f; }
-#pragma unroll
-        for (int ks = 0; ks < KS_QK; ks++) {
-          const v8 f = *(const v8*)(kl + KT::off(nb * 32 + ln, 16 * ks + 8 * g));
-          sa = MT<T>::mfma32(f, qf[ks], sa);
-        }
-#pragma unroll
-        for (int ks = 0; ks < KS_DV; ks++) {
-          const v8 f = *(const v8*)(vl + VT::off(nb * 32 + ln, 16 * ks + 8 * g));
-          dp = MT<T>::mfma32(f, dof[ks], dp);
+      constexpr int L1 = KS_QK + KS_DV, ACC0 = 2 * L1, ACC1 = ACC0 + 2 * DKB, NS = ACC1 + 2 * DKB;
+      constexpr int AHEAD = 3, NF = 4;
+      v8 fr[NF];
+      f32x16 s[2], dp[2];
+      v8 df[2][2];
+      auto frag = [&](auto I) -> v8 {
+        constexpr int i = decltype(I)::value;
+        if constexpr (i < ACC0) {
+          constexpr int nb = i / L1;
+          constexpr AbSlot sl = ab_slot(i % L1, KS_QK, KS_DV);
+          if constexpr (sl.kind == 0) return *(const v8*)(kl + KT::off(nb * 32 + ln, 16 * sl.k + 8 * g));
+          else return *(const v8*)(vl + VT::off(nb * 32 + ln, 16 * sl.k + 8 * g));
+        } else {
+          constexpr int nb = (i - ACC0) / (2 * DKB), j = (i - ACC0) % (2 * DKB), hh = j / DKB, d = j % DKB;
+          return *(const v8*)(ktl + ta[(2 * nb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
         }
       };
-      auto ds_of = [&](int nb, f32x16& sa, f32x16& dp, v8 (&df)[2]) {
+      auto mma = [&](auto I, const v8& f) {
+        constexpr int i = decltype(I)::value;
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if constexpr (i < ACC0) {
+          constexpr int nb = i / L1;
+          constexpr AbSlot sl = ab_slot(i % L1, KS_QK, KS_DV);
+          if constexpr (sl.kind == 0) s[nb] = MT<T>::mfma32(f, qf[sl.k], sl.k == 0 ? zero : s[nb]);
+          else dp[nb] = MT<T>::mfma32(f, dof[sl.k], sl.k == 0 ? zero : dp[nb]);
+        } else {
+          constexpr int nb = (i - ACC0) / (2 * DKB), j = (i - ACC0) % (2 * DKB), hh = j / DKB, d = j % DKB;
+          dqacc[d] = MT<T>::mfma32(f, df[nb][hh], dqacc[d]);
+        }
+      };
+      // elements [E0, E0 + N) of block NB spread evenly over the LEN slots starting at START
+      auto valu = [&](auto I, auto NBc, auto E0c, auto Nc, auto STARTc, auto LENc) {
+        constexpr int i = decltype(I)::value, nb = decltype(NBc)::value, e0 = decltype(E0c)::value, n = decltype(Nc)::value,
+                      st = decltype(STARTc)::value, len = decltype(LENc)::value;
+        if constexpr (i >= st && i < st + len) {
+          constexpr int k = i - st, lo = e0 + (k * n + len - 1) / len, hi = e0 + ((k + 1) * n + len - 1) / len;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-          float pv = fast_exp2(__builtin_fmaf(sa[v], c, -lse_s));
-          if (MASKED) {
-            const int kvl = nb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
-            const int kv = kv0 + kvl;
-            const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
-            pv = ok ? pv : 0.f;
+          for (int v = lo; v < hi; v++) {
+            float pv = fast_exp2(__builtin_fmaf(s[nb][v], c, -lse_s));
+            if (MASKED) {
+              const int kvl = nb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
+              const int kv = kv0 + kvl;
+              const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
+              pv = ok ? pv : 0.f;
+            }
+            float dsv = pv * (dp[nb][v] - delta_s);
+            asm volatile("" : "+v"(dsv));  // keeps the computation in this slot
+            dp[nb][v] = dsv;
           }
-          dp[v] = pv * (dp[v] - delta_s);
-        }
-#pragma unroll
-        for (int hh = 0; hh < 2; hh++)
-          df[hh] = pack8<T>(dp[8 * hh + 0], dp[8 * hh + 1], dp[8 * hh + 2], dp[8 * hh + 3], dp[8 * hh + 4],
-                            dp[8 * hh + 5], dp[8 * hh + 6], dp[8 * hh + 7]);
-      };
-      auto accumulate = [&](int nb, const v8 (&df)[2]) {
-#pragma unroll
-        for (int hh = 0; hh < 2; hh++)
-#pragma unroll
-          for (int d = 0; d < DKB; d++) {
-            const v8 f = *(const v8*)(ktl + TrTile64::chunk_off(d * 32 + ln, 2 * nb + hh, g));
-            dqacc[d] = MT<T>::mfma32(f, df[hh], dqacc[d]);
+          if constexpr (hi % 8 == 0 && hi > lo) {
+            constexpr int hh = hi / 8 - 1;
+            const f32x16& x = dp[nb];
+            df[nb][hh] = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4], x[8 * hh + 5],
+                                  x[8 * hh + 6], x[8 * hh + 7]);
           }
+        }
       };
-      f32x16 s0, dp0, s1, dp1;
-      v8 df0[2], df1[2];
-      s_dp(0, s0, dp0);
-      s_dp(1, s1, dp1);
-      ds_of(0, s0, dp0, df0);
-      accumulate(0, df0);
-      ds_of(1, s1, dp1, df1);
-      accumulate(1, df1);
+      typedef std::integral_constant<int, 0> I0;
+      typedef std::integral_constant<int, 1> I1;
+      typedef std::integral_constant<int, 8> I8;
+      typedef std::integral_constant<int, 16> I16;
+      static_for<0, AHEAD>([&](auto I) { fr[decltype(I)::value % NF] = frag(I); });
+      static_for<0, NS>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+        if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
+        mma(I, fr[i % NF]);
+        valu(I, I0{}, I0{}, I16{}, std::integral_constant<int, L1>{}, std::integral_constant<int, L1>{});
+        valu(I, I1{}, I0{}, I8{}, std::integral_constant<int, ACC0>{}, std::integral_constant<int, 2 * DKB>{});
+        valu(I, I1{}, I8{}, I8{}, std::integral_constant<int, ACC1>{}, std::integral_constant<int, DKB>{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
     };
     if (!skip) {
       if (need_mask) body(std::true_type{});
