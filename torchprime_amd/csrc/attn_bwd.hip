@@ -114,11 +114,18 @@ struct Stage64 {
   u32x4 r[ITEMS][4];
   unsigned vo[ITEMS][4];  // byte offsets of this thread's 16-byte pieces inside a tile
 
+  // block (column chunk c8, row quad rq) of work item `item`.  Row quads are dealt so that the 32 lanes
+  // whose transposed 8-byte stores are served together fall into 32 different bank pairs.
+  static __device__ __forceinline__ int c8_of(int item) { return item % (D / 8); }
+  static __device__ __forceinline__ int rq_of(int item) {
+    const int rqi = item / (D / 8);
+    return (rqi & ~3) | ((rqi & 1) << 1) | ((rqi >> 1) & 1);
+  }
   __device__ __forceinline__ void init(int64_t row_stride, int tid) {
 #pragma unroll
     for (int i = 0; i < ITEMS; i++) {
       const int item = tid + 256 * i;
-      const int c8 = item % (D / 8), rq = item / (D / 8);
+      const int c8 = c8_of(item), rq = rq_of(item);
 #pragma unroll
       for (int ii = 0; ii < 4; ii++) vo[i][ii] = (unsigned)(((4 * rq + ii) * row_stride + c8 * 8) * 2);
     }
@@ -138,7 +145,7 @@ struct Stage64 {
     for (int i = 0; i < ITEMS; i++) {
       const int item = tid + 256 * i;
       if (item < TOT) {
-        const int c8 = item % (D / 8), rq = item / (D / 8);
+        const int c8 = c8_of(item), rq = rq_of(item);
 #pragma unroll
         for (int ii = 0; ii < 4; ii++) *(u32x4*)(dst + RowTile<D>::off(4 * rq + ii, c8 * 8)) = r[i][ii];
       }
@@ -149,9 +156,20 @@ struct Stage64 {
     for (int i = 0; i < ITEMS; i++) {
       const int item = tid + 256 * i;
       if (item < TOT) {
-        const int c8 = item % (D / 8), rq = item / (D / 8);
+        const int c8 = c8_of(item), rq = rq_of(item);
+        // odd column chunks take their columns in the order 1,0,3,2,...: at every step half the lanes
+        // write even LDS rows and half odd ones
+        const int flip = c8 & 1;
+        const unsigned sel_even = flip ? 0x07060302u : 0x05040100u, sel_odd = flip ? 0x05040100u : 0x07060302u;
 #pragma unroll
-        for (int j = 0; j < 8; j++) *(u32x2*)(dst + TrTile64::quad_off(c8 * 8 + j, rq)) = transpose_col(r[i], j);
+        for (int j = 0; j < 8; j++) {
+          const unsigned sel = (j & 1) ? sel_odd : sel_even;
+          const int w = j >> 1;
+          u32x2 o;
+          o.x = __builtin_amdgcn_perm(r[i][1][w], r[i][0][w], sel);
+          o.y = __builtin_amdgcn_perm(r[i][3][w], r[i][2][w], sel);
+          *(u32x2*)(dst + TrTile64::quad_off(c8 * 8 + (j ^ flip), rq)) = o;
+        }
       }
     }
   }
