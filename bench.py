@@ -156,11 +156,15 @@ def bench_attention(args, dev):
     n: {"ms": round(avg[n], 4), "algorithmic_TFLOPs": round(algo[n] / (avg[n] * 1e-3) / 1e12, 2) if avg[n] > 0 else None}
     for n in names
   }
+  # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this script, each scaled by
+  # what the counter reads for the 256 MiB copy of --calib-copy); the summary with the commands is
+  # profiles/attn_fwd_bwd_llama3_8b_S8192_hbm_traffic.md.  Counters cannot be read from inside this process.
+  measured_traffic = {"attn_fwd": 9.05e8, "attn_bwd_dkdv": 9.86e9, "attn_bwd_dq": 1.38e9}
   dom = max(("attn_fwd", "attn_bwd_dkdv", "attn_bwd_dq"), key=lambda n: avg[n])
   achieved = algo[dom] / (avg[dom] * 1e-3) / 1e12
   roofline = {
     "bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-    "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None, "launch_ms": round(avg[dom], 4),
+    "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": measured_traffic[dom], "launch_ms": round(avg[dom], 4),
     "step_frac_of_peak": round(flops_step / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
   }  # fmt: skip
   return ms_per_step, flops_step, roofline, kernels, dict(B=B, Hq=Hq, Hkv=Hkv, S=S, D=D)
@@ -274,6 +278,8 @@ def main():
   ap.add_argument("--warmup", type=int, default=3)
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
   ap.add_argument("--no-extra", action="store_true", help="skip the RMSNorm / RoPE bandwidth leg")
+  ap.add_argument("--calib-copy", action="store_true",
+                  help="also run one 256 MiB device copy (the known-size kernel the HBM counters are scaled by)")
   args = ap.parse_args()
   if args.gpus != 1:
     sys.exit("bench.py measures the one-GPU hot path only: run with --gpus 1 (no multi-GPU path is part of this build)")
@@ -285,6 +291,12 @@ def main():
   if not torch.cuda.is_available():
     sys.exit("bench.py needs a GPU")
   dev = torch.device("cuda", 0)
+  if args.calib_copy:
+    src = torch.zeros((64 << 20,), dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+    torch.cuda.synchronize()
+    del src, dst
   ms_per_step, flops_step, roofline, kernels, shape = bench_attention(args, dev)
   extra = None if args.no_extra else bench_norm_rope(dev)
   torch.cuda.empty_cache()

@@ -125,6 +125,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
   }
 
   // ---- global -> register staging of one K/V tile (buffer loads, rows past Skv read as zero)
+  // V row quads are dealt to threads so that the 32 lanes whose transposed 8-byte stores are served
+  // together fall into 32 different bank pairs
+  auto v_quad = [](int rqi) { return (rqi & ~3) | ((rqi & 1) << 1) | ((rqi >> 1) & 1); };
   const rsrc_t krs = make_rsrc(kb, span_bytes(Skv, a.ks[2], DQK));
   const rsrc_t vrs = make_rsrc(vb, span_bytes(Skv, a.vs[2], DV));
   const unsigned k_tile_bytes = (unsigned)(BN * a.ks[2] * 2), v_tile_bytes = (unsigned)(BN * a.vs[2] * 2);
@@ -137,7 +140,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
 #pragma unroll
   for (int i = 0; i < V_ITEMS; i++) {
     const int item = tid + 256 * i;
-    const int c8 = item % (DV / 8), rq = item / (DV / 8);
+    const int c8 = item % (DV / 8), rq = v_quad(item / (DV / 8));
 #pragma unroll
     for (int ii = 0; ii < 4; ii++) vvo[i][ii] = (unsigned)(((4 * rq + ii) * a.vs[2] + c8 * 8) * 2);
   }
@@ -169,9 +172,20 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
     for (int i = 0; i < V_ITEMS; i++) {
       const int item = tid + 256 * i;
       if (item < V_TOT) {
-        const int c8 = item % (DV / 8), rq = item / (DV / 8);
+        const int c8 = item % (DV / 8), rq = v_quad(item / (DV / 8));
+        // odd column chunks take their columns in the order 1,0,3,2,...: at every step half the lanes
+        // write even LDS rows and half odd ones
+        const int flip = c8 & 1;
+        const unsigned sel_even = flip ? 0x07060302u : 0x05040100u, sel_odd = flip ? 0x05040100u : 0x07060302u;
 #pragma unroll
-        for (int j = 0; j < 8; j++) *(u32x2*)(vl + TrTile64::quad_off(c8 * 8 + j, rq)) = transpose_col(vreg[i], j);
+        for (int j = 0; j < 8; j++) {
+          const unsigned sel = (j & 1) ? sel_odd : sel_even;
+          const int w = j >> 1;
+          u32x2 o;
+          o.x = __builtin_amdgcn_perm(vreg[i][1][w], vreg[i][0][w], sel);
+          o.y = __builtin_amdgcn_perm(vreg[i][3][w], vreg[i][2][w], sel);
+          *(u32x2*)(vl + TrTile64::quad_off(c8 * 8 + (j ^ flip), rq)) = o;
+        }
       }
     }
     if (SEG && tid < BN) ((int*)(vl + V_BYTES))[tid] = sreg;
