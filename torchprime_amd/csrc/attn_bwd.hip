@@ -439,14 +439,21 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   for (int m = 0; m < 4; m++) ta[m] = (unsigned)TrTile64::chunk_off(ln, m, g);
 
   f32x16 dkacc[DKB], dvacc[DVB];
+  {
+    // whole-vector values from the start: element-wise initialisation makes the compiler track 16 scalars per
+    // accumulator across the loop and reassemble the tuple around every accumulating MFMA
+    f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int d = 0; d < DKB; d++)
+    for (int d = 0; d < DKB; d++) {
+      asm volatile("" : "+a"(zero16));
+      dkacc[d] = zero16;
+    }
 #pragma unroll
-    for (int v = 0; v < 16; v++) dkacc[d][v] = 0.f;
-#pragma unroll
-  for (int d = 0; d < DVB; d++)
-#pragma unroll
-    for (int v = 0; v < 16; v++) dvacc[d][v] = 0.f;
+    for (int d = 0; d < DVB; d++) {
+      asm volatile("" : "+a"(zero16));
+      dvacc[d] = zero16;
+    }
+  }
   const float c = a.scale_log2;
 
   // wave-level decisions for a query tile (uniform): skip if every query row precedes every kv row
@@ -494,6 +501,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     }
     __syncthreads();
 
+    // fragment ring: slot i's LDS fragment is requested AHEAD slots earlier and kept in fr[i % NF]; the
+    // first AHEAD fragments of a tile are requested at the end of the tile before it (its row-major
+    // tiles are complete by then), so that the LDS round trip and the scalar bookkeeping at the top of
+    // the loop overlap
+    constexpr int AHEAD = 7, NF = 8;
+    v8 fr[NF];
+    static_for<0, AHEAD>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      static_assert(AHEAD <= 2 * KS_QK, "the carried fragments all belong to the first query block");
+      fr[i % NF] = (i % 2 == 0) ? *(const v8*)(smem + faq[i / 2]) : *(const v8*)(smem + Q_BYTES + fao[i / 2]);
+    });
     int rslot = 0;
     for (int it = 0; it < n_iter; it++) {
       const int buf = it & 1;
@@ -542,7 +560,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         constexpr int K = KS_QK, CL = 2 * DVB;
         static_assert(KS_QK == KS_DV && DKB == DVB, "the slot plan assumes equal head dims");
         constexpr int C0 = 4 * K, NS = C0 + 4 * CL;
-        constexpr int AHEAD = 3, NF = 4;  // fragment read-ahead, fragment ring size
         // VALU groups: P of a block starts when its S is complete, dS half a group later; each group ends
         // right before the MFMAs that consume its packed operand
         constexpr int EPS = K >= 8 ? 1 : 2, VL = 16 / EPS;
@@ -555,7 +572,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         constexpr int N_DMA = QT::PER_WAVE + OT::PER_WAVE + 1, DMA_EVERY = (NS - C0) / N_DMA;
         static_assert(DMA_EVERY >= 1, "second half too short for the loads");
         const int kvcol = wkv0 + ln;
-        v8 fr[NF];
         f32x16 s[2], dp[2];
         v8 pf[2][2], df[2][2];
         f32x4 rowv[4][2];  // per VALU group: LSE or delta of four query rows, requested two slots before use
@@ -581,8 +597,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
             else dp[qb] = MT<T>::mfma32(f, vf[ks], ks == 0 ? zero : dp[qb]);
           } else {
             constexpr int ph = (i - C0) / CL, qb = ph / 2, j = (i - C0) % CL, hh = j / DVB, d = j % DVB;
-            if constexpr (ph % 2 == 0) dvacc[d] = MT<T>::mfma32(f, pf[qb][hh], dvacc[d]);
-            else dkacc[d] = MT<T>::mfma32(f, df[qb][hh], dkacc[d]);
+            if constexpr (ph % 2 == 0) MT<T>::mfma32_acc(dvacc[d], f, pf[qb][hh]);
+            else MT<T>::mfma32_acc(dkacc[d], f, df[qb][hh]);
           }
         };
         // VALU group of query block QB starting at slot START: EPS elements per slot for VL slots.
@@ -646,7 +662,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         };
         typedef std::integral_constant<int, 0> I0;
         typedef std::integral_constant<int, 1> I1;
-        if constexpr (COMPUTE) static_for<0, AHEAD>([&](auto I) { fr[decltype(I)::value % NF] = frag(I); });
         static_for<0, NS>([&](auto I) {
           constexpr int i = decltype(I)::value;
           if constexpr (i == C0) {
@@ -675,6 +690,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
           }
           transpose_step(I);
           __builtin_amdgcn_sched_barrier(0);
+        });
+        static_for<0, AHEAD>([&](auto I) {
+          constexpr int i = decltype(I)::value;
+          fr[i % NF] = (i % 2 == 0) ? *(const v8*)(bn + faq[i / 2]) : *(const v8*)(bn + Q_BYTES + fao[i / 2]);
         });
       };
       if (mode == 1) body(std::integral_constant<int, 1>{});

@@ -22,6 +22,10 @@ template <> struct MT<bf16_t> {
   static __device__ __forceinline__ f32x16 mfma32(v8 a, v8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  // c += a b with the accumulator pinned to the accumulation registers (see mfma32_acc below)
+  static __device__ __forceinline__ void mfma32_acc(f32x16& c, v8 a, v8 b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
 };
 template <> struct MT<f16_t> {
   typedef f16x8 v8;
@@ -29,7 +33,17 @@ template <> struct MT<f16_t> {
   static __device__ __forceinline__ f32x16 mfma32(v8 a, v8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
+  static __device__ __forceinline__ void mfma32_acc(f32x16& c, v8 a, v8 b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
 };
+// mfma32_acc: long-lived accumulators that only MFMAs touch inside a loop (dK, dV) are kept in the
+// accumulation half of the register file by writing the instruction out with an "a" constraint.  With the
+// compiler's own MFMA form every result sits in the 256 architectural VGPRs, which then cannot also hold
+// the K/V fragments, and each fragment is copied out of an AGPR right before the MFMA that needs it.
+// What the compiler no longer sees, and the callers guarantee: the same accumulator is reused by a later
+// mfma32_acc only (exactly overlapping destination, for which the matrix unit forwards), and it is read
+// by ordinary instructions only after the loop and a barrier, hundreds of cycles after the last MFMA.
 
 // eight floats -> one 16-byte MFMA operand (round to nearest even)
 template <typename T>
