@@ -839,16 +839,19 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
 // ------------------------------------------------------------------------------------------------
 // dQ
 // ------------------------------------------------------------------------------------------------
-template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
-__global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
+// NW = waves per workgroup.  With 8 (head dims up to 128) two waves share a SIMD, 256 registers each: a wave
+// issues at most one instruction every four cycles, and at ~600 instructions for 48 MFMAs per tile a single
+// wave per SIMD leaves the matrix unit idle most of the time, whatever the order of its instructions.
+template <typename T, int DQK, int DV, int NW, bool CAUSAL, bool SEG>
+__global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   typedef typename MT<T>::v8 v8;
-  constexpr int BN = 64, BM = 128;
+  constexpr int BN = 64, BM = 32 * NW;
+  static_assert(NW == 4 || (NW == 8 && DQK == DV && DQK <= 128), "8 waves: equal head dims up to 128");
   constexpr int KS_QK = DQK / 16, KS_DV = DV / 16, DKB = DQK / 32;
   typedef RowTile<DQK> KT;
   typedef RowTile<DV> VT;
   constexpr int K_BYTES = BN * KT::STRIDE, V_BYTES = BN * VT::STRIDE, KTR_BYTES = DQK * TrTile64::ROW_BYTES;
   constexpr int BUF_BYTES = K_BYTES + V_BYTES + KTR_BYTES + BN * 4;
-  constexpr int VCH = DV / 8, V_ITEMS = BN * VCH / 256;
 
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -900,10 +903,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
     wqmin = __builtin_amdgcn_readfirstlane(wqmin);
     wqmax = __builtin_amdgcn_readfirstlane(wqmax);
     if (lane == 0) { bq[2 * wave] = wqmin; bq[2 * wave + 1] = wqmax; }
-    seg_tile_ranges(segb, Skv, 0, ntiles, kvmin, kvmax, wave, lane);
+    if (wave < 4) seg_tile_ranges(segb, Skv, 0, ntiles, kvmin, kvmax, wave, lane);
     __syncthreads();
-    const int bqmin = min(min(bq[0], bq[2]), min(bq[4], bq[6]));
-    const int bqmax = max(max(bq[1], bq[3]), max(bq[5], bq[7]));
+    int bqmin = bq[0], bqmax = bq[1];
+#pragma unroll
+    for (int w = 1; w < NW; w++) { bqmin = min(bqmin, bq[2 * w]); bqmax = max(bqmax, bq[2 * w + 1]); }
     int cnt = 0;
     for (int base = 0; base < ntiles; base += 64) {
       const int t = base + lane;
@@ -916,34 +920,45 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
     __syncthreads();
   }
 
-  Stage64<DQK> kst;
-  kst.init(a.ks[2], tid);
+  // ---- staging of one K/V tile through registers.  Every thread owns one 4-row x 8-column block of K and
+  // (4 waves) one of V; with 8 waves a wave stages K on even iterations and V on odd ones, or the other way
+  // round, in the same registers.
+  const int stid = tid & 255;
   const rsrc_t krs = make_rsrc(kb, span_bytes(Skv, a.ks[2], DQK));
   const rsrc_t vrs = make_rsrc(vb, span_bytes(Skv, a.vs[2], DV));
   const unsigned k_tile_bytes = (unsigned)(BN * a.ks[2] * 2), v_tile_bytes = (unsigned)(BN * a.vs[2] * 2);
-  u32x4 vreg[V_ITEMS];
-  unsigned vvo[V_ITEMS];
-#pragma unroll
-  for (int i = 0; i < V_ITEMS; i++) {
-    const int item = tid + 256 * i;
-    vvo[i] = (unsigned)(((item / VCH) * a.vs[2] + (item % VCH) * 8) * 2);
-  }
+  Stage64<DQK> kst;
+  Stage64<DV> vst;
+  kst.init(a.ks[2], stid);
+  vst.init(a.vs[2], stid);
   int sreg = 0;
-  auto load_tile = [&](int t) {
-    kst.load(krs, (unsigned)t * k_tile_bytes, tid);
+  auto stages_k = [&](int it) { return NW == 4 || ((wave >> 2) == (it & 1)); };
+  auto load_tile = [&](int t, int it) {
+    if (NW == 4) {
+      kst.load(krs, (unsigned)t * k_tile_bytes, stid);
+      vst.load(vrs, (unsigned)t * v_tile_bytes, stid);
+    } else {
+      // same registers for either role (the offsets and the resource are picked, not the code path)
+      const bool sk = stages_k(it);
+      const rsrc_t rs = sk ? krs : vrs;
+      const unsigned off = sk ? (unsigned)t * k_tile_bytes : (unsigned)t * v_tile_bytes;
 #pragma unroll
-    for (int i = 0; i < V_ITEMS; i++) vreg[i] = buf_load16(vrs, vvo[i], (unsigned)t * v_tile_bytes);
+      for (int ii = 0; ii < 4; ii++) kst.r[0][ii] = buf_load16(rs, sk ? kst.vo[0][ii] : vst.vo[0][ii], off);
+    }
     if (SEG && tid < BN) sreg = segb[min(t * BN + tid, Skv - 1)];
   };
-  auto store_tile = [&](int buf) {
+  auto store_tile = [&](int buf, int it) {
     unsigned char* base = smem + buf * BUF_BYTES;
-    kst.store_rowmajor(base, tid);
-#pragma unroll
-    for (int i = 0; i < V_ITEMS; i++) {
-      const int item = tid + 256 * i;
-      *(u32x4*)(base + K_BYTES + VT::off(item / VCH, (item % VCH) * 8)) = vreg[i];
+    if (NW == 4) {
+      kst.store_rowmajor(base, stid);
+      vst.store_rowmajor(base + K_BYTES, stid);
+      kst.store_transposed(base + K_BYTES + V_BYTES, stid);
+    } else if (stages_k(it)) {
+      kst.store_rowmajor(base, stid);
+      kst.store_transposed(base + K_BYTES + V_BYTES, stid);
+    } else {
+      kst.store_rowmajor(base + K_BYTES, stid);  // K and V tiles have the same shape here
     }
-    kst.store_transposed(base + K_BYTES + V_BYTES, tid);
     if (SEG && tid < BN) ((int*)(base + K_BYTES + V_BYTES + KTR_BYTES))[tid] = sreg;
   };
 
@@ -961,8 +976,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
   const int qrow = wq0 + ln;
 
   if (nact > 0) {
-    load_tile(SEG ? active[0] : 0);
-    store_tile(0);
+    load_tile(SEG ? active[0] : 0, 1);
+    store_tile(0, 1);
+    if (NW == 8) {  // the other half of the tile (roles swapped)
+      load_tile(SEG ? active[0] : 0, 0);
+      store_tile(0, 0);
+    }
   }
   __builtin_amdgcn_s_waitcnt(0);  // Q / dO fragments, LSE and delta have landed (see the dK/dV kernel)
   __syncthreads();
@@ -971,7 +990,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
     const int t = SEG ? active[it] : it;
     const int kv0 = t * BN;
     const int buf = it & 1;
-    if (it + 1 < nact) load_tile(SEG ? active[it + 1] : it + 1);
+    if (it + 1 < nact) load_tile(SEG ? active[it + 1] : it + 1, it);
 
     const unsigned char* kl = smem + buf * BUF_BYTES;
     const unsigned char* vl = kl + K_BYTES;
@@ -993,33 +1012,42 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
     //   VALU    dS0^T under S1^T/dP1^T; dS1^T under the dQ^T slots that do not need it yet
     auto body = [&](auto masked_c) {
       constexpr bool MASKED = decltype(masked_c)::value;
-      constexpr int L1 = KS_QK + KS_DV, ACC0 = 2 * L1, ACC1 = ACC0 + 2 * DKB, NS = ACC1 + 2 * DKB;
+      // 4 waves: S/dP of both kv blocks first, so that dS of block 0 has the MFMAs of block 1 next to it.
+      // 8 waves: block by block (S/dP, dS, dQ), which keeps one pair of 32x32 tiles live; the other wave on
+      // the SIMD supplies the overlap.
+      constexpr bool STAG = NW == 4;
+      constexpr int L1 = KS_QK + KS_DV, A2 = 2 * DKB, NS = 2 * L1 + 2 * A2;
+      constexpr int AB1 = STAG ? L1 : L1 + A2;          // first slot of S1/dP1
+      constexpr int ACC0 = STAG ? 2 * L1 : L1;          // first slot of dQ += K0^T dS0
+      constexpr int ACC1 = 2 * L1 + A2;                 // first slot of dQ += K1^T dS1
       constexpr int AHEAD = 3, NF = 4;
       v8 fr[NF];
       f32x16 s[2], dp[2];
       v8 df[2][2];
       auto frag = [&](auto I) -> v8 {
         constexpr int i = decltype(I)::value;
-        if constexpr (i < ACC0) {
-          constexpr int nb = i / L1;
-          constexpr AbSlot sl = ab_slot(i % L1, KS_QK, KS_DV);
+        constexpr bool is_acc = (i >= ACC0 && i < ACC0 + A2) || i >= ACC1;
+        if constexpr (!is_acc) {
+          constexpr int nb = i >= AB1 ? 1 : 0;
+          constexpr AbSlot sl = ab_slot(nb ? i - AB1 : i, KS_QK, KS_DV);
           if constexpr (sl.kind == 0) return *(const v8*)(kl + KT::off(nb * 32 + ln, 16 * sl.k + 8 * g));
           else return *(const v8*)(vl + VT::off(nb * 32 + ln, 16 * sl.k + 8 * g));
         } else {
-          constexpr int nb = (i - ACC0) / (2 * DKB), j = (i - ACC0) % (2 * DKB), hh = j / DKB, d = j % DKB;
+          constexpr int nb = i >= ACC1 ? 1 : 0, j = nb ? i - ACC1 : i - ACC0, hh = j / DKB, d = j % DKB;
           return *(const v8*)(ktl + ta[(2 * nb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
         }
       };
       auto mma = [&](auto I, const v8& f) {
         constexpr int i = decltype(I)::value;
+        constexpr bool is_acc = (i >= ACC0 && i < ACC0 + A2) || i >= ACC1;
         const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        if constexpr (i < ACC0) {
-          constexpr int nb = i / L1;
-          constexpr AbSlot sl = ab_slot(i % L1, KS_QK, KS_DV);
+        if constexpr (!is_acc) {
+          constexpr int nb = i >= AB1 ? 1 : 0;
+          constexpr AbSlot sl = ab_slot(nb ? i - AB1 : i, KS_QK, KS_DV);
           if constexpr (sl.kind == 0) s[nb] = MT<T>::mfma32(f, qf[sl.k], sl.k == 0 ? zero : s[nb]);
           else dp[nb] = MT<T>::mfma32(f, dof[sl.k], sl.k == 0 ? zero : dp[nb]);
         } else {
-          constexpr int nb = (i - ACC0) / (2 * DKB), j = (i - ACC0) % (2 * DKB), hh = j / DKB, d = j % DKB;
+          constexpr int nb = i >= ACC1 ? 1 : 0, j = nb ? i - ACC1 : i - ACC0, hh = j / DKB, d = j % DKB;
           dqacc[d] = MT<T>::mfma32(f, df[nb][hh], dqacc[d]);
         }
       };
@@ -1042,12 +1070,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
             asm volatile("" : "+v"(dsv));  // keeps the computation in this slot
             dp[nb][v] = dsv;
           }
-          if constexpr (hi % 8 == 0 && hi > lo) {
-            constexpr int hh = hi / 8 - 1;
-            const f32x16& x = dp[nb];
-            df[nb][hh] = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4], x[8 * hh + 5],
-                                  x[8 * hh + 6], x[8 * hh + 7]);
-          }
+          static_for<0, 2>([&](auto H) {  // every half whose eighth value was produced in this slot
+            constexpr int hh = decltype(H)::value;
+            if constexpr (8 * hh + 8 > lo && 8 * hh + 8 <= hi) {
+              const f32x16& x = dp[nb];
+              df[nb][hh] = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4],
+                                    x[8 * hh + 5], x[8 * hh + 6], x[8 * hh + 7]);
+            }
+          });
         }
       };
       typedef std::integral_constant<int, 0> I0;
@@ -1058,10 +1088,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
       static_for<0, NS>([&](auto I) {
         constexpr int i = decltype(I)::value;
         if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
+        if constexpr (!STAG) {
+          // whole dS of a block right before the dQ slots that consume it
+          valu(I, I0{}, I0{}, I16{}, std::integral_constant<int, ACC0>{}, I1{});
+          valu(I, I1{}, I0{}, I16{}, std::integral_constant<int, ACC1>{}, I1{});
+        }
         mma(I, fr[i % NF]);
-        valu(I, I0{}, I0{}, I16{}, std::integral_constant<int, L1>{}, std::integral_constant<int, L1>{});
-        valu(I, I1{}, I0{}, I8{}, std::integral_constant<int, ACC0>{}, std::integral_constant<int, 2 * DKB>{});
-        valu(I, I1{}, I8{}, I8{}, std::integral_constant<int, ACC1>{}, std::integral_constant<int, DKB>{});
+        if constexpr (STAG) {
+          valu(I, I0{}, I0{}, I16{}, std::integral_constant<int, L1>{}, std::integral_constant<int, L1>{});
+          valu(I, I1{}, I0{}, I8{}, std::integral_constant<int, ACC0>{}, std::integral_constant<int, 2 * DKB>{});
+          valu(I, I1{}, I8{}, I8{}, std::integral_constant<int, ACC1>{}, std::integral_constant<int, DKB>{});
+        }
         __builtin_amdgcn_sched_barrier(0);
       });
     };
@@ -1069,7 +1106,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const BwdArgs a) {
       if (need_mask) body(std::true_type{});
       else body(std::false_type{});
     }
-    if (it + 1 < nact) store_tile(buf ^ 1);
+    if (it + 1 < nact) store_tile(buf ^ 1, it);
     __syncthreads();
   }
 
@@ -1135,19 +1172,22 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
   mark(ev, 2, st);
   // dQ
   {
-    constexpr int BN = 64, BM = 128;
+    // eight waves (two per SIMD) where a wave's registers fit in half a SIMD's file
+    // (the non-causal 128-wide variant does not fit 256 registers without spilling: it keeps four waves)
+    constexpr int NW = (DQK == DV && (DQK <= 64 || (DQK <= 128 && CAUSAL))) ? 8 : 4;
+    constexpr int BN = 64, BM = 32 * NW;
     constexpr int BUF = BN * RowTile<DQK>::STRIDE + BN * RowTile<DV>::STRIDE + DQK * TrTile64::ROW_BYTES + BN * 4;
     const int nt = (a.Skv + BN - 1) / BN;
-    const size_t smem = 2 * (size_t)BUF + (SEG ? (size_t)(3 * nt + 8) * 4 : 0);
+    const size_t smem = 2 * (size_t)BUF + (SEG ? (size_t)(3 * nt + 2 * NW) * 4 : 0);
     TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_bwd: Skv=%d needs %zu bytes of LDS (max 163840)", a.Skv, smem);
-    auto kern = attn_bwd_dq_kernel<T, DQK, DV, CAUSAL, SEG>;
+    auto kern = attn_bwd_dq_kernel<T, DQK, DV, NW, CAUSAL, SEG>;
     static bool attr_set = false;
     if (!attr_set) {
       int rc = set_max_lds(kern, "tp_attn_bwd(dq)");
       if (rc) return rc;
       attr_set = true;
     }
-    kern<<<dim3(xcd_grid((a.Sq + BM - 1) / BM, a.n_rep, a.B * a.Hkv)), dim3(256), smem, st>>>(a);
+    kern<<<dim3(xcd_grid((a.Sq + BM - 1) / BM, a.n_rep, a.B * a.Hkv)), dim3(64 * NW), smem, st>>>(a);
     int rc = check_launch("tp_attn_bwd(dq)");
     if (rc) return rc;
   }
