@@ -512,6 +512,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       static_assert(AHEAD <= 2 * KS_QK, "the carried fragments all belong to the first query block");
       fr[i % NF] = (i % 2 == 0) ? *(const v8*)(smem + faq[i / 2]) : *(const v8*)(smem + Q_BYTES + fao[i / 2]);
     });
+    struct { u32x4 rq, ro, rr; unsigned offq, offo, offr; } nx;
     int rslot = 0;
     for (int it = 0; it < n_iter; it++) {
       const int buf = it & 1;
@@ -528,17 +529,19 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       const float* deltal = lsel + BMQ;
       const int* segl = (const int*)(deltal + BMQ);
       const int rnext = rslot >= 1 ? rslot - 1 : 2;  // (it + 2) % 3, the slot tile t-1 used
-      // descriptors of tile t+2's loads (wave-uniform), issued piecewise in part 2
-      struct { u32x4 rq, ro, rr; unsigned offq, offo, offr; } nx;
-      {
+      // descriptors of tile t+2's loads (wave-uniform), issued piecewise in part 2.  The bases change with
+      // the query head only; they are rebuilt when a new head starts (and when the tiles run out: size 0).
+      if (it == 0 || n_idx == 0 || !issue_next) {
         const int hq = hk * a.n_rep + (issue_next ? n_hl : 0);
-        const int qt = issue_next ? qtile_of(n_idx) : 0;
         nx.rq = make_rsrc_words((const T*)a.q + b * a.qs[0] + hq * a.qs[1], issue_next ? q_span : 0u);
         nx.ro = make_rsrc_words((const T*)a.dout + b * a.dos[0] + hq * a.dos[1], issue_next ? do_span : 0u);
         const int64_t ro = ((int64_t)b * a.Hq + hq) * Sq;
         const void* src = wave == 0 ? (const void*)(lse2 + ro) : wave == 1 ? (const void*)(a.delta + ro) : (const void*)segb;
         // wave 3 (and wave 2 without segment ids) fetches nothing: size 0
         nx.rr = make_rsrc_words(src, (issue_next && (wave < 2 || (SEG && wave == 2))) ? (unsigned)Sq * 4u : 0u);
+      }
+      {
+        const int qt = issue_next ? qtile_of(n_idx) : 0;
         nx.offq = __builtin_amdgcn_readfirstlane((unsigned)qt * q_tile_bytes);
         nx.offo = __builtin_amdgcn_readfirstlane((unsigned)qt * do_tile_bytes);
         nx.offr = __builtin_amdgcn_readfirstlane((unsigned)(qt * BMQ) * 4u);
