@@ -505,12 +505,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     // first AHEAD fragments of a tile are requested at the end of the tile before it (its row-major
     // tiles are complete by then), so that the LDS round trip and the scalar bookkeeping at the top of
     // the loop overlap
-    constexpr int AHEAD = 7, NF = 8;
+    constexpr int AHEAD = KS_QK >= 8 ? 7 : 3, NF = AHEAD + 1;
     v8 fr[NF];
     static_for<0, AHEAD>([&](auto I) {
       constexpr int i = decltype(I)::value;
-      static_assert(AHEAD <= 2 * KS_QK, "the carried fragments all belong to the first query block");
-      fr[i % NF] = (i % 2 == 0) ? *(const v8*)(smem + faq[i / 2]) : *(const v8*)(smem + Q_BYTES + fao[i / 2]);
+      static_assert(AHEAD <= KS_QK, "the carried fragments all belong to S of the first query block");
+      fr[i % NF] = *(const v8*)(smem + faq[i]);
     });
     struct { u32x4 rq, ro, rr; unsigned offq, offo, offr; } nx;
     int rslot = 0;
@@ -552,22 +552,24 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       // exponentials / products that turn S, dP into the 16-bit operands P, dS are spread over the slots
       // under the MFMAs of the other query block.  (Left to itself the compiler reads each fragment right
       // before its MFMA and the matrix unit waits out every LDS round trip.)
-      //   slots   part 1: S0 = Q0 K^T with dP0 = dO0 V^T, then S1 with dP1
+      //   slots   part 1: S0 = Q0 K^T, S1 = Q1 K^T, dP0 = dO0 V^T, dP1 = dO1 V^T
       //           part 2: dV^T += dO0^T P0, dK^T += Q0^T dS0, dV^T += dO1^T P1, dK^T += Q1^T dS1
-      //   VALU    P0 and dS0 under S1/dP1 and the first of part 2, P1 and dS1 under part 2
+      //   VALU    P0 from S1 on, P1 from dP0 on, dS0 from dP1 on, dS1 from part 2 on
       auto body = [&](auto mode_c) {
         constexpr int MODE = decltype(mode_c)::value;
         constexpr bool COMPUTE = MODE != 0, MASKED = MODE == 2;
-        // part 1: S and dP steps of a query block alternate (two independent accumulation chains);
+        // part 1: S0, S1, dP0, dP1 (the exponentials can start as soon as S0 is complete and are over
+        // before part 2, which carries the transposition of the next tile);
         // part 2: dV0, dK0, dV1, dK1 (four accumulators each, used round robin)
         constexpr int K = KS_QK, CL = 2 * DVB;
         static_assert(KS_QK == KS_DV && DKB == DVB, "the slot plan assumes equal head dims");
         constexpr int C0 = 4 * K, NS = C0 + 4 * CL;
-        // VALU groups: P of a block starts when its S is complete, dS half a group later; each group ends
-        // right before the MFMAs that consume its packed operand
+        // VALU groups, 2K slots each: P of a block starts when its S is complete, dS when its dP is; each
+        // group is over before the MFMAs that consume its packed operand
         constexpr int EPS = K >= 8 ? 1 : 2, VL = 16 / EPS;
-        constexpr int VP0 = 2 * K, VS0 = VP0 + VL / 2, VP1 = 4 * K, VS1 = VP1 + VL / 2;
-        static_assert(VP0 + VL <= C0 && VS0 + VL <= C0 + CL && VP1 + VL <= C0 + 2 * CL && VS1 + VL <= C0 + 3 * CL,
+        constexpr int VP0 = K, VP1 = 2 * K, VS0 = 3 * K, VS1 = 4 * K;
+        static_assert(VL == 2 * K && VP0 + VL <= C0 && VS0 + VL <= C0 + CL && VP1 + VL <= C0 + 2 * CL &&
+                          VS1 + VL <= C0 + 3 * CL,
                       "operands not ready");
         // transposing the next tile: reads of a tile in one slot, then WPS column pairs per slot
         constexpr int WPS = (NS - C0 >= 24) ? 1 : 2, TQ0 = C0, TO0 = TQ0 + 2 + 8 / WPS;
@@ -582,8 +584,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         auto frag = [&](auto I) -> v8 {
           constexpr int i = decltype(I)::value;
           if constexpr (i < C0) {
-            constexpr int qb = i / (2 * K), ks = (i % (2 * K)) / 2;
-            if constexpr (i % 2 == 0) return *(const v8*)(ql + faq[ks] + qb * 32 * QT::ROWB);
+            constexpr int qb = (i / K) % 2, ks = i % K;
+            if constexpr (i < 2 * K) return *(const v8*)(ql + faq[ks] + qb * 32 * QT::ROWB);
             else return *(const v8*)(dol + fao[ks] + qb * 32 * OT::ROWB);
           } else {
             constexpr int ph = (i - C0) / CL, qb = ph / 2, j = (i - C0) % CL, hh = j / DVB, d = j % DVB;
@@ -595,8 +597,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
           constexpr int i = decltype(I)::value;
           const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
           if constexpr (i < C0) {
-            constexpr int qb = i / (2 * K), ks = (i % (2 * K)) / 2;
-            if constexpr (i % 2 == 0) s[qb] = MT<T>::mfma32(f, kf[ks], ks == 0 ? zero : s[qb]);
+            constexpr int qb = (i / K) % 2, ks = i % K;
+            if constexpr (i < 2 * K) s[qb] = MT<T>::mfma32(f, kf[ks], ks == 0 ? zero : s[qb]);
             else dp[qb] = MT<T>::mfma32(f, vf[ks], ks == 0 ? zero : dp[qb]);
           } else {
             constexpr int ph = (i - C0) / CL, qb = ph / 2, j = (i - C0) % CL, hh = j / DVB, d = j % DVB;
@@ -696,7 +698,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         });
         static_for<0, AHEAD>([&](auto I) {
           constexpr int i = decltype(I)::value;
-          fr[i % NF] = (i % 2 == 0) ? *(const v8*)(bn + faq[i / 2]) : *(const v8*)(bn + Q_BYTES + fao[i / 2]);
+          fr[i % NF] = *(const v8*)(bn + faq[i]);
         });
       };
       if (mode == 1) body(std::integral_constant<int, 1>{});
