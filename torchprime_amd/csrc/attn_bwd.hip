@@ -151,6 +151,20 @@ struct Stage64 {
       }
     }
   }
+  // column pair member J (0..7) of the transposed copy, for tiles with one block per thread
+  template <int J>
+  __device__ __forceinline__ void store_transposed_step(unsigned char* dst, int tid) const {
+    static_assert(ITEMS == 1, "one block per thread");
+    if (tid < TOT) {
+      const int c8 = c8_of(tid), rq = rq_of(tid), flip = c8 & 1;
+      const unsigned sel = ((J & 1) ^ flip) ? 0x07060302u : 0x05040100u;
+      constexpr int w = J >> 1;
+      u32x2 o;
+      o.x = __builtin_amdgcn_perm(r[0][1][w], r[0][0][w], sel);
+      o.y = __builtin_amdgcn_perm(r[0][3][w], r[0][2][w], sel);
+      *(u32x2*)(dst + TrTile64::quad_off(c8 * 8 + (J ^ flip), rq)) = o;
+    }
+  }
   __device__ __forceinline__ void store_transposed(unsigned char* dst, int tid) const {
 #pragma unroll
     for (int i = 0; i < ITEMS; i++) {
@@ -926,8 +940,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   }
 
   // ---- staging of one K/V tile through registers.  Every thread owns one 4-row x 8-column block of K and
-  // (4 waves) one of V; with 8 waves a wave stages K on even iterations and V on odd ones, or the other way
-  // round, in the same registers.
+  // (4 waves) one of V; with 8 waves the first four stage K, the last four V.
   const int stid = tid & 255;
   const rsrc_t krs = make_rsrc(kb, span_bytes(Skv, a.ks[2], DQK));
   const rsrc_t vrs = make_rsrc(vb, span_bytes(Skv, a.vs[2], DV));
@@ -937,7 +950,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   kst.init(a.ks[2], stid);
   vst.init(a.vs[2], stid);
   int sreg = 0;
-  auto stages_k = [&](int it) { return NW == 4 || ((wave >> 2) == (it & 1)); };
+  // 8 waves: waves 0..3 stage K (and its transposed copy), waves 4..7 stage V, in the same registers
+  auto stages_k = [&](int) { return NW == 4 || wave < 4; };
   auto load_tile = [&](int t, int it) {
     if (NW == 4) {
       kst.load(krs, (unsigned)t * k_tile_bytes, stid);
@@ -981,12 +995,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   const int qrow = wq0 + ln;
 
   if (nact > 0) {
-    load_tile(SEG ? active[0] : 0, 1);
-    store_tile(0, 1);
-    if (NW == 8) {  // the other half of the tile (roles swapped)
-      load_tile(SEG ? active[0] : 0, 0);
-      store_tile(0, 0);
-    }
+    load_tile(SEG ? active[0] : 0, 0);
+    store_tile(0, 0);
   }
   __builtin_amdgcn_s_waitcnt(0);  // Q / dO fragments, LSE and delta have landed (see the dK/dV kernel)
   __syncthreads();
@@ -1099,6 +1109,16 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
           valu(I, I1{}, I0{}, I16{}, std::integral_constant<int, ACC1>{}, I1{});
         }
         mma(I, fr[i % NF]);
+        if constexpr (!STAG) {
+          // the next tile (requested at the top of this one) goes to the other buffer under the last MFMAs
+          // instead of in a phase of its own; after the last tile this stores stale registers nobody reads
+          constexpr int ST0 = NS - 12;
+          unsigned char* nb_base = smem + (buf ^ 1) * BUF_BYTES;
+          if constexpr (i == ST0) kst.store_rowmajor(nb_base + (wave < 4 ? 0 : K_BYTES), stid);
+          if constexpr (i >= ST0 + 2 && i < ST0 + 10) {
+            if (wave < 4) kst.template store_transposed_step<i - ST0 - 2>(nb_base + K_BYTES + V_BYTES, stid);
+          }
+        }
         if constexpr (STAG) {
           valu(I, I0{}, I0{}, I16{}, std::integral_constant<int, L1>{}, std::integral_constant<int, L1>{});
           valu(I, I1{}, I0{}, I8{}, std::integral_constant<int, ACC0>{}, std::integral_constant<int, 2 * DKB>{});
@@ -1111,7 +1131,11 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
       if (need_mask) body(std::true_type{});
       else body(std::false_type{});
     }
-    if (it + 1 < nact) store_tile(buf ^ 1, it);
+    if (NW == 4 || skip) {
+      if (it + 1 < nact) store_tile(buf ^ 1, it);
+    } else if (SEG && tid < BN) {
+      ((int*)(smem + (buf ^ 1) * BUF_BYTES + K_BYTES + V_BYTES + KTR_BYTES))[tid] = sreg;
+    }
     __syncthreads();
   }
 
