@@ -9,7 +9,7 @@
 
 namespace tp {
 
-constexpr int RMS_MAX_PARTS = 1024;  // partial dw rows written by the backward (multiple of 4)
+constexpr int RMS_MAX_PARTS = 512;  // partial dw rows written by the backward (multiple of 4)
 
 static inline int rms_parts(int64_t rows) {
   int64_t p = (rows + 3) / 4 * 4;
