@@ -7,7 +7,7 @@
 // and dK, dV summed over the n_rep query heads that share a KV head.
 //
 // Three kernels:
-//   attn_delta_kernel     delta[b,h,i] = sum_d dO*O                                   (HBM-bound)
+//   attn_delta_kernel     -delta[b,h,i] = -sum_d dO*O, and the LSE in log2 units      (HBM-bound)
 //   attn_bwd_dkdv_kernel  one workgroup = 128 KV rows of one (batch, kv head); K and V fragments stay
 //                         in registers, Q / dO tiles of every query head of the group stream through
 //                         LDS in both orientations (row-major for S = QK^T and dP = dO V^T, transposed
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
 #pragma unroll
   for (int off = TPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
   if (valid && ch == 0) {
-    a.delta[rowid] = acc;
+    a.delta[rowid] = -acc;  // stored negated: the dK/dV kernel starts its dP accumulators from it
     // second half of the workspace: LSE in log2 units for the dK/dV kernel; a row with no allowed key
     // (LSE = -inf) gets +inf so that its P = exp2(s - inf) = 0
     const float l = a.lse[rowid];
@@ -593,7 +593,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         const int kvcol = wkv0 + ln;
         f32x16 s[2], dp[2];
         v8 pf[2][2], df[2][2];
-        f32x4 rowv[4][2];  // per VALU group: LSE or delta of four query rows, requested two slots before use
+        f32x4 rowv[2][2];  // per P group: LSE of four query rows, requested two slots before use
+        f32x4 nd[4];       // -delta of the 16 rows a lane holds of a query block, requested before its dP
 
         auto frag = [&](auto I) -> v8 {
           constexpr int i = decltype(I)::value;
@@ -612,8 +613,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
           const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
           if constexpr (i < C0) {
             constexpr int qb = (i / K) % 2, ks = i % K;
-            if constexpr (i < 2 * K) s[qb] = MT<T>::mfma32(f, kf[ks], ks == 0 ? zero : s[qb]);
-            else dp[qb] = MT<T>::mfma32(f, vf[ks], ks == 0 ? zero : dp[qb]);
+            if constexpr (i < 2 * K) {
+              s[qb] = MT<T>::mfma32(f, kf[ks], ks == 0 ? zero : s[qb]);
+            } else if constexpr (ks == 0) {
+              // dP starts from -delta of its rows (C layout: value v belongs to row 8 (v/4) + 4 g + v%4), so
+              // that dS = P o dP needs no subtraction
+              const f32x16 init = {nd[0][0], nd[0][1], nd[0][2], nd[0][3], nd[1][0], nd[1][1], nd[1][2], nd[1][3],
+                                   nd[2][0], nd[2][1], nd[2][2], nd[2][3], nd[3][0], nd[3][1], nd[3][2], nd[3][3]};
+              dp[qb] = MT<T>::mfma32(f, vf[ks], init);
+            } else {
+              dp[qb] = MT<T>::mfma32(f, vf[ks], dp[qb]);
+            }
           } else {
             constexpr int ph = (i - C0) / CL, qb = ph / 2, j = (i - C0) % CL, hh = j / DVB, d = j % DVB;
             if constexpr (ph % 2 == 0) MT<T>::mfma32_acc(dvacc[d], f, pf[qb][hh]);
@@ -626,16 +636,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         auto valu = [&](auto I, auto START, auto QBc, auto IS_Pc) {
           constexpr int i = decltype(I)::value, st = decltype(START)::value, qb = decltype(QBc)::value;
           constexpr bool IS_P = decltype(IS_Pc)::value;
-          constexpr int GI = (IS_P ? 0 : 2) + qb;
+          constexpr int GI = qb;
           constexpr int QS = 4 / EPS;  // slots per quad of rows
-          // request the row values of quad vq two slots before its first element (slot st + QS vq)
-          if constexpr (i + 2 >= st && i + 2 < st + VL && (i + 2 - st) % QS == 0) {
+          // request the LSE of quad vq two slots before its first element (slot st + QS vq)
+          if constexpr (IS_P && i + 2 >= st && i + 2 < st + VL && (i + 2 - st) % QS == 0) {
             constexpr int vq = (i + 2 - st) / QS;
-            rowv[GI][vq & 1] = *(const f32x4*)((IS_P ? lsel : deltal) + qb * 32 + 8 * vq + 4 * g);
+            rowv[GI][vq & 1] = *(const f32x4*)(lsel + qb * 32 + 8 * vq + 4 * g);
           }
           if constexpr (i >= st && i < st + VL) {
             constexpr int k = i - st, vq = k / QS;
-            const f32x4 r4 = rowv[GI][vq & 1];
+            const f32x4 r4 = IS_P ? rowv[GI][vq & 1] : f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int e2 = 0; e2 < EPS; e2++) {
               const int e = EPS * (k % QS) + e2, v = 4 * vq + e;
@@ -650,7 +660,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
                 asm volatile("" : "+v"(pv));  // anchors the computation in this slot (it would sink past the barrier)
                 s[qb][v] = pv;
               } else {
-                float dsv = s[qb][v] * (dp[qb][v] - r4[e]);
+                float dsv = s[qb][v] * dp[qb][v];
                 asm volatile("" : "+v"(dsv));
                 dp[qb][v] = dsv;
               }
@@ -700,6 +710,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
             else dma_dword(nx.rr, nx.offr, rows_base + rnext * ROW_BYTES + wave * BMQ * 4, lane);
           }
           if constexpr (COMPUTE) {
+            if constexpr (i + 2 == 2 * K || i + 2 == 3 * K) {
+              constexpr int qb = (i + 2 - 2 * K) / K;
+#pragma unroll
+              for (int vq = 0; vq < 4; vq++) nd[vq] = *(const f32x4*)(deltal + qb * 32 + 8 * vq + 4 * g);
+            }
             if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
             mma(I, fr[i % NF]);
             valu(I, std::integral_constant<int, VP0>{}, I0{}, std::true_type{});
@@ -798,7 +813,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
           for (int vq = 0; vq < 4; vq++) {
             const f32x4 d4 = *(const f32x4*)(deltal + qb * 32 + 8 * vq + 4 * g);
 #pragma unroll
-            for (int e = 0; e < 4; e++) dpacc[qb][4 * vq + e] = sacc[qb][4 * vq + e] * (dpacc[qb][4 * vq + e] - d4[e]);
+            for (int e = 0; e < 4; e++) dpacc[qb][4 * vq + e] = sacc[qb][4 * vq + e] * (dpacc[qb][4 * vq + e] + d4[e]);
           }
 #pragma unroll
           for (int hh = 0; hh < 2; hh++) {
@@ -903,7 +918,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   const int64_t ro = ((int64_t)b * a.Hq + h) * Sq + qrow_c;
   const float lraw = a.lse[ro];
   const float lse_s = (lraw == -INFINITY) ? INFINITY : lraw * LOG2E;
-  const float delta_s = a.delta[ro];
+  const float ndelta_s = a.delta[ro];  // -rowsum(dO o O)
   const int segq = SEG ? segb[qrow_c] : 0;
 
   int* kvmin = (int*)(smem + 2 * BUF_BYTES);
@@ -1081,7 +1096,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
               const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
               pv = ok ? pv : 0.f;
             }
-            float dsv = pv * (dp[nb][v] - delta_s);
+            float dsv = pv * (dp[nb][v] + ndelta_s);
             asm volatile("" : "+v"(dsv));  // keeps the computation in this slot
             dp[nb][v] = dsv;
           }
