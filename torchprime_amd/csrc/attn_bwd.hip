@@ -962,8 +962,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   const unsigned k_tile_bytes = (unsigned)(BN * a.ks[2] * 2), v_tile_bytes = (unsigned)(BN * a.vs[2] * 2);
   Stage64<DQK> kst;
   Stage64<DV> vst;
-  kst.init(a.ks[2], stid);
-  vst.init(a.vs[2], stid);
+  kst.init((NW == 4 || wave < 4) ? a.ks[2] : a.vs[2], stid);  // 8 waves: one set of offsets, the role's
+  if (NW == 4) vst.init(a.vs[2], stid);
   int sreg = 0;
   // 8 waves: waves 0..3 stage K (and its transposed copy), waves 4..7 stage V, in the same registers
   auto stages_k = [&](int) { return NW == 4 || wave < 4; };
@@ -977,7 +977,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
       const rsrc_t rs = sk ? krs : vrs;
       const unsigned off = sk ? (unsigned)t * k_tile_bytes : (unsigned)t * v_tile_bytes;
 #pragma unroll
-      for (int ii = 0; ii < 4; ii++) kst.r[0][ii] = buf_load16(rs, sk ? kst.vo[0][ii] : vst.vo[0][ii], off);
+      for (int ii = 0; ii < 4; ii++) kst.r[0][ii] = buf_load16(rs, kst.vo[0][ii], off);
     }
     if (SEG && tid < BN) sreg = segb[min(t * BN + tid, Skv - 1)];
   };
