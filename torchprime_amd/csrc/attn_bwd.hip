@@ -846,6 +846,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     }
   }
 
+  // every LDS-writing load of this wave has landed before it leaves (the last ones write zeros nobody reads,
+  // but they must not outlive the workgroup's LDS allocation)
+  __builtin_amdgcn_s_waitcnt(0);
   // ---- epilogue: lane = kv row, 4 consecutive head-dim values per store
   const int row = wkv0 + ln;
   if (row < Skv) {
