@@ -26,14 +26,6 @@
 
 namespace tp {
 
-template <int B, int E, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (B < E) {
-    f(std::integral_constant<int, B>{});
-    static_for<B + 1, E>(f);
-  }
-}
-
 // position j of a sequence that alternates the steps of two accumulation chains of lengths n0 and n1
 struct AbSlot {
   int kind, k;

@@ -11,9 +11,21 @@
 // 16h + 8a + 4g + e (a = 0..1, e = 0..3), and the other operand is laid out in LDS so that a lane's
 // 16 bytes hold exactly those rows ("quad-swapped" order, see vt_offset).
 #pragma once
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace tp {
+
+// compile-time loop: f(std::integral_constant<int, B>{}), ..., f(std::integral_constant<int, E - 1>{})
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
 
 template <typename T> struct MT;
 template <> struct MT<bf16_t> {

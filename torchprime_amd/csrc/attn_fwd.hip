@@ -235,37 +235,17 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
 #pragma unroll
       for (int v = 0; v < 16; v++) oacc[d][v] *= alpha;
   };
-  auto exp_half = [&](f32x16& s, v8 (&pf)[2]) {
-    // (plain adds for the row sum: v_dot2 shares the matrix pipe and would serialise with the MFMAs)
-    float rs0 = 0.f, rs1 = 0.f;
-#pragma unroll
-    for (int v = 0; v < 16; v += 2) {
-      s[v] = fast_exp2(__builtin_fmaf(s[v], c, -m_use));
-      s[v + 1] = fast_exp2(__builtin_fmaf(s[v + 1], c, -m_use));
-      rs0 += s[v];
-      rs1 += s[v + 1];
-    }
-    l_run += rs0 + rs1;
-#pragma unroll
-    for (int hh = 0; hh < 2; hh++)
-      pf[hh] = pack8<T>(s[8 * hh + 0], s[8 * hh + 1], s[8 * hh + 2], s[8 * hh + 3], s[8 * hh + 4], s[8 * hh + 5],
-                        s[8 * hh + 6], s[8 * hh + 7]);
-  };
-
-  // One LDS tile.  Source order = intended overlap (each line is MFMA work next to independent VALU work):
-  //   S0 = K[0:32] Q^T                       | -
-  //   S1 = K[32:64] Q^T                      | exp(S0)
-  //   O += V[0:32]^T P0                      | exp(S1)
-  //   O += V[32:64]^T P1                     | transpose + LDS store of the next tile
-  // Fragments are read from LDS one phase ahead of their use.
+  // One LDS tile, laid out slot by slot (one MFMA per slot, a scheduling barrier after each): the LDS
+  // fragment of a slot is requested AHEAD slots earlier, so no phase starts by waiting out an LDS round trip,
+  // and the softmax arithmetic of one 32-row half is spread under the MFMAs that follow it:
+  //   slots   S0 = K[0:32] Q^T | S1 = K[32:64] Q^T | O += V[0:32]^T P0 | O += V[32:64]^T P1
+  //   VALU                     | max0, exp(S0)     | max1, exp(S1)     | (LDS store of the next tile after)
   auto tile_body = [&](auto masked_c, int t, int buf, bool has_next) {
     constexpr bool MASKED = decltype(masked_c)::value;
     const int kv0 = t * BN;
     const unsigned char* kl = smem + buf * BUF_BYTES;
     const unsigned char* vl = kl + K_BYTES;
     const int* sl = (const int*)(vl + V_BYTES);
-    auto kfrag = [&](int hf, int ks) { return *(const v8*)(kl + KT::off(hf * 32 + ln, 16 * ks + 8 * g)); };
-    auto vfrag = [&](int hf, int kk, int d) { return *(const v8*)(vl + TrTile64::chunk_off(d * 32 + ln, 2 * hf + kk, g)); };
     auto mask_half = [&](f32x16& s, int hf) {
 #pragma unroll
       for (int v = 0; v < 16; v++) {
@@ -275,41 +255,88 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
         s[v] = ok ? s[v] : -INFINITY;
       }
     };
-
-    v8 fr[KSTEPS > 2 * DVB ? KSTEPS : 2 * DVB];  // fragments of the current phase
-    f32x16 s0, s1;
+    constexpr int S1 = KSTEPS, PV0 = 2 * KSTEPS, PV1 = PV0 + 2 * DVB, NS = PV1 + 2 * DVB;
+    constexpr int AHEAD = 3, NF = 4;
+    v8 fr[NF];
+    f32x16 s[2];
+    v8 pf[2][2];
+    float alpha0 = 1.f, alpha1 = 1.f, rs0 = 0.f, rs1 = 0.f;
+    bool moved1 = false;
+    auto frag = [&](auto I) -> v8 {
+      constexpr int i = decltype(I)::value;
+      if constexpr (i < PV0) {
+        constexpr int hf = i / KSTEPS, ks = i % KSTEPS;
+        return *(const v8*)(kl + KT::off(hf * 32 + ln, 16 * ks + 8 * g));
+      } else {
+        constexpr int hf = (i - PV0) / (2 * DVB), j = (i - PV0) % (2 * DVB), kk = j / DVB, d = j % DVB;
+        return *(const v8*)(vl + TrTile64::chunk_off(d * 32 + ln, 2 * hf + kk, g));
+      }
+    };
+    auto mma = [&](auto I, const v8& f) {
+      constexpr int i = decltype(I)::value;
+      const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if constexpr (i < PV0) {
+        constexpr int hf = i / KSTEPS, ks = i % KSTEPS;
+        s[hf] = MT<T>::mfma32(f, qf[ks], ks == 0 ? zero : s[hf]);
+      } else {
+        constexpr int hf = (i - PV0) / (2 * DVB), j = (i - PV0) % (2 * DVB), kk = j / DVB, d = j % DVB;
+        oacc[d] = MT<T>::mfma32(f, pf[hf][kk], oacc[d]);
+      }
+    };
+    // exponentials of half HF: its 16 values spread over the LEN slots from START on (plain adds for the row
+    // sum: v_dot2 shares the matrix pipe and would serialise with the MFMAs)
+    auto exp_part = [&](auto I, auto HFc, auto STARTc, auto LENc) {
+      constexpr int i = decltype(I)::value, hf = decltype(HFc)::value, st = decltype(STARTc)::value, len = decltype(LENc)::value;
+      if constexpr (i >= st && i < st + len) {
+        constexpr int k = i - st, lo = (k * 16 + len - 1) / len, hi = ((k + 1) * 16 + len - 1) / len;
 #pragma unroll
-    for (int v = 0; v < 16; v++) { s0[v] = 0.f; s1[v] = 0.f; }
-    // phase 1
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) fr[ks] = kfrag(0, ks);
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) s0 = MT<T>::mfma32(fr[ks], qf[ks], s0);
-    if (MASKED) mask_half(s0, 0);
-    float alpha0, alpha1;
-    if (row_max_update(s0, alpha0)) rescale_o(alpha0);
-    // phase 2: S1 MFMAs next to exp(S0)
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) fr[ks] = kfrag(1, ks);
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) s1 = MT<T>::mfma32(fr[ks], qf[ks], s1);
-    v8 p0[2], p1[2];
-    exp_half(s0, p0);
-    if (MASKED) mask_half(s1, 1);
-    // P0 is relative to the reference max before this update: O is rescaled only after V0^T P0 is in it
-    const bool moved1 = row_max_update(s1, alpha1);
-    // phase 3: O += V0^T P0 next to exp(S1)
-#pragma unroll
-    for (int i = 0; i < 2 * DVB; i++) fr[i] = vfrag(0, i / DVB, i % DVB);
-#pragma unroll
-    for (int i = 0; i < 2 * DVB; i++) oacc[i % DVB] = MT<T>::mfma32(fr[i], p0[i / DVB], oacc[i % DVB]);
-    exp_half(s1, p1);
-    if (moved1) rescale_o(alpha1);
-    // phase 4: O += V1^T P1 next to the LDS store of the prefetched tile
-#pragma unroll
-    for (int i = 0; i < 2 * DVB; i++) fr[i] = vfrag(1, i / DVB, i % DVB);
-#pragma unroll
-    for (int i = 0; i < 2 * DVB; i++) oacc[i % DVB] = MT<T>::mfma32(fr[i], p1[i / DVB], oacc[i % DVB]);
+        for (int v = lo; v < hi; v++) {
+          float pv = fast_exp2(__builtin_fmaf(s[hf][v], c, -m_use));
+          asm volatile("" : "+v"(pv));  // keeps the computation in this slot
+          s[hf][v] = pv;
+          if (v & 1) rs1 += pv;
+          else rs0 += pv;
+        }
+        static_for<0, 2>([&](auto H) {
+          constexpr int hh = decltype(H)::value;
+          if constexpr (8 * hh + 8 > lo && 8 * hh + 8 <= hi) {
+            const f32x16& x = s[hf];
+            pf[hf][hh] = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4],
+                                  x[8 * hh + 5], x[8 * hh + 6], x[8 * hh + 7]);
+          }
+        });
+      }
+    };
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 1> I1;
+    static_for<0, AHEAD>([&](auto I) { fr[decltype(I)::value % NF] = frag(I); });
+    static_for<0, NS>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
+      mma(I, fr[i % NF]);
+      // one slot after the last MFMA of a half: mask, running max (the rare rescale of O is a wave-uniform
+      // branch), then the exponentials under the following MFMAs
+      if constexpr (i == S1) {
+        if (MASKED) mask_half(s[0], 0);
+        if (row_max_update(s[0], alpha0)) rescale_o(alpha0);
+      }
+      if constexpr (i == PV0) {
+        if (MASKED) mask_half(s[1], 1);
+        // half 0's row sums join l_run before the update can rescale it; P0 itself is relative to the
+        // reference max before this update: O is rescaled only after V0^T P0 is in it
+        l_run += rs0 + rs1;
+        rs0 = 0.f;
+        rs1 = 0.f;
+        moved1 = row_max_update(s[1], alpha1);
+      }
+      exp_part(I, I0{}, std::integral_constant<int, S1 + 1>{}, std::integral_constant<int, KSTEPS - 1>{});
+      exp_part(I, I1{}, std::integral_constant<int, PV0 + 1>{}, std::integral_constant<int, 2 * DVB - 1>{});
+      if constexpr (i == PV1 - 1) {
+        if (moved1) rescale_o(alpha1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    l_run += rs0 + rs1;
     if (has_next) store_tile(buf ^ 1);
   };
 
