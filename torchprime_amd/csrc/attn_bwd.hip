@@ -219,6 +219,13 @@ struct DmaTile {
     asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :: "s"(dst), "v"(vo[I]), "s"(rs), "s"(tile_byte_offset) : "memory");
   }
+  // same, with the wave's first LDS destination given as a scalar byte address (keeps the address
+  // arithmetic on the scalar unit)
+  template <int I>
+  __device__ __forceinline__ void issue_one_at(u32x4 rs, unsigned tile_byte_offset, unsigned wave_dst) const {
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(wave_dst + I * 1024), "v"(vo[I]), "s"(rs), "s"(tile_byte_offset) : "memory");
+  }
   __device__ __forceinline__ void issue(u32x4 rs, unsigned tile_byte_offset, unsigned char* lds_tile, int wave) const {
     tile_byte_offset = __builtin_amdgcn_readfirstlane(tile_byte_offset);
     if constexpr (PER_WAVE > 0) issue_one<0>(rs, tile_byte_offset, lds_tile, wave);
@@ -275,6 +282,10 @@ __device__ __forceinline__ void dma_dword(u32x4 rs, unsigned byte_offset, unsign
   byte_offset = __builtin_amdgcn_readfirstlane(byte_offset);
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, %3 offen lds"
                :: "s"(d), "v"((unsigned)lane * 4u), "s"(rs), "s"(byte_offset) : "memory");
+}
+__device__ __forceinline__ void dma_dword_at(u32x4 rs, unsigned byte_offset, unsigned dst, int lane) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+               :: "s"(dst), "v"((unsigned)lane * 4u), "s"(rs), "s"(byte_offset) : "memory");
 }
 // The same transposition as transpose_tile, cut into steps that can be placed between MFMAs: read() fetches
 // this thread's 4-row x 8-column block, write(J) stores column pair member J (0..7) as 8 bytes.  Threads
@@ -519,6 +530,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       fr[i % NF] = *(const v8*)(smem + faq[i]);
     });
     struct { u32x4 rq, ro, rr; unsigned offq, offo, offr; } nx;
+    const unsigned lds_base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)smem);
+    const unsigned wave_q = __builtin_amdgcn_readfirstlane((unsigned)(wave * QT::PER_WAVE * 1024));
+    const unsigned wave_o = __builtin_amdgcn_readfirstlane((unsigned)(wave * OT::PER_WAVE * 1024));
+    const unsigned wave_r = __builtin_amdgcn_readfirstlane((unsigned)(wave * BMQ * 4));
     int rslot = 0;
     for (int it = 0; it < n_iter; it++) {
       const int buf = it & 1;
@@ -535,6 +550,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       const float* deltal = lsel + BMQ;
       const int* segl = (const int*)(deltal + BMQ);
       const int rnext = rslot >= 1 ? rslot - 1 : 2;  // (it + 2) % 3, the slot tile t-1 used
+      // LDS destinations of this wave's loads of tile t+2 (scalar byte addresses)
+      const unsigned dma_q = lds_base + (unsigned)(buf * BUF_BYTES) + wave_q, dma_o = dma_q - wave_q + Q_BYTES + wave_o;
+      const unsigned dma_r = lds_base + (unsigned)(NBUF * BUF_BYTES + rnext * ROW_BYTES) + wave_r;
       // descriptors of tile t+2's loads (wave-uniform), issued piecewise in part 2.  The bases change with
       // the query head only; they are rebuilt when a new head starts (and when the tiles run out: size 0).
       if (it == 0 || n_idx == 0 || !issue_next) {
@@ -697,9 +715,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
             constexpr int m = (i - C0) / DMA_EVERY;
             // (no branch here: past the last tile the descriptors have size 0 and the loads deliver zeros
             // into buffers nobody reads any more)
-            if constexpr (m < QT::PER_WAVE) qdma.template issue_one<m>(nx.rq, nx.offq, bl, wave);
-            else if constexpr (m < QT::PER_WAVE + OT::PER_WAVE) dodma.template issue_one<m - QT::PER_WAVE>(nx.ro, nx.offo, bl + Q_BYTES, wave);
-            else dma_dword(nx.rr, nx.offr, rows_base + rnext * ROW_BYTES + wave * BMQ * 4, lane);
+            if constexpr (m < QT::PER_WAVE) qdma.template issue_one_at<m>(nx.rq, nx.offq, dma_q);
+            else if constexpr (m < QT::PER_WAVE + OT::PER_WAVE) dodma.template issue_one_at<m - QT::PER_WAVE>(nx.ro, nx.offo, dma_o);
+            else dma_dword_at(nx.rr, nx.offr, dma_r, lane);
           }
           if constexpr (COMPUTE) {
             if constexpr (i + 2 == 2 * K || i + 2 == 3 * K) {
