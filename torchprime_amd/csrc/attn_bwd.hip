@@ -296,16 +296,20 @@ struct TransposeSteps {
   static constexpr int CPR = D / 8, TOT = CPR * 16;
   static_assert(TOT <= 256, "one block per thread");
   u32x4 r[4];
-  unsigned rd, zs, wbase, y, sel_even, sel_odd;
-  __device__ __forceinline__ void init(int tid) {
+  unsigned rd, zs, wo[8], sel_even, sel_odd;
+  // bias: added to every store offset (write() is then given destinations less that amount: a caller whose
+  // transposed tiles lie beyond the reach of a 16-bit instruction offset keeps the excess in these registers)
+  __device__ __forceinline__ void init(int tid, unsigned bias) {
     const int item = tid % TOT, c8 = item % CPR, rqi = item / CPR;
     const int rq = (rqi & ~3) | ((rqi & 1) << 1) | ((rqi >> 1) & 1);
     rd = (unsigned)(4 * rq * DmaTile<D>::ROWB);
     zs = (unsigned)((c8 ^ DmaTile<D>::swz(4 * rq)) << 4);
     const int flip = c8 & 1;
     const int k = (((c8 & 1) << 2) ^ (c8 >> 1)) & 7, rqc = 2 * (rq >> 2) + (rq & 1);
-    wbase = (unsigned)(c8 * 8 * TrTile64::ROW_BYTES + (((rq >> 1) & 1) << 3));
-    y = (unsigned)((flip << 7) | ((rqc ^ k) << 4));
+    const unsigned wbase = (unsigned)(c8 * 8 * TrTile64::ROW_BYTES + (((rq >> 1) & 1) << 3));
+    const unsigned y = (unsigned)((flip << 7) | ((rqc ^ k) << 4));
+#pragma unroll
+    for (int j = 0; j < 8; j++) wo[j] = bias + wbase + (y ^ (unsigned)(((j & 1) << 7) | ((j >> 1) << 4)));
     sel_even = flip ? 0x07060302u : 0x05040100u;
     sel_odd = flip ? 0x05040100u : 0x07060302u;
   }
@@ -319,12 +323,11 @@ struct TransposeSteps {
   template <typename J>
   __device__ __forceinline__ void write(unsigned char* dst, J) const {
     constexpr int j = J::value, w = j >> 1;
-    constexpr unsigned cj = (unsigned)(((j & 1) << 7) | ((j >> 1) << 4));
     const unsigned sel = (j & 1) ? sel_odd : sel_even;
     u32x2 o;
     o.x = __builtin_amdgcn_perm(r[1][w], r[0][w], sel);
     o.y = __builtin_amdgcn_perm(r[3][w], r[2][w], sel);
-    *(u32x2*)(dst + wbase + (y ^ cj) + (j >> 1) * 2 * TrTile64::ROW_BYTES) = o;
+    *(u32x2*)(dst + wo[j] + (j >> 1) * 2 * TrTile64::ROW_BYTES) = o;
   }
 };
 
@@ -359,6 +362,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   constexpr int ROW_BYTES = BMQ * 4 * 4;  // lse (log2 units), delta, segment id per query row (+1 unused): 3 slots
   constexpr int BUF_BYTES = Q_BYTES + DO_BYTES + QTR_BYTES + DOTR_BYTES;
   constexpr bool PIPE = NBUF == 2 && DQK == DV && DQK <= 128;
+  // LDS layout: the NBUF copies of each kind of tile lie side by side (Q.. dO.. Q^T.. dO^T.., then the row
+  // vectors), so that with the buffer index a constant every fragment address is a loop-invariant per-lane
+  // offset plus an immediate
+  constexpr int Q_AT = 0, DO_AT = NBUF * Q_BYTES, QTR_AT = DO_AT + NBUF * DO_BYTES, DOTR_AT = QTR_AT + NBUF * QTR_BYTES;
 
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -435,10 +442,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   auto issue_tile = [&](int hl, int idx, int buf, int rslot) {
     const int hq = hk * a.n_rep + hl;
     const int qt = qtile_of(idx);
-    unsigned char* base = smem + buf * BUF_BYTES;
-    qdma.issue(make_rsrc_words((const T*)a.q + b * a.qs[0] + hq * a.qs[1], q_span), (unsigned)qt * q_tile_bytes, base, wave);
+    qdma.issue(make_rsrc_words((const T*)a.q + b * a.qs[0] + hq * a.qs[1], q_span), (unsigned)qt * q_tile_bytes,
+               smem + Q_AT + buf * Q_BYTES, wave);
     dodma.issue(make_rsrc_words((const T*)a.dout + b * a.dos[0] + hq * a.dos[1], do_span), (unsigned)qt * do_tile_bytes,
-                base + Q_BYTES, wave);
+                smem + DO_AT + buf * DO_BYTES, wave);
     // waves 0..2 fetch one 64-entry row vector each: 4 bytes per lane, rows past Sq arrive as zeros
     const int64_t ro = ((int64_t)b * a.Hq + hq) * Sq;
     const void* src = wave == 0 ? (const void*)(lse2 + ro) : wave == 1 ? (const void*)(a.delta + ro) : (const void*)segb;
@@ -501,19 +508,27 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     int c_hl = 0, c_idx = 0, n_hl = 0, n_idx = 0;  // tile being computed, tile whose loads are issued next
     TransposeSteps<DQK> trq;
     TransposeSteps<DV> tro;
-    trq.init(tid);
-    tro.init(tid);
+    // offsets into the transposed tiles carry TR_BIAS in their registers (an opaque value: the compiler would
+    // otherwise fold it back into constants too large for an instruction offset and add it at every use)
+    constexpr int TR_BIAS = QTR_AT;
+    unsigned tr_bias = (unsigned)TR_BIAS;
+    asm volatile("" : "+v"(tr_bias));
+    trq.init(tid, tr_bias);
+    tro.init(tid, tr_bias);
+    unsigned tb[4];
+#pragma unroll
+    for (int m = 0; m < 4; m++) tb[m] = ta[m] + tr_bias;
     if (n_iter > 0) { issue_tile(n_hl, n_idx, 0, 0); advance(n_hl, n_idx); }
     if (n_iter > 1) { issue_tile(n_hl, n_idx, 1, 1); advance(n_hl, n_idx); }
     // all earlier loads (the K/V fragments, the first tiles) have landed
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (n_iter > 0) {
-      trq.read(smem);
-      tro.read(smem + Q_BYTES);
+      trq.read(smem + Q_AT);
+      tro.read(smem + DO_AT);
       static_for<0, 8>([&](auto J) {
-        trq.write(smem + Q_BYTES + DO_BYTES, J);
-        tro.write(smem + Q_BYTES + DO_BYTES + QTR_BYTES, J);
+        trq.write(smem + (QTR_AT - TR_BIAS), J);
+        tro.write(smem + (DOTR_AT - TR_BIAS), J);
       });
     }
     __syncthreads();
@@ -527,7 +542,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     static_for<0, AHEAD>([&](auto I) {
       constexpr int i = decltype(I)::value;
       static_assert(AHEAD <= KS_QK, "the carried fragments all belong to S of the first query block");
-      fr[i % NF] = *(const v8*)(smem + faq[i]);
+      fr[i % NF] = *(const v8*)(smem + Q_AT + faq[i]);
     });
     struct { u32x4 rq, ro, rr; unsigned offq, offo, offr; } nx;
     const unsigned lds_base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)smem);
@@ -535,23 +550,28 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     const unsigned wave_o = __builtin_amdgcn_readfirstlane((unsigned)(wave * OT::PER_WAVE * 1024));
     const unsigned wave_r = __builtin_amdgcn_readfirstlane((unsigned)(wave * BMQ * 4));
     int rslot = 0;
-    for (int it = 0; it < n_iter; it++) {
-      const int buf = it & 1;
+    // one query tile; the buffer index is a constant (the loop below alternates two copies of this)
+    auto iteration = [&](auto BUFc, const int it) {
+      constexpr int buf = decltype(BUFc)::value;
       const int qi0 = qtile_of(c_idx) * BMQ;
       const int mode = tile_mode(c_idx, qi0);
       const bool issue_next = it + 2 < n_iter;
-      unsigned char* const bl = smem + buf * BUF_BYTES;
-      unsigned char* const bn = smem + (buf ^ 1) * BUF_BYTES;
-      const unsigned char* ql = bl;
-      const unsigned char* dol = ql + Q_BYTES;
-      const unsigned char* qtl = dol + DO_BYTES;
-      const unsigned char* dotl = qtl + QTR_BYTES;
+      const unsigned char* ql = smem + Q_AT + buf * Q_BYTES;
+      const unsigned char* dol = smem + DO_AT + buf * DO_BYTES;
+      const unsigned char* qtl = smem + (QTR_AT + buf * QTR_BYTES - TR_BIAS);     // + tb[]
+      const unsigned char* dotl = smem + (DOTR_AT + buf * DOTR_BYTES - TR_BIAS);  // + tb[]
+      // tile t+1 (being transposed, then read first in the next iteration) lives in the other buffer
+      unsigned char* const nxq = smem + Q_AT + (buf ^ 1) * Q_BYTES;
+      unsigned char* const nxdo = smem + DO_AT + (buf ^ 1) * DO_BYTES;
+      unsigned char* const nxqt = smem + (QTR_AT + (buf ^ 1) * QTR_BYTES - TR_BIAS);
+      unsigned char* const nxdot = smem + (DOTR_AT + (buf ^ 1) * DOTR_BYTES - TR_BIAS);
       const float* lsel = (const float*)(rows_base + rslot * ROW_BYTES);
       const float* deltal = lsel + BMQ;
       const int* segl = (const int*)(deltal + BMQ);
       const int rnext = rslot >= 1 ? rslot - 1 : 2;  // (it + 2) % 3, the slot tile t-1 used
       // LDS destinations of this wave's loads of tile t+2 (scalar byte addresses)
-      const unsigned dma_q = lds_base + (unsigned)(buf * BUF_BYTES) + wave_q, dma_o = dma_q - wave_q + Q_BYTES + wave_o;
+      const unsigned dma_q = lds_base + (unsigned)(Q_AT + buf * Q_BYTES) + wave_q;
+      const unsigned dma_o = lds_base + (unsigned)(DO_AT + buf * DO_BYTES) + wave_o;
       const unsigned dma_r = lds_base + (unsigned)(NBUF * BUF_BYTES + rnext * ROW_BYTES) + wave_r;
       // descriptors of tile t+2's loads (wave-uniform), issued piecewise in part 2.  The bases change with
       // the query head only; they are rebuilt when a new head starts (and when the tiles run out: size 0).
@@ -615,7 +635,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
           } else {
             constexpr int ph = (i - C0) / CL, qb = ph / 2, j = (i - C0) % CL, hh = j / DVB, d = j % DVB;
             const unsigned char* base = (ph % 2 == 0) ? dotl : qtl;
-            return *(const v8*)(base + ta[(2 * qb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+            return *(const v8*)(base + tb[(2 * qb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
           }
         };
         auto mma = [&](auto I, const v8& f) {
@@ -688,15 +708,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         // transposition of tile t+1 (buffer bn), one step per slot from slot C0 on
         auto transpose_step = [&](auto I) {
           constexpr int i = decltype(I)::value;
-          if constexpr (i == TQ0) trq.read(bn);
-          if constexpr (i == TO0) tro.read(bn + Q_BYTES);
+          if constexpr (i == TQ0) trq.read(nxq);
+          if constexpr (i == TO0) tro.read(nxdo);
           if constexpr (i >= TQ0 + 2 && i < TQ0 + 2 + 8 / WPS)
             static_for<0, WPS>([&](auto W) {
-              trq.write(bn + Q_BYTES + DO_BYTES, std::integral_constant<int, (i - TQ0 - 2) * WPS + decltype(W)::value>{});
+              trq.write(nxqt, std::integral_constant<int, (i - TQ0 - 2) * WPS + decltype(W)::value>{});
             });
           if constexpr (i >= TO0 + 2 && i < TO0 + 2 + 8 / WPS)
             static_for<0, WPS>([&](auto W) {
-              tro.write(bn + Q_BYTES + DO_BYTES + QTR_BYTES, std::integral_constant<int, (i - TO0 - 2) * WPS + decltype(W)::value>{});
+              tro.write(nxdot, std::integral_constant<int, (i - TO0 - 2) * WPS + decltype(W)::value>{});
             });
         };
         typedef std::integral_constant<int, 0> I0;
@@ -737,7 +757,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         });
         static_for<0, AHEAD>([&](auto I) {
           constexpr int i = decltype(I)::value;
-          fr[i % NF] = *(const v8*)(bn + faq[i]);
+          fr[i % NF] = *(const v8*)(nxq + faq[i]);
         });
       };
       if (mode == 1) body(std::integral_constant<int, 1>{});
@@ -747,6 +767,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       if (issue_next) advance(n_hl, n_idx);
       advance(c_hl, c_idx);
       rslot = rslot == 2 ? 0 : rslot + 1;
+    };
+    for (int it = 0; it < n_iter; it += 2) {
+      iteration(std::integral_constant<int, 0>{}, it);
+      if (it + 1 < n_iter) iteration(std::integral_constant<int, 1>{}, it + 1);
     }
   } else {
     // Wide heads: one buffer, and the register file does not hold the staggered schedule: the next tile is
@@ -756,8 +780,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       issue_tile(hl, idx, 0, 0);
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
-      transpose_tile<DQK>(smem, smem + Q_BYTES + DO_BYTES, tid);
-      transpose_tile<DV>(smem + Q_BYTES, smem + Q_BYTES + DO_BYTES + QTR_BYTES, tid);
+      transpose_tile<DQK>(smem + Q_AT, smem + QTR_AT, tid);
+      transpose_tile<DV>(smem + DO_AT, smem + DOTR_AT, tid);
       __syncthreads();
     };
     if (n_iter > 0) stage(0, 0);
@@ -765,10 +789,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       const int qi0 = qtile_of(c_idx) * BMQ;
       const int mode = tile_mode(c_idx, qi0);
       const bool need_mask = mode == 2;
-      const unsigned char* ql = smem;
-      const unsigned char* dol = ql + Q_BYTES;
-      const unsigned char* qtl = dol + DO_BYTES;
-      const unsigned char* dotl = qtl + QTR_BYTES;
+      const unsigned char* ql = smem + Q_AT;
+      const unsigned char* dol = smem + DO_AT;
+      const unsigned char* qtl = smem + QTR_AT;
+      const unsigned char* dotl = smem + DOTR_AT;
       const float* lsel = (const float*)rows_base;
       const float* deltal = lsel + BMQ;
       const int* segl = (const int*)(deltal + BMQ);
