@@ -922,7 +922,11 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   typedef RowTile<DQK> KT;
   typedef RowTile<DV> VT;
   constexpr int K_BYTES = BN * KT::STRIDE, V_BYTES = BN * VT::STRIDE, KTR_BYTES = DQK * TrTile64::ROW_BYTES;
-  constexpr int BUF_BYTES = K_BYTES + V_BYTES + KTR_BYTES + BN * 4;
+  // LDS: two row-major K/V buffers, NKTR transposed K tiles (three with 8 waves: the dQ MFMAs of a tile's
+  // second kv block run in the next iteration), two segment-id rows, then the per-tile id ranges
+  constexpr int NKTR = NW == 8 ? 3 : 2;
+  constexpr int KV_BYTES = K_BYTES + V_BYTES;
+  constexpr int KTR_AT = 2 * KV_BYTES, SEG_AT = KTR_AT + NKTR * KTR_BYTES, META_AT = SEG_AT + 2 * BN * 4;
 
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -958,7 +962,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   const float ndelta_s = a.delta[ro];  // -rowsum(dO o O)
   const int segq = SEG ? segb[qrow_c] : 0;
 
-  int* kvmin = (int*)(smem + 2 * BUF_BYTES);
+  int* kvmin = (int*)(smem + META_AT);
   int* kvmax = kvmin + ntiles;
   int* active = kvmax + ntiles;
   int* bq = active + ntiles;
@@ -1010,7 +1014,9 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
       vst.load(vrs, (unsigned)t * v_tile_bytes, stid);
     } else {
       // same registers for either role (the offsets and the resource are picked, not the code path)
-      const bool sk = stages_k(it);
+      // (a scalar choice: with the descriptor in vector registers every load would sit in a loop over its
+      // distinct values)
+      const bool sk = __builtin_amdgcn_readfirstlane((int)stages_k(it)) != 0;
       const rsrc_t rs = sk ? krs : vrs;
       const unsigned off = sk ? (unsigned)t * k_tile_bytes : (unsigned)t * v_tile_bytes;
 #pragma unroll
@@ -1018,19 +1024,21 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
     }
     if (SEG && tid < BN) sreg = segb[min(t * BN + tid, Skv - 1)];
   };
-  auto store_tile = [&](int buf, int it) {
-    unsigned char* base = smem + buf * BUF_BYTES;
+  // (kslot: which transposed tile; the row-major buffer is buf)
+  auto store_tile = [&](int buf, int kslot, int it) {
+    unsigned char* base = smem + buf * KV_BYTES;
+    unsigned char* ktr = smem + KTR_AT + kslot * KTR_BYTES;
     if (NW == 4) {
       kst.store_rowmajor(base, stid);
       vst.store_rowmajor(base + K_BYTES, stid);
-      kst.store_transposed(base + K_BYTES + V_BYTES, stid);
+      kst.store_transposed(ktr, stid);
     } else if (stages_k(it)) {
       kst.store_rowmajor(base, stid);
-      kst.store_transposed(base + K_BYTES + V_BYTES, stid);
+      kst.store_transposed(ktr, stid);
     } else {
       kst.store_rowmajor(base + K_BYTES, stid);  // K and V tiles have the same shape here
     }
-    if (SEG && tid < BN) ((int*)(base + K_BYTES + V_BYTES + KTR_BYTES))[tid] = sreg;
+    if (SEG && tid < BN) ((int*)(smem + SEG_AT + buf * BN * 4))[tid] = sreg;
   };
 
   unsigned ta[4];  // per-lane byte offsets of the K^T fragments (swizzle resolved once)
@@ -1048,147 +1056,309 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
 
   if (nact > 0) {
     load_tile(SEG ? active[0] : 0, 0);
-    store_tile(0, 0);
+    store_tile(0, 0, 0);
   }
   __builtin_amdgcn_s_waitcnt(0);  // Q / dO fragments, LSE and delta have landed (see the dK/dV kernel)
   __syncthreads();
 
-  for (int it = 0; it < nact; it++) {
-    const int t = SEG ? active[it] : it;
-    const int kv0 = t * BN;
-    const int buf = it & 1;
-    if (it + 1 < nact) load_tile(SEG ? active[it + 1] : it + 1, it);
-
-    const unsigned char* kl = smem + buf * BUF_BYTES;
-    const unsigned char* vl = kl + K_BYTES;
-    const unsigned char* ktl = vl + V_BYTES;
-    const int* sl = (const int*)(ktl + KTR_BYTES);
-
-    bool skip = CAUSAL && kv0 > wq_last;
-    bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0);
-    if (SEG) {
-      const int lo = kvmin[t], hi = kvmax[t];
-      skip = skip || hi < wqmin || lo > wqmax;
-      need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
-    }
-    // The tile body is laid out slot by slot (one MFMA each, a scheduling barrier after every slot): the
-    // LDS fragment of a slot is requested AHEAD slots earlier, and the element-wise work that turns
-    // S^T, dP^T into the 16-bit operand dS^T is spread under the MFMAs of the following slots.
-    //   slots   S0^T = K0 Q^T alternating with dP0^T = V0 dO^T;  S1^T with dP1^T;
-    //           dQ^T += K0^T dS0^T;  dQ^T += K1^T dS1^T (first the half whose operand is ready first)
-    //   VALU    dS0^T under S1^T/dP1^T; dS1^T under the dQ^T slots that do not need it yet
-    auto body = [&](auto masked_c) {
-      constexpr bool MASKED = decltype(masked_c)::value;
-      // 4 waves: S/dP of both kv blocks first, so that dS of block 0 has the MFMAs of block 1 next to it.
-      // 8 waves: block by block (S/dP, dS, dQ), which keeps one pair of 32x32 tiles live; the other wave on
-      // the SIMD supplies the overlap.
-      constexpr bool STAG = NW == 4;
-      constexpr int L1 = KS_QK + KS_DV, A2 = 2 * DKB, NS = 2 * L1 + 2 * A2;
-      constexpr int AB1 = STAG ? L1 : L1 + A2;          // first slot of S1/dP1
-      constexpr int ACC0 = STAG ? 2 * L1 : L1;          // first slot of dQ += K0^T dS0
-      constexpr int ACC1 = 2 * L1 + A2;                 // first slot of dQ += K1^T dS1
-      constexpr int AHEAD = 3, NF = 4;
-      v8 fr[NF];
-      f32x16 s[2], dp[2];
-      v8 df[2][2];
-      auto frag = [&](auto I) -> v8 {
-        constexpr int i = decltype(I)::value;
-        constexpr bool is_acc = (i >= ACC0 && i < ACC0 + A2) || i >= ACC1;
-        if constexpr (!is_acc) {
-          constexpr int nb = i >= AB1 ? 1 : 0;
-          constexpr AbSlot sl = ab_slot(nb ? i - AB1 : i, KS_QK, KS_DV);
-          if constexpr (sl.kind == 0) return *(const v8*)(kl + KT::off(nb * 32 + ln, 16 * sl.k + 8 * g));
-          else return *(const v8*)(vl + VT::off(nb * 32 + ln, 16 * sl.k + 8 * g));
-        } else {
-          constexpr int nb = i >= ACC1 ? 1 : 0, j = nb ? i - ACC1 : i - ACC0, hh = j / DKB, d = j % DKB;
-          return *(const v8*)(ktl + ta[(2 * nb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
-        }
-      };
-      auto mma = [&](auto I, const v8& f) {
-        constexpr int i = decltype(I)::value;
-        constexpr bool is_acc = (i >= ACC0 && i < ACC0 + A2) || i >= ACC1;
-        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        if constexpr (!is_acc) {
-          constexpr int nb = i >= AB1 ? 1 : 0;
-          constexpr AbSlot sl = ab_slot(nb ? i - AB1 : i, KS_QK, KS_DV);
-          if constexpr (sl.kind == 0) s[nb] = MT<T>::mfma32(f, qf[sl.k], sl.k == 0 ? zero : s[nb]);
-          else dp[nb] = MT<T>::mfma32(f, dof[sl.k], sl.k == 0 ? zero : dp[nb]);
-        } else {
-          constexpr int nb = i >= ACC1 ? 1 : 0, j = nb ? i - ACC1 : i - ACC0, hh = j / DKB, d = j % DKB;
-          dqacc[d] = MT<T>::mfma32(f, df[nb][hh], dqacc[d]);
-        }
-      };
-      // elements [E0, E0 + N) of block NB spread evenly over the LEN slots starting at START
-      auto valu = [&](auto I, auto NBc, auto E0c, auto Nc, auto STARTc, auto LENc) {
-        constexpr int i = decltype(I)::value, nb = decltype(NBc)::value, e0 = decltype(E0c)::value, n = decltype(Nc)::value,
-                      st = decltype(STARTc)::value, len = decltype(LENc)::value;
-        if constexpr (i >= st && i < st + len) {
-          constexpr int k = i - st, lo = e0 + (k * n + len - 1) / len, hi = e0 + ((k + 1) * n + len - 1) / len;
+  if constexpr (NW == 8) {
+    // Eight waves (two per SIMD).  A wave's VALU work runs beside its own MFMAs only when the two are mixed
+    // finely: a run of back-to-back MFMAs holds up the vector issue port of the SIMD, the other wave's
+    // included.  So the element-wise work is cut into pieces of a few instructions, one per slot, and the
+    // slots are ordered so that every piece has its inputs a slot or more before it runs:
+    //   slots   S0 = K0 Q^T | dQ += K1'^T dS1' | dP0 = V0 dO^T | S1 = K1 Q^T | dQ += K0^T dS0 | dP1 = V1 dO^T
+    //   VALU    dS1'        | P0 ..............................| dS0         | P1 ...........................
+    // (primed: second kv block of the tile before, whose P and dP are carried over in s[1], dp[1]; its
+    // transposed K tile is still in LDS, which is why there are three of them).  A wave that skips a tile,
+    // and the end of the loop, finish the carried block on their own (drain).
+    constexpr int A2 = 2 * DKB;
+    constexpr int P1 = KS_QK, P2 = P1 + A2, P3 = P2 + KS_DV, P4 = P3 + KS_QK, P5 = P4 + A2, NS = P5 + KS_DV;
+    constexpr int LEN_P = A2 + KS_DV - 1;  // slots of a P group (starts one slot after its S is complete)
+    constexpr int AHEAD = 3, NF = 4;
+    f32x16 s[2], dp[2];
 #pragma unroll
-          for (int v = lo; v < hi; v++) {
-            float pv = fast_exp2(__builtin_fmaf(s[nb][v], c, -lse_s));
-            if (MASKED) {
-              const int kvl = nb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
-              const int kv = kv0 + kvl;
-              const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
-              pv = ok ? pv : 0.f;
-            }
-            float dsv = pv * (dp[nb][v] + ndelta_s);
-            asm volatile("" : "+v"(dsv));  // keeps the computation in this slot
-            dp[nb][v] = dsv;
-          }
-          static_for<0, 2>([&](auto H) {  // every half whose eighth value was produced in this slot
-            constexpr int hh = decltype(H)::value;
-            if constexpr (8 * hh + 8 > lo && 8 * hh + 8 <= hi) {
-              const f32x16& x = dp[nb];
-              df[nb][hh] = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4],
-                                    x[8 * hh + 5], x[8 * hh + 6], x[8 * hh + 7]);
-            }
-          });
-        }
-      };
-      typedef std::integral_constant<int, 0> I0;
-      typedef std::integral_constant<int, 1> I1;
-      typedef std::integral_constant<int, 8> I8;
-      typedef std::integral_constant<int, 16> I16;
-      static_for<0, AHEAD>([&](auto I) { fr[decltype(I)::value % NF] = frag(I); });
-      static_for<0, NS>([&](auto I) {
-        constexpr int i = decltype(I)::value;
-        if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
-        if constexpr (!STAG) {
-          // whole dS of a block right before the dQ slots that consume it
-          valu(I, I0{}, I0{}, I16{}, std::integral_constant<int, ACC0>{}, I1{});
-          valu(I, I1{}, I0{}, I16{}, std::integral_constant<int, ACC1>{}, I1{});
-        }
-        mma(I, fr[i % NF]);
-        if constexpr (!STAG) {
-          // the next tile (requested at the top of this one) goes to the other buffer under the last MFMAs
-          // instead of in a phase of its own; after the last tile this stores stale registers nobody reads
-          constexpr int ST0 = NS - 12;
-          unsigned char* nb_base = smem + (buf ^ 1) * BUF_BYTES;
-          if constexpr (i == ST0) kst.store_rowmajor(nb_base + (wave < 4 ? 0 : K_BYTES), stid);
-          if constexpr (i >= ST0 + 2 && i < ST0 + 10) {
-            if (wave < 4) kst.template store_transposed_step<i - ST0 - 2>(nb_base + K_BYTES + V_BYTES, stid);
-          }
-        }
-        if constexpr (STAG) {
-          valu(I, I0{}, I0{}, I16{}, std::integral_constant<int, L1>{}, std::integral_constant<int, L1>{});
-          valu(I, I1{}, I0{}, I8{}, std::integral_constant<int, ACC0>{}, std::integral_constant<int, 2 * DKB>{});
-          valu(I, I1{}, I8{}, I8{}, std::integral_constant<int, ACC1>{}, std::integral_constant<int, DKB>{});
-        }
-        __builtin_amdgcn_sched_barrier(0);
+    for (int v = 0; v < 16; v++) { s[1][v] = 0.f; dp[1][v] = 0.f; }
+    // the first tile's carried block is all zeros: its K^T operand must be finite
+    for (int o = tid * 16; o < KTR_BYTES; o += 64 * NW * 16) *(u32x4*)(smem + KTR_AT + 2 * KTR_BYTES + o) = u32x4{0u, 0u, 0u, 0u};
+    __syncthreads();
+
+    // dS of elements [LO, HI) of a block: d <- p (d - delta); a half is packed once its eight values are there
+    auto ds_chunk = [&](auto LOc, auto HIc, const f32x16& p, f32x16& d, v8* dfb) {
+      constexpr int lo = decltype(LOc)::value, hi = decltype(HIc)::value;
+#pragma unroll
+      for (int v = lo; v < hi; v++) {
+        float dsv = p[v] * (d[v] + ndelta_s);
+        asm volatile("" : "+v"(dsv));  // keeps the computation in its slot
+        d[v] = dsv;
+      }
+      static_for<0, 2>([&](auto H) {
+        constexpr int hh = decltype(H)::value;
+        if constexpr (8 * hh + 8 > lo && 8 * hh + 8 <= hi)
+          dfb[hh] = pack8<T>(d[8 * hh + 0], d[8 * hh + 1], d[8 * hh + 2], d[8 * hh + 3], d[8 * hh + 4], d[8 * hh + 5],
+                             d[8 * hh + 6], d[8 * hh + 7]);
       });
     };
-    if (!skip) {
-      if (need_mask) body(std::true_type{});
-      else body(std::false_type{});
+    // finishes the carried block without a tile around it
+    auto drain = [&](const unsigned char* ktp) {
+      v8 d1[2];
+      ds_chunk(std::integral_constant<int, 0>{}, std::integral_constant<int, 16>{}, s[1], dp[1], d1);
+#pragma unroll
+      for (int j = 0; j < A2; j++) {
+        const int hh = j / DKB, d = j % DKB;
+        const v8 f = *(const v8*)(ktp + ta[(2 + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+        dqacc[d] = MT<T>::mfma32(f, d1[hh], dqacc[d]);
+      }
+#pragma unroll
+      for (int v = 0; v < 16; v++) { s[1][v] = 0.f; dp[1][v] = 0.f; }
+    };
+
+    bool pending = false;
+    int kslot = 0;
+    for (int it = 0; it < nact; it++) {
+      const int t = SEG ? active[it] : it;
+      const int kv0 = t * BN;
+      const int buf = it & 1;
+      if (it + 1 < nact) load_tile(SEG ? active[it + 1] : it + 1, it);
+      const int kprev = kslot == 0 ? 2 : kslot - 1, knext = kslot == 2 ? 0 : kslot + 1;
+      const unsigned char* kl = smem + buf * KV_BYTES;
+      const unsigned char* vl = kl + K_BYTES;
+      const unsigned char* ktl = smem + KTR_AT + kslot * KTR_BYTES;
+      const unsigned char* ktp = smem + KTR_AT + kprev * KTR_BYTES;
+      const int* sl = (const int*)(smem + SEG_AT + buf * BN * 4);
+
+      bool skip = CAUSAL && kv0 > wq_last;
+      bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0);
+      if (SEG) {
+        const int lo = kvmin[t], hi = kvmax[t];
+        skip = skip || hi < wqmin || lo > wqmax;
+        need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
+      }
+      auto body = [&](auto masked_c) {
+        constexpr bool MASKED = decltype(masked_c)::value;
+        v8 fr[NF];
+        v8 df0[2], df1[2];
+        auto frag = [&](auto I) -> v8 {
+          constexpr int i = decltype(I)::value;
+          if constexpr (i < P1) return *(const v8*)(kl + KT::off(ln, 16 * i + 8 * g));
+          else if constexpr (i < P2) {
+            constexpr int j = i - P1, hh = j / DKB, d = j % DKB;
+            return *(const v8*)(ktp + ta[(2 + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+          } else if constexpr (i < P3) return *(const v8*)(vl + VT::off(ln, 16 * (i - P2) + 8 * g));
+          else if constexpr (i < P4) return *(const v8*)(kl + KT::off(32 + ln, 16 * (i - P3) + 8 * g));
+          else if constexpr (i < P5) {
+            constexpr int j = i - P4, hh = j / DKB, d = j % DKB;
+            return *(const v8*)(ktl + ta[hh ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+          } else return *(const v8*)(vl + VT::off(32 + ln, 16 * (i - P5) + 8 * g));
+        };
+        auto mma = [&](auto I, const v8& f) {
+          constexpr int i = decltype(I)::value;
+          const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          if constexpr (i < P1) s[0] = MT<T>::mfma32(f, qf[i], i == 0 ? zero : s[0]);
+          else if constexpr (i < P2) dqacc[(i - P1) % DKB] = MT<T>::mfma32(f, df1[(i - P1) / DKB], dqacc[(i - P1) % DKB]);
+          else if constexpr (i < P3) dp[0] = MT<T>::mfma32(f, dof[i - P2], i == P2 ? zero : dp[0]);
+          else if constexpr (i < P4) s[1] = MT<T>::mfma32(f, qf[i - P3], i == P3 ? zero : s[1]);
+          else if constexpr (i < P5) dqacc[(i - P4) % DKB] = MT<T>::mfma32(f, df0[(i - P4) / DKB], dqacc[(i - P4) % DKB]);
+          else dp[1] = MT<T>::mfma32(f, dof[i - P5], i == P5 ? zero : dp[1]);
+        };
+        // piece K of LEN of a 16-element group
+        auto ds_piece = [&](auto I, auto STARTc, const f32x16& p, f32x16& d, v8* dfb) {
+          constexpr int i = decltype(I)::value, st = decltype(STARTc)::value, len = KS_QK;
+          if constexpr (i >= st && i < st + len) {
+            constexpr int k = i - st, lo = (k * 16 + len - 1) / len, hi = ((k + 1) * 16 + len - 1) / len;
+            ds_chunk(std::integral_constant<int, lo>{}, std::integral_constant<int, hi>{}, p, d, dfb);
+          }
+        };
+        auto p_piece = [&](auto I, auto STARTc, auto NBc, f32x16& sv) {
+          constexpr int i = decltype(I)::value, st = decltype(STARTc)::value, nb = decltype(NBc)::value, len = LEN_P;
+          if constexpr (i >= st && i < st + len) {
+            constexpr int k = i - st, lo = (k * 16 + len - 1) / len, hi = ((k + 1) * 16 + len - 1) / len;
+#pragma unroll
+            for (int v = lo; v < hi; v++) {
+              float pv = fast_exp2(__builtin_fmaf(sv[v], c, -lse_s));
+              if (MASKED) {
+                const int kvl = nb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
+                const int kv = kv0 + kvl;
+                const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
+                pv = ok ? pv : 0.f;
+              }
+              asm volatile("" : "+v"(pv));
+              sv[v] = pv;
+            }
+          }
+        };
+        typedef std::integral_constant<int, 0> I0;
+        typedef std::integral_constant<int, 1> I1;
+        static_for<0, AHEAD>([&](auto I) { fr[decltype(I)::value % NF] = frag(I); });
+        static_for<0, NS>([&](auto I) {
+          constexpr int i = decltype(I)::value;
+          if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
+          mma(I, fr[i % NF]);
+          ds_piece(I, std::integral_constant<int, 1>{}, s[1], dp[1], df1);
+          p_piece(I, std::integral_constant<int, P1 + 1>{}, I0{}, s[0]);
+          ds_piece(I, std::integral_constant<int, P3 + 1>{}, s[0], dp[0], df0);
+          p_piece(I, std::integral_constant<int, P4 + 1>{}, I1{}, s[1]);
+          // the next tile (requested at the top of this one) goes to LDS under the last MFMAs; after the last
+          // tile this stores stale registers nobody reads
+          constexpr int ST0 = NS - 12;
+          if constexpr (i == ST0) kst.store_rowmajor(smem + (buf ^ 1) * KV_BYTES + (wave < 4 ? 0 : K_BYTES), stid);
+          if constexpr (i >= ST0 + 2 && i < ST0 + 10) {
+            if (wave < 4) kst.template store_transposed_step<i - ST0 - 2>(smem + KTR_AT + knext * KTR_BYTES, stid);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      };
+      if (!skip) {
+        if (need_mask) body(std::true_type{});
+        else body(std::false_type{});
+        pending = true;
+        if (SEG && tid < BN) ((int*)(smem + SEG_AT + (buf ^ 1) * BN * 4))[tid] = sreg;
+      } else {
+        if (pending) { drain(ktp); pending = false; }
+        if (it + 1 < nact) store_tile(buf ^ 1, knext, it);
+      }
+      __syncthreads();
+      kslot = knext;
     }
-    if (NW == 4 || skip) {
-      if (it + 1 < nact) store_tile(buf ^ 1, it);
-    } else if (SEG && tid < BN) {
-      ((int*)(smem + (buf ^ 1) * BUF_BYTES + K_BYTES + V_BYTES + KTR_BYTES))[tid] = sreg;
+    if (pending) drain(smem + KTR_AT + (kslot == 0 ? 2 : kslot - 1) * KTR_BYTES);
+  } else {
+  for (int it = 0; it < nact; it++) {
+      const int t = SEG ? active[it] : it;
+      const int kv0 = t * BN;
+      const int buf = it & 1;
+      if (it + 1 < nact) load_tile(SEG ? active[it + 1] : it + 1, it);
+  
+      const unsigned char* kl = smem + buf * KV_BYTES;
+      const unsigned char* vl = kl + K_BYTES;
+      const unsigned char* ktl = smem + KTR_AT + buf * KTR_BYTES;
+      const int* sl = (const int*)(smem + SEG_AT + buf * BN * 4);
+  
+      bool skip = CAUSAL && kv0 > wq_last;
+      bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0);
+      if (SEG) {
+        const int lo = kvmin[t], hi = kvmax[t];
+        skip = skip || hi < wqmin || lo > wqmax;
+        need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
+      }
+      // The tile body is laid out slot by slot (one MFMA each, a scheduling barrier after every slot): the
+      // LDS fragment of a slot is requested AHEAD slots earlier, and the element-wise work that turns
+      // S^T, dP^T into the 16-bit operand dS^T is spread under the MFMAs of the following slots.
+      //   slots   S0^T = K0 Q^T alternating with dP0^T = V0 dO^T;  S1^T with dP1^T;
+      //           dQ^T += K0^T dS0^T;  dQ^T += K1^T dS1^T (first the half whose operand is ready first)
+      //   VALU    dS0^T under S1^T/dP1^T; dS1^T under the dQ^T slots that do not need it yet
+      auto body = [&](auto masked_c) {
+        constexpr bool MASKED = decltype(masked_c)::value;
+        // 4 waves: S/dP of both kv blocks first, so that dS of block 0 has the MFMAs of block 1 next to it.
+        // 8 waves: block by block (S/dP, dS, dQ), which keeps one pair of 32x32 tiles live; the other wave on
+        // the SIMD supplies the overlap.
+        constexpr bool STAG = NW == 4;
+        constexpr int L1 = KS_QK + KS_DV, A2 = 2 * DKB, NS = 2 * L1 + 2 * A2;
+        constexpr int AB1 = STAG ? L1 : L1 + A2;          // first slot of S1/dP1
+        constexpr int ACC0 = STAG ? 2 * L1 : L1;          // first slot of dQ += K0^T dS0
+        constexpr int ACC1 = 2 * L1 + A2;                 // first slot of dQ += K1^T dS1
+        constexpr int AHEAD = 3, NF = 4;
+        v8 fr[NF];
+        f32x16 s[2], dp[2];
+        v8 df[2][2];
+        auto frag = [&](auto I) -> v8 {
+          constexpr int i = decltype(I)::value;
+          constexpr bool is_acc = (i >= ACC0 && i < ACC0 + A2) || i >= ACC1;
+          if constexpr (!is_acc) {
+            constexpr int nb = i >= AB1 ? 1 : 0;
+            constexpr AbSlot sl = ab_slot(nb ? i - AB1 : i, KS_QK, KS_DV);
+            if constexpr (sl.kind == 0) return *(const v8*)(kl + KT::off(nb * 32 + ln, 16 * sl.k + 8 * g));
+            else return *(const v8*)(vl + VT::off(nb * 32 + ln, 16 * sl.k + 8 * g));
+          } else {
+            constexpr int nb = i >= ACC1 ? 1 : 0, j = nb ? i - ACC1 : i - ACC0, hh = j / DKB, d = j % DKB;
+            return *(const v8*)(ktl + ta[(2 * nb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+          }
+        };
+        auto mma = [&](auto I, const v8& f) {
+          constexpr int i = decltype(I)::value;
+          constexpr bool is_acc = (i >= ACC0 && i < ACC0 + A2) || i >= ACC1;
+          const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          if constexpr (!is_acc) {
+            constexpr int nb = i >= AB1 ? 1 : 0;
+            constexpr AbSlot sl = ab_slot(nb ? i - AB1 : i, KS_QK, KS_DV);
+            if constexpr (sl.kind == 0) s[nb] = MT<T>::mfma32(f, qf[sl.k], sl.k == 0 ? zero : s[nb]);
+            else dp[nb] = MT<T>::mfma32(f, dof[sl.k], sl.k == 0 ? zero : dp[nb]);
+          } else {
+            constexpr int nb = i >= ACC1 ? 1 : 0, j = nb ? i - ACC1 : i - ACC0, hh = j / DKB, d = j % DKB;
+            dqacc[d] = MT<T>::mfma32(f, df[nb][hh], dqacc[d]);
+          }
+        };
+        // elements [E0, E0 + N) of block NB spread evenly over the LEN slots starting at START
+        auto valu = [&](auto I, auto NBc, auto E0c, auto Nc, auto STARTc, auto LENc) {
+          constexpr int i = decltype(I)::value, nb = decltype(NBc)::value, e0 = decltype(E0c)::value, n = decltype(Nc)::value,
+                        st = decltype(STARTc)::value, len = decltype(LENc)::value;
+          if constexpr (i >= st && i < st + len) {
+            constexpr int k = i - st, lo = e0 + (k * n + len - 1) / len, hi = e0 + ((k + 1) * n + len - 1) / len;
+  #pragma unroll
+            for (int v = lo; v < hi; v++) {
+              float pv = fast_exp2(__builtin_fmaf(s[nb][v], c, -lse_s));
+              if (MASKED) {
+                const int kvl = nb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
+                const int kv = kv0 + kvl;
+                const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
+                pv = ok ? pv : 0.f;
+              }
+              float dsv = pv * (dp[nb][v] + ndelta_s);
+              asm volatile("" : "+v"(dsv));  // keeps the computation in this slot
+              dp[nb][v] = dsv;
+            }
+            static_for<0, 2>([&](auto H) {  // every half whose eighth value was produced in this slot
+              constexpr int hh = decltype(H)::value;
+              if constexpr (8 * hh + 8 > lo && 8 * hh + 8 <= hi) {
+                const f32x16& x = dp[nb];
+                df[nb][hh] = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4],
+                                      x[8 * hh + 5], x[8 * hh + 6], x[8 * hh + 7]);
+              }
+            });
+          }
+        };
+        typedef std::integral_constant<int, 0> I0;
+        typedef std::integral_constant<int, 1> I1;
+        typedef std::integral_constant<int, 8> I8;
+        typedef std::integral_constant<int, 16> I16;
+        static_for<0, AHEAD>([&](auto I) { fr[decltype(I)::value % NF] = frag(I); });
+        static_for<0, NS>([&](auto I) {
+          constexpr int i = decltype(I)::value;
+          if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
+          if constexpr (!STAG) {
+            // whole dS of a block right before the dQ slots that consume it
+            valu(I, I0{}, I0{}, I16{}, std::integral_constant<int, ACC0>{}, I1{});
+            valu(I, I1{}, I0{}, I16{}, std::integral_constant<int, ACC1>{}, I1{});
+          }
+          mma(I, fr[i % NF]);
+          if constexpr (!STAG) {
+            // the next tile (requested at the top of this one) goes to the other buffer under the last MFMAs
+            // instead of in a phase of its own; after the last tile this stores stale registers nobody reads
+            constexpr int ST0 = NS - 12;
+            unsigned char* nb_base = smem + (buf ^ 1) * KV_BYTES;
+            if constexpr (i == ST0) kst.store_rowmajor(nb_base + (wave < 4 ? 0 : K_BYTES), stid);
+            if constexpr (i >= ST0 + 2 && i < ST0 + 10) {
+              if (wave < 4) kst.template store_transposed_step<i - ST0 - 2>(smem + KTR_AT + (buf ^ 1) * KTR_BYTES, stid);
+            }
+          }
+          if constexpr (STAG) {
+            valu(I, I0{}, I0{}, I16{}, std::integral_constant<int, L1>{}, std::integral_constant<int, L1>{});
+            valu(I, I1{}, I0{}, I8{}, std::integral_constant<int, ACC0>{}, std::integral_constant<int, 2 * DKB>{});
+            valu(I, I1{}, I8{}, I8{}, std::integral_constant<int, ACC1>{}, std::integral_constant<int, DKB>{});
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      };
+      if (!skip) {
+        if (need_mask) body(std::true_type{});
+        else body(std::false_type{});
+      }
+      if (NW == 4 || skip) {
+        if (it + 1 < nact) store_tile(buf ^ 1, buf ^ 1, it);
+      } else if (SEG && tid < BN) {
+        ((int*)(smem + SEG_AT + (buf ^ 1) * BN * 4))[tid] = sreg;
+      }
+      __syncthreads();
     }
-    __syncthreads();
+  
   }
 
   if (qrow < Sq) {
@@ -1259,7 +1429,8 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
     constexpr int BN = 64, BM = 32 * NW;
     constexpr int BUF = BN * RowTile<DQK>::STRIDE + BN * RowTile<DV>::STRIDE + DQK * TrTile64::ROW_BYTES + BN * 4;
     const int nt = (a.Skv + BN - 1) / BN;
-    const size_t smem = 2 * (size_t)BUF + (SEG ? (size_t)(3 * nt + 2 * NW) * 4 : 0);
+    // (8 waves: a third transposed K tile)
+    const size_t smem = 2 * (size_t)BUF + (NW == 8 ? (size_t)DQK * TrTile64::ROW_BYTES : 0) + (SEG ? (size_t)(3 * nt + 2 * NW) * 4 : 0);
     TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_bwd: Skv=%d needs %zu bytes of LDS (max 163840)", a.Skv, smem);
     auto kern = attn_bwd_dq_kernel<T, DQK, DV, NW, CAUSAL, SEG>;
     static bool attr_set = false;
