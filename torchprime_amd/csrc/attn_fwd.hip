@@ -160,6 +160,16 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
     }
     if (SEG && tid < BN) sreg = segb[min(t * BN + tid, Skv - 1)];
   };
+  // the same loads one at a time (piece P of K_ITEMS + 4 V_ITEMS), for issuing between MFMAs
+  auto load_piece = [&](auto Pc, int t) {
+    constexpr int p = decltype(Pc)::value;
+    if constexpr (p < K_ITEMS) {
+      kreg[p] = buf_load16(krs, kvo[p], (unsigned)t * k_tile_bytes);
+    } else {
+      constexpr int i = (p - K_ITEMS) / 4, ii = (p - K_ITEMS) % 4;
+      if (tid + 256 * i < V_TOT) vreg[i][ii] = buf_load16(vrs, vvo[i][ii], (unsigned)t * v_tile_bytes);
+    }
+  };
   auto store_tile = [&](int buf) {
     unsigned char* kl = smem + buf * BUF_BYTES;
     unsigned char* vl = kl + K_BYTES;
@@ -240,7 +250,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
   // and the softmax arithmetic of one 32-row half is spread under the MFMAs that follow it:
   //   slots   S0 = K[0:32] Q^T | S1 = K[32:64] Q^T | O += V[0:32]^T P0 | O += V[32:64]^T P1
   //   VALU                     | max0, exp(S0)     | max1, exp(S1)     | (LDS store of the next tile after)
-  auto tile_body = [&](auto masked_c, int t, int buf, bool has_next) {
+  auto tile_body = [&](auto masked_c, int t, int buf, bool has_next, int t_next) {
     constexpr bool MASKED = decltype(masked_c)::value;
     const int kv0 = t * BN;
     const unsigned char* kl = smem + buf * BUF_BYTES;
@@ -314,6 +324,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
       constexpr int i = decltype(I)::value;
       if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
       mma(I, fr[i % NF]);
+      // the next tile's loads, one per slot (past the last tile they re-read the last one: no branch here)
+      if constexpr (i < K_ITEMS + 4 * V_ITEMS) load_piece(I, t_next);
+      if constexpr (i == 0) {
+        if (SEG && tid < BN) sreg = segb[min(t_next * BN + tid, Skv - 1)];
+      }
       // one slot after the last MFMA of a half: mask, running max (the rare rescale of O is a wave-uniform
       // branch), then the exponentials under the following MFMAs
       if constexpr (i == S1) {
@@ -357,7 +372,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
     const int kv0 = t * BN;
     const int buf = it & 1;
     const bool has_next = it + 1 < nact;
-    if (has_next) load_tile(SEG ? active[it + 1] : it + 1);
+    const int t_next = has_next ? (SEG ? active[it + 1] : it + 1) : t;
 
     // wave-uniform decisions: nothing to do above the diagonal or outside the rows' segments; element
     // masks only on tiles that straddle the diagonal, the tail, or a segment boundary
@@ -369,11 +384,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
       need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
     }
     if (skip) {
-      if (has_next) store_tile(buf ^ 1);
+      if (has_next) {
+        load_tile(t_next);
+        store_tile(buf ^ 1);
+      }
     } else if (need_mask) {
-      tile_body(std::true_type{}, t, buf, has_next);
+      tile_body(std::true_type{}, t, buf, has_next, t_next);
     } else {
-      tile_body(std::false_type{}, t, buf, has_next);
+      tile_body(std::false_type{}, t, buf, has_next, t_next);
     }
     __syncthreads();
   }
