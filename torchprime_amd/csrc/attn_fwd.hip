@@ -45,6 +45,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
   constexpr int V_BYTES = DV * TrTile64::ROW_BYTES;
   constexpr int SEG_BYTES = SEG ? BN * 4 : 0;
   constexpr int BUF_BYTES = K_BYTES + V_BYTES + SEG_BYTES;
+  // LDS layout: the two K tiles, then the two V^T tiles, then the two segment-id rows: with the buffer index a
+  // constant, every address is a loop-invariant per-lane offset plus an immediate
+  constexpr int K_AT = 0, V_AT = 2 * K_BYTES, SEG_AT = V_AT + 2 * V_BYTES;
   constexpr int KCH = DQK / 8;                      // 16-byte chunks per K row
   constexpr int K_ITEMS = BN * KCH / 256;           // chunks per thread
   constexpr int V_TOT = (DV / 8) * (BN / 4);        // 4x8 blocks of the V tile
@@ -171,8 +174,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
     }
   };
   auto store_tile = [&](int buf) {
-    unsigned char* kl = smem + buf * BUF_BYTES;
-    unsigned char* vl = kl + K_BYTES;
+    unsigned char* kl = smem + K_AT + buf * K_BYTES;
+    unsigned char* vl = smem + V_AT + buf * V_BYTES;
 #pragma unroll
     for (int i = 0; i < K_ITEMS; i++) {
       const int item = tid + 256 * i;
@@ -198,7 +201,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
         }
       }
     }
-    if (SEG && tid < BN) ((int*)(vl + V_BYTES))[tid] = sreg;
+    if (SEG && tid < BN) ((int*)(smem + SEG_AT + buf * SEG_BYTES))[tid] = sreg;
   };
 
   // ---- accumulators: O^T blocks, running max (log2 units), per-lane partial row sum
@@ -250,12 +253,22 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
   // and the softmax arithmetic of one 32-row half is spread under the MFMAs that follow it:
   //   slots   S0 = K[0:32] Q^T | S1 = K[32:64] Q^T | O += V[0:32]^T P0 | O += V[32:64]^T P1
   //   VALU                     | max0, exp(S0)     | max1, exp(S1)     | (LDS store of the next tile after)
-  auto tile_body = [&](auto masked_c, int t, int buf, bool has_next, int t_next) {
+  // per-lane offsets of the V^T fragments; they carry the start of the V^T region (an opaque value, or the
+  // compiler folds it back into constants beyond the reach of an instruction offset)
+  unsigned tb[4];
+  {
+    unsigned v_at = (unsigned)V_AT;
+    asm volatile("" : "+v"(v_at));
+#pragma unroll
+    for (int m = 0; m < 4; m++) tb[m] = (unsigned)TrTile64::chunk_off(ln, m, g) + v_at;
+  }
+  auto tile_body = [&](auto masked_c, auto BUFc, int t, bool has_next, int t_next) {
     constexpr bool MASKED = decltype(masked_c)::value;
+    constexpr int buf = decltype(BUFc)::value;
     const int kv0 = t * BN;
-    const unsigned char* kl = smem + buf * BUF_BYTES;
-    const unsigned char* vl = kl + K_BYTES;
-    const int* sl = (const int*)(vl + V_BYTES);
+    const unsigned char* kl = smem + K_AT + buf * K_BYTES;
+    const unsigned char* vl = smem + buf * V_BYTES;  // + tb[]
+    const int* sl = (const int*)(smem + SEG_AT + buf * SEG_BYTES);
     auto mask_half = [&](f32x16& s, int hf) {
 #pragma unroll
       for (int v = 0; v < 16; v++) {
@@ -279,7 +292,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
         return *(const v8*)(kl + KT::off(hf * 32 + ln, 16 * ks + 8 * g));
       } else {
         constexpr int hf = (i - PV0) / (2 * DVB), j = (i - PV0) % (2 * DVB), kk = j / DVB, d = j % DVB;
-        return *(const v8*)(vl + TrTile64::chunk_off(d * 32 + ln, 2 * hf + kk, g));
+        return *(const v8*)(vl + tb[(2 * hf + kk) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
       }
     };
     auto mma = [&](auto I, const v8& f) {
@@ -367,10 +380,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
   __syncthreads();
 
   const int wq_last = wq0 + 31;
-  for (int it = 0; it < nact; it++) {
+  // one kv tile; the buffer index is a constant (the loop below alternates two copies of this)
+  auto iteration = [&](auto BUFc, const int it) {
+    constexpr int buf = decltype(BUFc)::value;
     const int t = SEG ? active[it] : it;
     const int kv0 = t * BN;
-    const int buf = it & 1;
     const bool has_next = it + 1 < nact;
     const int t_next = has_next ? (SEG ? active[it + 1] : it + 1) : t;
 
@@ -389,11 +403,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
         store_tile(buf ^ 1);
       }
     } else if (need_mask) {
-      tile_body(std::true_type{}, t, buf, has_next, t_next);
+      tile_body(std::true_type{}, BUFc, t, has_next, t_next);
     } else {
-      tile_body(std::false_type{}, t, buf, has_next, t_next);
+      tile_body(std::false_type{}, BUFc, t, has_next, t_next);
     }
     __syncthreads();
+  };
+  for (int it = 0; it < nact; it += 2) {
+    iteration(std::integral_constant<int, 0>{}, it);
+    if (it + 1 < nact) iteration(std::integral_constant<int, 1>{}, it + 1);
   }
 
   // ---- epilogue: normalise, write O (row = query, 4 consecutive v-dims per store) and LSE
