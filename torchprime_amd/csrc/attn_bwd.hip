@@ -331,20 +331,6 @@ struct TransposeSteps {
   }
 };
 
-// per-tile [min,max] of segment ids for 64-row tiles t0..t1-1 into LDS (lane = row of the tile)
-__device__ __forceinline__ void seg_tile_ranges(const int32_t* segb, int S, int t0, int t1, int* tmin, int* tmax,
-                                                int wave, int lane) {
-  for (int t = t0 + wave; t < t1; t += 4) {
-    int lo = segb[min(t * 64 + lane, S - 1)], hi = lo;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      lo = min(lo, __shfl_xor(lo, o, 64));
-      hi = max(hi, __shfl_xor(hi, o, 64));
-    }
-    if (lane == 0) { tmin[t - t0] = lo; tmax[t - t0] = hi; }
-  }
-}
-
 // ------------------------------------------------------------------------------------------------
 // dK / dV
 // ------------------------------------------------------------------------------------------------
@@ -411,7 +397,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     wkmin = __builtin_amdgcn_readfirstlane(wkmin);
     wkmax = __builtin_amdgcn_readfirstlane(wkmax);
     if (lane == 0) { bk[2 * wave] = wkmin; bk[2 * wave + 1] = wkmax; }
-    seg_tile_ranges(segb, Sq, qt_first, nqt_all, qmin, qmax, wave, lane);
+    seg_tile_ranges(segb, Sq, qt_first, nqt_all, qmin, qmax, tid, 256);
     __syncthreads();
     const int bkmin = min(min(bk[0], bk[2]), min(bk[4], bk[6]));
     const int bkmax = max(max(bk[1], bk[3]), max(bk[5], bk[7]));
@@ -978,7 +964,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
     wqmin = __builtin_amdgcn_readfirstlane(wqmin);
     wqmax = __builtin_amdgcn_readfirstlane(wqmax);
     if (lane == 0) { bq[2 * wave] = wqmin; bq[2 * wave + 1] = wqmax; }
-    if (wave < 4) seg_tile_ranges(segb, Skv, 0, ntiles, kvmin, kvmax, wave, lane);
+    seg_tile_ranges(segb, Skv, 0, ntiles, kvmin, kvmax, tid, 64 * NW);
     __syncthreads();
     int bqmin = bq[0], bqmax = bq[1];
 #pragma unroll
@@ -1054,8 +1040,11 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   const int wq_last = wq0 + 31;
   const int qrow = wq0 + ln;
 
+  // i-th kv tile to visit, as a scalar (a tile offset in vector registers would put every staging load into a
+  // loop over its distinct values)
+  auto tile_at = [&](int i) { return SEG ? __builtin_amdgcn_readfirstlane(active[i]) : i; };
   if (nact > 0) {
-    load_tile(SEG ? active[0] : 0, 0);
+    load_tile(tile_at(0), 0);
     store_tile(0, 0, 0);
   }
   __builtin_amdgcn_s_waitcnt(0);  // Q / dO fragments, LSE and delta have landed (see the dK/dV kernel)
@@ -1115,10 +1104,10 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
     bool pending = false;
     int kslot = 0;
     for (int it = 0; it < nact; it++) {
-      const int t = SEG ? active[it] : it;
+      const int t = tile_at(it);
       const int kv0 = t * BN;
       const int buf = it & 1;
-      if (it + 1 < nact) load_tile(SEG ? active[it + 1] : it + 1, it);
+      if (it + 1 < nact) load_tile(tile_at(it + 1), it);
       const int kprev = kslot == 0 ? 2 : kslot - 1, knext = kslot == 2 ? 0 : kslot + 1;
       const unsigned char* kl = smem + buf * KV_BYTES;
       const unsigned char* vl = kl + K_BYTES;
@@ -1222,10 +1211,10 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
     if (pending) drain(smem + KTR_AT + (kslot == 0 ? 2 : kslot - 1) * KTR_BYTES);
   } else {
   for (int it = 0; it < nact; it++) {
-      const int t = SEG ? active[it] : it;
+      const int t = tile_at(it);
       const int kv0 = t * BN;
       const int buf = it & 1;
-      if (it + 1 < nact) load_tile(SEG ? active[it + 1] : it + 1, it);
+      if (it + 1 < nact) load_tile(tile_at(it + 1), it);
   
       const unsigned char* kl = smem + buf * KV_BYTES;
       const unsigned char* vl = kl + K_BYTES;

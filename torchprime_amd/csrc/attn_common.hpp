@@ -141,6 +141,40 @@ inline unsigned xcd_grid(int n_tiles, int n_inner, int n_groups) {
   return (unsigned)(NUM_XCD * ((n_groups + NUM_XCD - 1) / NUM_XCD) * n_tiles * n_inner);
 }
 
+// Per-tile [min, max] of the segment ids of the 64-row tiles t0..t1-1, into LDS.  One thread per tile: its 64
+// ids are independent loads in flight together (a lane-per-row reduction waits out one load and twelve
+// shuffles per tile, which for short documents took longer than the tiles' own work).  Rows past S repeat the
+// last id.
+__device__ __forceinline__ void seg_tile_ranges(const int32_t* segb, int S, int t0, int t1, int* tmin, int* tmax,
+                                                int tid, int nthreads) {
+  const bool vec = (((size_t)segb) & 15) == 0;
+  for (int t = t0 + tid; t < t1; t += nthreads) {
+    const int base = t * 64;
+    int lo, hi;
+    if (vec && base + 64 <= S) {
+      const int4* p = (const int4*)(segb + base);
+      int4 v = p[0];
+      lo = min(min(v.x, v.y), min(v.z, v.w));
+      hi = max(max(v.x, v.y), max(v.z, v.w));
+#pragma unroll
+      for (int i = 1; i < 16; i++) {
+        v = p[i];
+        lo = min(min(lo, v.x), min(min(v.y, v.z), v.w));
+        hi = max(max(hi, v.x), max(max(v.y, v.z), v.w));
+      }
+    } else {
+      lo = hi = segb[min(base, S - 1)];
+      for (int i = 1; i < 64; i++) {
+        const int v = segb[min(base + i, S - 1)];
+        lo = min(lo, v);
+        hi = max(hi, v);
+      }
+    }
+    tmin[t - t0] = lo;
+    tmax[t - t0] = hi;
+  }
+}
+
 // ---- LDS layouts ---------------------------------------------------------------------------------
 // Row-major tile [rows][D] of 16-bit elements: rows padded by 16 bytes so that 16-byte reads by lanes
 // in consecutive rows land in different banks.

@@ -47,7 +47,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
   constexpr int BUF_BYTES = K_BYTES + V_BYTES + SEG_BYTES;
   // LDS layout: the two K tiles, then the two V^T tiles, then the two segment-id rows: with the buffer index a
   // constant, every address is a loop-invariant per-lane offset plus an immediate
-  constexpr int K_AT = 0, V_AT = 2 * K_BYTES, SEG_AT = V_AT + 2 * V_BYTES;
+  // (the plain causal kernel only: the other variants keep a buffer's K, V^T and ids together, one base
+  // register for all three, which is what their register budget allows)
+  constexpr bool STATIC_BUF = CAUSAL && !SEG;
+  constexpr int K_AT = 0, K_STEP = STATIC_BUF ? K_BYTES : BUF_BYTES;
+  constexpr int V_AT = STATIC_BUF ? 2 * K_BYTES : K_BYTES, V_STEP = STATIC_BUF ? V_BYTES : BUF_BYTES;
+  constexpr int SEG_AT = STATIC_BUF ? 2 * (K_BYTES + V_BYTES) : K_BYTES + V_BYTES, SEG_STEP = STATIC_BUF ? SEG_BYTES : BUF_BYTES;
   constexpr int KCH = DQK / 8;                      // 16-byte chunks per K row
   constexpr int K_ITEMS = BN * KCH / 256;           // chunks per thread
   constexpr int V_TOT = (DV / 8) * (BN / 4);        // 4x8 blocks of the V tile
@@ -101,16 +106,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
     wqmin = __builtin_amdgcn_readfirstlane(wqmin);
     wqmax = __builtin_amdgcn_readfirstlane(wqmax);
     if (lane == 0) { bq[2 * wave] = wqmin; bq[2 * wave + 1] = wqmax; }
-    for (int t = wave; t < ntiles; t += 4) {
-      const int idx = min(t * BN + lane, Skv - 1);
-      int lo = segb[idx], hi = lo;
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) {
-        lo = min(lo, __shfl_xor(lo, o, 64));
-        hi = max(hi, __shfl_xor(hi, o, 64));
-      }
-      if (lane == 0) { kvmin[t] = lo; kvmax[t] = hi; }
-    }
+    static_assert(BN == 64, "seg_tile_ranges works on 64-row tiles");
+    seg_tile_ranges(segb, Skv, 0, ntiles, kvmin, kvmax, tid, 256);
     __syncthreads();
     const int bqmin = min(min(bq[0], bq[2]), min(bq[4], bq[6]));
     const int bqmax = max(max(bq[1], bq[3]), max(bq[5], bq[7]));
@@ -174,8 +171,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
     }
   };
   auto store_tile = [&](int buf) {
-    unsigned char* kl = smem + K_AT + buf * K_BYTES;
-    unsigned char* vl = smem + V_AT + buf * V_BYTES;
+    unsigned char* kl = smem + K_AT + buf * K_STEP;
+    unsigned char* vl = kl + (V_AT - K_AT) + buf * (V_STEP - K_STEP);
 #pragma unroll
     for (int i = 0; i < K_ITEMS; i++) {
       const int item = tid + 256 * i;
@@ -201,7 +198,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
         }
       }
     }
-    if (SEG && tid < BN) ((int*)(smem + SEG_AT + buf * SEG_BYTES))[tid] = sreg;
+    if (SEG && tid < BN) ((int*)(smem + SEG_AT + buf * SEG_STEP))[tid] = sreg;
   };
 
   // ---- accumulators: O^T blocks, running max (log2 units), per-lane partial row sum
@@ -256,19 +253,20 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
   // per-lane offsets of the V^T fragments; they carry the start of the V^T region (an opaque value, or the
   // compiler folds it back into constants beyond the reach of an instruction offset)
   unsigned tb[4];
-  {
+  if constexpr (STATIC_BUF) {
     unsigned v_at = (unsigned)V_AT;
     asm volatile("" : "+v"(v_at));
 #pragma unroll
     for (int m = 0; m < 4; m++) tb[m] = (unsigned)TrTile64::chunk_off(ln, m, g) + v_at;
   }
-  auto tile_body = [&](auto masked_c, auto BUFc, int t, bool has_next, int t_next) {
+  auto tile_body = [&](auto masked_c, auto BUFc, int buf_rt, int t, bool has_next, int t_next) {
     constexpr bool MASKED = decltype(masked_c)::value;
-    constexpr int buf = decltype(BUFc)::value;
+    // the buffer index: a constant, or (-1) the run-time one
+    const int buf = decltype(BUFc)::value >= 0 ? decltype(BUFc)::value : buf_rt;
     const int kv0 = t * BN;
-    const unsigned char* kl = smem + K_AT + buf * K_BYTES;
+    const unsigned char* kl = smem + K_AT + buf * K_STEP;
     const unsigned char* vl = smem + buf * V_BYTES;  // + tb[]
-    const int* sl = (const int*)(smem + SEG_AT + buf * SEG_BYTES);
+    const int* sl = (const int*)(kl + (SEG_AT - K_AT) + buf * (SEG_STEP - K_STEP));
     auto mask_half = [&](f32x16& s, int hf) {
 #pragma unroll
       for (int v = 0; v < 16; v++) {
@@ -292,7 +290,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
         return *(const v8*)(kl + KT::off(hf * 32 + ln, 16 * ks + 8 * g));
       } else {
         constexpr int hf = (i - PV0) / (2 * DVB), j = (i - PV0) % (2 * DVB), kk = j / DVB, d = j % DVB;
-        return *(const v8*)(vl + tb[(2 * hf + kk) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+        if constexpr (STATIC_BUF) return *(const v8*)(vl + tb[(2 * hf + kk) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+        else return *(const v8*)(kl + (V_AT - K_AT) + TrTile64::chunk_off(d * 32 + ln, 2 * hf + kk, g));
       }
     };
     auto mma = [&](auto I, const v8& f) {
@@ -368,8 +367,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
     if (has_next) store_tile(buf ^ 1);
   };
 
+  // i-th kv tile to visit, as a scalar: a tile offset in vector registers would put every staging load into a
+  // loop over its distinct values
+  auto tile_at = [&](int i) { return SEG ? __builtin_amdgcn_readfirstlane(active[i]) : i; };
   if (nact > 0) {
-    load_tile(SEG ? active[0] : 0);
+    load_tile(tile_at(0));
     store_tile(0);
   }
   // Everything loaded so far (the Q fragments above all) has landed before the loop starts.  Without
@@ -380,16 +382,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
   __syncthreads();
 
   const int wq_last = wq0 + 31;
-  // one kv tile; the buffer index is a constant (the loop below alternates two copies of this)
+  // One kv tile.  BUFc: the buffer index as a constant, or (-1) taken at run time.
+  // wave-uniform decisions: nothing to do above the diagonal or outside the rows' segments; element masks
+  // only on tiles that straddle the diagonal, the tail, or a segment boundary
   auto iteration = [&](auto BUFc, const int it) {
-    constexpr int buf = decltype(BUFc)::value;
-    const int t = SEG ? active[it] : it;
+    const int buf = decltype(BUFc)::value >= 0 ? decltype(BUFc)::value : (it & 1);
+    const int t = tile_at(it);
     const int kv0 = t * BN;
     const bool has_next = it + 1 < nact;
-    const int t_next = has_next ? (SEG ? active[it + 1] : it + 1) : t;
-
-    // wave-uniform decisions: nothing to do above the diagonal or outside the rows' segments; element
-    // masks only on tiles that straddle the diagonal, the tail, or a segment boundary
+    const int t_next = has_next ? tile_at(it + 1) : t;
     bool skip = CAUSAL && kv0 > wq_last;
     bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0);
     if (SEG) {
@@ -403,15 +404,47 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
         store_tile(buf ^ 1);
       }
     } else if (need_mask) {
-      tile_body(std::true_type{}, BUFc, t, has_next, t_next);
+      tile_body(std::true_type{}, BUFc, buf, t, has_next, t_next);
     } else {
-      tile_body(std::false_type{}, BUFc, t, has_next, t_next);
+      tile_body(std::false_type{}, BUFc, buf, t, has_next, t_next);
     }
     __syncthreads();
   };
-  for (int it = 0; it < nact; it += 2) {
-    iteration(std::integral_constant<int, 0>{}, it);
-    if (it + 1 < nact) iteration(std::integral_constant<int, 1>{}, it + 1);
+  if constexpr (STATIC_BUF) {
+    // the plain causal kernel: the loop alternates two copies of the body, one per buffer
+    for (int it = 0; it < nact; it += 2) {
+      iteration(std::integral_constant<int, 0>{}, it);
+      if (it + 1 < nact) iteration(std::integral_constant<int, 1>{}, it + 1);
+    }
+  } else {
+    // The masked variants have no registers to spare for two copies.  (Their loop body is written out here:
+    // routed through the closure above, the compiler keeps part of the captured state in scratch memory.)
+    for (int it = 0; it < nact; it++) {
+      const int buf = it & 1;
+      const int t = tile_at(it);
+      const int kv0 = t * BN;
+      const bool has_next = it + 1 < nact;
+      const int t_next = has_next ? tile_at(it + 1) : t;
+      bool skip = CAUSAL && kv0 > wq_last;
+      bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0);
+      if (SEG) {
+        const int lo = kvmin[t], hi = kvmax[t];
+        skip = skip || hi < wqmin || lo > wqmax;
+        need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
+      }
+      typedef std::integral_constant<int, -1> RT;
+      if (skip) {
+        if (has_next) {
+          load_tile(t_next);
+          store_tile(buf ^ 1);
+        }
+      } else if (need_mask) {
+        tile_body(std::true_type{}, RT{}, buf, t, has_next, t_next);
+      } else {
+        tile_body(std::false_type{}, RT{}, buf, t, has_next, t_next);
+      }
+      __syncthreads();
+    }
   }
 
   // ---- epilogue: normalise, write O (row = query, 4 consecutive v-dims per store) and LSE
