@@ -94,6 +94,17 @@ def test_segment_ids_unsorted_and_negative_ids():
   _check(2, 2, 1, 260, 64, 64, torch.bfloat16, False, seg=seg)
 
 
+@pytest.mark.parametrize("D", [128, 64])
+def test_segment_ids_alternating_blocks(D):
+  # ids alternate every 64 rows (0,1,0,1,... and 0,0,1,1,...): inside one 256-row workgroup some waves need a
+  # kv tile that the others skip, tile after tile, so the backward's carried second kv block is finished both
+  # ways (inside the next tile's body and on its own after a skipped tile)
+  S = 1024
+  r = torch.arange(S)
+  seg = torch.stack([(r // 64) % 2, (r // 128) % 2]).to(torch.int32)
+  _check(2, 4, 2, S, D, D, torch.bfloat16, True, seg=seg)
+
+
 def test_segment_equals_block_diagonal_decomposition():
   """Document masking == running each document through causal attention on its own."""
   B, Hq, Hkv, S, D = 1, 4, 2, 448, 128
