@@ -1446,8 +1446,35 @@ static int dispatch_bwd(const BwdArgs& a, int causal, hipStream_t st, void* cons
   return launch_bwd<T, DQK, DV, false, false>(a, st, ev);
 }
 
+// One element type per translation unit: this file is compiled twice (TP_BWD_F16 = 0 and 1, side by side, which
+// halves the build time).  Either unit defines its own dispatcher over the head dims; the bf16 unit also holds
+// the C entry points.  A dispatcher returns TP_DIMS_NOT_BUILT for head dims it has no kernels for.
+#ifndef TP_BWD_F16
+#define TP_BWD_F16 0
+#endif
+constexpr int TP_DIMS_NOT_BUILT = -1000;
+int bwd_by_dims_bf16(const BwdArgs& a, int Dqk, int Dv, int causal, hipStream_t st, void* const* ev);
+int bwd_by_dims_f16(const BwdArgs& a, int Dqk, int Dv, int causal, hipStream_t st, void* const* ev);
+template <typename T>
+static int bwd_by_dims(const BwdArgs& a, int Dqk, int Dv, int causal, hipStream_t st, void* const* ev) {
+  if (Dqk == 128 && Dv == 128) return dispatch_bwd<T, 128, 128>(a, causal, st, ev);
+  if (Dqk == 64 && Dv == 64) return dispatch_bwd<T, 64, 64>(a, causal, st, ev);
+  if (Dqk == 192 && Dv == 128) return dispatch_bwd<T, 192, 128>(a, causal, st, ev);
+  return TP_DIMS_NOT_BUILT;
+}
+#if TP_BWD_F16
+int bwd_by_dims_f16(const BwdArgs& a, int Dqk, int Dv, int causal, hipStream_t st, void* const* ev) {
+  return bwd_by_dims<f16_t>(a, Dqk, Dv, causal, st, ev);
+}
+#else
+int bwd_by_dims_bf16(const BwdArgs& a, int Dqk, int Dv, int causal, hipStream_t st, void* const* ev) {
+  return bwd_by_dims<bf16_t>(a, Dqk, Dv, causal, st, ev);
+}
+#endif
+
 }  // namespace tp
 
+#if !TP_BWD_F16
 using namespace tp;
 
 extern "C" size_t tp_attn_bwd_workspace_bytes(int B, int Hq, int Sq) {
@@ -1496,18 +1523,9 @@ extern "C" int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, co
   a.scale_log2 = sm_scale * LOG2E;
   a.sm_scale = sm_scale;
   hipStream_t st = (hipStream_t)stream;
-#define TP_BWD(T, DQ, DVV) return dispatch_bwd<T, DQ, DVV>(a, causal, st, events)
-  if (dtype == TP_BF16) {
-    if (Dqk == 128 && Dv == 128) TP_BWD(bf16_t, 128, 128);
-    if (Dqk == 64 && Dv == 64) TP_BWD(bf16_t, 64, 64);
-    if (Dqk == 192 && Dv == 128) TP_BWD(bf16_t, 192, 128);
-  } else {
-    if (Dqk == 128 && Dv == 128) TP_BWD(f16_t, 128, 128);
-    if (Dqk == 64 && Dv == 64) TP_BWD(f16_t, 64, 64);
-    if (Dqk == 192 && Dv == 128) TP_BWD(f16_t, 192, 128);
-  }
-#undef TP_BWD
-  TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_attn_bwd: head dims (qk=%d, v=%d) not built", Dqk, Dv);
+  const int rc = dtype == TP_BF16 ? bwd_by_dims_bf16(a, Dqk, Dv, causal, st, events) : bwd_by_dims_f16(a, Dqk, Dv, causal, st, events);
+  TP_REQUIRE(rc != TP_DIMS_NOT_BUILT, TP_ERR_UNSUPPORTED, "tp_attn_bwd: head dims (qk=%d, v=%d) not built", Dqk, Dv);
+  return rc;
 }
 
 extern "C" int tp_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
@@ -1520,3 +1538,4 @@ extern "C" int tp_attn_bwd(const void* dout, const void* q, const void* k, const
                         k_strides, v_strides, o_strides, dq_strides, dk_strides, dv_strides, sm_scale, causal, dtype, stream,
                         nullptr);
 }
+#endif  // !TP_BWD_F16
