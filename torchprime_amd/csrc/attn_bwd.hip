@@ -14,7 +14,7 @@
 //                         for dV^T += dO^T P and dK^T += Q^T dS).  S is computed un-transposed here so
 //                         that a lane owns one KV column: P and dS converted to 16 bit are directly the
 //                         B operands of the two accumulating products.
-//   attn_bwd_dq_kernel    one workgroup = 128 query rows of one (batch, head); Q and dO fragments in
+//   attn_bwd_dq_kernel    one workgroup = 128 or 256 query rows (4 or 8 waves) of one (batch, head); Q and dO fragments in
 //                         registers, K (row-major + transposed) and V (row-major) tiles stream through
 //                         LDS; S^T, dP^T are computed transposed (a lane owns one query column, so LSE
 //                         and delta are per-lane scalars) and dS^T feeds dQ^T += K^T dS^T.
