@@ -1,7 +1,7 @@
 """Benchmark of the attention hot path on one MI355X.
 
 One step = one forward + backward pass of causal GQA attention at the Llama-3-8B layer shape
-(BASELINE config 2: B=4, S=8192, 32 q heads / 8 kv heads, d=128, bf16) with q, k, v and dO already
+(benchmark configuration 2: B=4, S=8192, 32 q heads / 8 kv heads, d=128, bf16) with q, k, v and dO already
 resident in HBM.  Prints ONE JSON line:
 
   value        algorithmic TFLOP/s of the whole step, 6*B*Hq*S^2*d FLOP per step (the reference's own

@@ -23,7 +23,7 @@ from tests.util import packed_segment_ids, randn  # noqa: E402
 
 
 def c1_inputs():
-  """BASELINE config 1: tiny Llama attention block, fp32 (the reference's test fixture shape)."""
+  """benchmark configuration 1: tiny Llama attention block, fp32 (the reference's test fixture shape)."""
   x = randn((2, 128, 512), 1234)
   w = {n: randn((512, 512), 1234 + i + 1, std=0.02) for i, n in enumerate(("wq", "wk", "wv", "wo"))}
   w_norm = 1 + randn((512,), 1239, std=0.02)

@@ -63,7 +63,7 @@ def test_hip_attention_matches_golden():
 
 @pytest.mark.gpu
 def test_hip_llama_block_matches_golden_c1():
-  """BASELINE config 1 on the GPU: RMSNorm (fp32 kernel) -> projections -> RoPE -> attention -> o_proj.
+  """benchmark configuration 1 on the GPU: RMSNorm (fp32 kernel) -> projections -> RoPE -> attention -> o_proj.
   The attention kernels are 16-bit, so q/k/v are cast to bf16 around the attention call only."""
   import torchprime_amd as tpa
 

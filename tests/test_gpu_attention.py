@@ -232,7 +232,7 @@ def test_unsupported_inputs_raise():
     tpa.ops.attention(q.cpu(), q.cpu(), q.cpu())
 
 
-# ---- BASELINE-size cases ----------------------------------------------------------------------------
+# ---- full-size cases ----------------------------------------------------------------------------
 def _slice_check(B, Hq, Hkv, S, Dqk, Dv, seg, seed, b_sel, g_sel, sm_scale=None):
   """Run the kernels on the full problem, check one (batch, kv-head group) slice against the oracle
   (attention is independent per batch and kv head, so the slice is an exact sub-problem)."""
@@ -254,18 +254,18 @@ def _slice_check(B, Hq, Hkv, S, Dqk, Dv, seg, seed, b_sel, g_sel, sm_scale=None)
   assert torch.isfinite(lse).all() and torch.isfinite(dq.float()).all()
 
 
-def test_llama3_8b_shape_slice():  # BASELINE config 2: B=4, S=8192, 32q/8kv, d=128
+def test_llama3_8b_shape_slice():  # benchmark configuration 2: B=4, S=8192, 32q/8kv, d=128
   _slice_check(4, 32, 8, 8192, 128, 128, None, 1234 + 1, b_sel=3, g_sel=5)
 
 
-def test_llama3_8b_packed_segments_slice():  # BASELINE config 3: documents of 64..4096 packed to 8192
+def test_llama3_8b_packed_segments_slice():  # benchmark configuration 3: documents of 64..4096 packed to 8192
   seg, _ = packed_segment_ids(4, 8192, 64, 4096, seed=1234 + 2)
   _slice_check(4, 32, 8, 8192, 128, 128, seg, 1234 + 2, b_sel=1, g_sel=2)
 
 
-def test_llama3_70b_shape_slice():  # BASELINE config 3: B=1, S=8192, 64q/8kv
+def test_llama3_70b_shape_slice():  # benchmark configuration 3: B=1, S=8192, 64q/8kv
   _slice_check(1, 64, 8, 8192, 128, 128, None, 1234 + 3, b_sel=0, g_sel=7)
 
 
-def test_deepseek_v3_shape_slice():  # BASELINE config 4: B=1, S=4096, 128 heads, qk 192 / v 128, scale 1/sqrt(128)
+def test_deepseek_v3_shape_slice():  # benchmark configuration 4: B=1, S=4096, 128 heads, qk 192 / v 128, scale 1/sqrt(128)
   _slice_check(1, 128, 128, 4096, 192, 128, None, 1234 + 4, b_sel=0, g_sel=77)

@@ -2,7 +2,7 @@
 
 import torch
 
-# BASELINE tolerance for 16-bit outputs and gradients against the fp32 oracle
+# tolerance for 16-bit outputs and gradients against the fp32 oracle
 MAX_ABS = 2e-2
 REL_L2 = 1e-2
 
