@@ -79,8 +79,9 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
   const int64_t bh = rowid / a.Sq;
   const int h = (int)(bh % a.Hq), b = (int)(bh / a.Hq);
   float o[8], g[8];
-  load_f<T, 8>((const T*)a.out + b * a.os[0] + h * a.os[1] + s * a.os[2] + ch * 8, o);
-  load_f<T, 8>((const T*)a.dout + b * a.dos[0] + h * a.dos[1] + s * a.dos[2] + ch * 8, g);
+  // (streamed once here: non-temporal loads, as in the other HBM-bound kernels)
+  load_f_nt<T, 8>((const T*)a.out + b * a.os[0] + h * a.os[1] + s * a.os[2] + ch * 8, o);
+  load_f_nt<T, 8>((const T*)a.dout + b * a.dos[0] + h * a.dos[1] + s * a.dos[2] + ch * 8, g);
   float acc = 0.f;
 #pragma unroll
   for (int e = 0; e < 8; e++) acc += o[e] * g[e];
