@@ -277,7 +277,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
       }
     };
     constexpr int S1 = KSTEPS, PV0 = 2 * KSTEPS, PV1 = PV0 + 2 * DVB, NS = PV1 + 2 * DVB;
-    constexpr int AHEAD = 3, NF = 4;
+    constexpr int AHEAD = STATIC_BUF ? 5 : 3, NF = AHEAD + 1;  // (the plain causal kernel has registers left for a deeper ring)
     v8 fr[NF];
     f32x16 s[2];
     v8 pf[2][2];
