@@ -159,7 +159,7 @@ def bench_attention(args, dev):
   # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this script, each scaled by
   # what the counter reads for the 256 MiB copy of --calib-copy); the summary with the commands is
   # profiles/attn_fwd_bwd_llama3_8b_S8192_hbm_traffic.md.  Counters cannot be read from inside this process.
-  measured_traffic = {"attn_fwd": 9.06e8, "attn_bwd_dkdv": 9.72e9, "attn_bwd_dq": 1.2e9}
+  measured_traffic = {"attn_fwd": 9.04e8, "attn_bwd_dkdv": 9.67e9, "attn_bwd_dq": 1.2e9}
   dom = max(("attn_fwd", "attn_bwd_dkdv", "attn_bwd_dq"), key=lambda n: avg[n])
   achieved = algo[dom] / (avg[dom] * 1e-3) / 1e12
   roofline = {
