@@ -21,7 +21,7 @@ def _load(name):
 def test_oracle_reproduces_golden():
   x, w_norm, w = c1_inputs()
   y = orc.llama_attention_block(x, w_norm, w["wq"], w["wk"], w["wv"], w["wo"], 8, 8, 1e-5, 500000.0)
-  torch.testing.assert_close(y[:, ::8], _load("c1_llama_block.npz")["out_rows"], rtol=1e-4, atol=1e-6)
+  torch.testing.assert_close(y[:, ::8], _load("c1_llama_block.npz")["out_rows"], rtol=1e-4, atol=2e-5)  # fp32 matmul chains: reduction order differs with the thread count
   q, k, v, do, seg = attn_inputs()
   g = _load("attn_segments_small.npz")
   out, dq, dk, dv = orc.attention_grads_ref(q, k, v, do, seg, True, None, torch.float64)

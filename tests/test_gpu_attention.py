@@ -23,7 +23,8 @@ def _run(q, k, v, do, seg, causal, sm_scale):
   return out.detach(), lse, qd.grad, kd.grad, vd.grad
 
 
-def _check(B, Hq, Hkv, S, Dqk, Dv, dtype, causal, seg=None, layout="bshd", seed=0, Skv=None, sm_scale=None, std=1.0, v_std=None):
+def _check(B, Hq, Hkv, S, Dqk, Dv, dtype, causal, seg=None, layout="bshd", seed=0, Skv=None, sm_scale=None, std=1.0, v_std=None,
+           grad_abs=2e-2):
   Skv = S if Skv is None else Skv
   mk = heads_view if layout == "bshd" else (lambda B_, H, S_, D, sd, dt, std=1.0: randn((B_, H, S_, D), sd, dt, std))
   q = mk(B, Hq, S, Dqk, seed + 1, dtype, std)
@@ -37,11 +38,11 @@ def _check(B, Hq, Hkv, S, Dqk, Dv, dtype, causal, seg=None, layout="bshd", seed=
   assert out.shape == (B, Hq, S, Dv) and out.dtype == dtype
   assert_close(out, o_ref, "out")
   assert_close(lse, lse_ref, "lse", max_abs=5e-3, rel_l2=1e-3)  # row sums add the 16-bit-rounded p the PV product uses
-  # gradients reach |x| > 4 with N(0,1) inputs, where one bf16 rounding alone is up to 1.6e-2:
-  # the max-abs bound is taken relative to the tensor's scale there (tests/util.py)
-  assert_close(dq, dq_ref, "dq", scale_abs=True)
-  assert_close(dk, dk_ref, "dk", scale_abs=True)
-  assert_close(dv, dv_ref, "dv", scale_abs=True)
+  # gradients reach |x| > 4 with N(0,1) inputs, where one bf16 rounding alone is up to 1.6e-2: every element
+  # gets the stated bound plus one bf16 ulp of its own magnitude, |err| <= 2e-2 + 2^-7 |ref| (tests/util.py)
+  assert_close(dq, dq_ref, "dq", max_abs=grad_abs, scale_abs=True)
+  assert_close(dk, dk_ref, "dk", max_abs=grad_abs, scale_abs=True)
+  assert_close(dv, dv_ref, "dv", max_abs=grad_abs, scale_abs=True)
   return out
 
 
@@ -72,8 +73,11 @@ def test_full_attention_fwd_bwd(B, Hq, Hkv, S, Skv, Dqk, Dv):
 def test_running_max_moves_often(seed):
   # large score spread: the row maximum keeps growing by more than the lazy-rescale threshold, in either
   # half of a KV tile, so the rescale paths (including the one deferred past the first half's P V) run
-  _check(1, 4, 2, 512, 128, 128, torch.bfloat16, True, seed=10 * seed, std=2.5, v_std=1.0)
-  _check(1, 2, 2, 300, 64, 64, torch.bfloat16, False, seed=10 * seed + 5, std=3.0, v_std=1.0)
+  # (q and k are 2.5x / 3x the N(0,1) scale the tolerance is stated for: the scores, and with them the rounding
+  # errors of P and dS that dq = sm_scale dS K and dk = sm_scale dS^T Q multiply by the larger q / k values, grow
+  # with the square of that factor, and so does the absolute bound here; relative-L2 stays at 1e-2)
+  _check(1, 4, 2, 512, 128, 128, torch.bfloat16, True, seed=10 * seed, std=2.5, v_std=1.0, grad_abs=2e-2 * 2.5**2)
+  _check(1, 2, 2, 300, 64, 64, torch.bfloat16, False, seed=10 * seed + 5, std=3.0, v_std=1.0, grad_abs=2e-2 * 3.0**2)
 
 
 def test_contiguous_bhsd_layout_and_scale():

@@ -89,10 +89,10 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
   for (int off = TPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
   if (valid && ch == 0) {
     a.delta[rowid] = -acc;  // stored negated: the dK/dV kernel starts its dP accumulators from it
-    // second half of the workspace: LSE in log2 units for the dK/dV kernel; a row with no allowed key
-    // (LSE = -inf) gets +inf so that its P = exp2(s - inf) = 0
+    // second half of the workspace: minus the LSE in log2 units, which the dK/dV kernel starts its S
+    // accumulators from; a row with no allowed key (LSE = -inf) gets -inf so that its P = exp2(-inf) = 0
     const float l = a.lse[rowid];
-    a.delta[total + rowid] = (l == -INFINITY) ? INFINITY : l * LOG2E;
+    a.delta[total + rowid] = (l == -INFINITY) ? -INFINITY : -l * LOG2E;
   }
 }
 
@@ -218,14 +218,14 @@ struct DmaTile {
   __device__ __forceinline__ void issue_one(u32x4 rs, unsigned tile_byte_offset, unsigned char* lds_tile, int wave) const {
     const unsigned dst = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lds_tile + (wave * PER_WAVE + I) * 1024));
     asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :: "s"(dst), "v"(vo[I]), "s"(rs), "s"(tile_byte_offset) : "memory");
+                 :: "s"(dst), "v"(vo[I]), "s"(rs), "s"(tile_byte_offset) : "memory", "m0");
   }
   // same, with the wave's first LDS destination given as a scalar byte address (keeps the address
   // arithmetic on the scalar unit)
   template <int I>
   __device__ __forceinline__ void issue_one_at(u32x4 rs, unsigned tile_byte_offset, unsigned wave_dst) const {
     asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                 :: "s"(wave_dst + I * 1024), "v"(vo[I]), "s"(rs), "s"(tile_byte_offset) : "memory");
+                 :: "s"(wave_dst + I * 1024), "v"(vo[I]), "s"(rs), "s"(tile_byte_offset) : "memory", "m0");
   }
   __device__ __forceinline__ void issue(u32x4 rs, unsigned tile_byte_offset, unsigned char* lds_tile, int wave) const {
     tile_byte_offset = __builtin_amdgcn_readfirstlane(tile_byte_offset);
@@ -282,11 +282,11 @@ __device__ __forceinline__ void dma_dword(u32x4 rs, unsigned byte_offset, unsign
   const unsigned d = __builtin_amdgcn_readfirstlane((unsigned)(size_t)dst);
   byte_offset = __builtin_amdgcn_readfirstlane(byte_offset);
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, %3 offen lds"
-               :: "s"(d), "v"((unsigned)lane * 4u), "s"(rs), "s"(byte_offset) : "memory");
+               :: "s"(d), "v"((unsigned)lane * 4u), "s"(rs), "s"(byte_offset) : "memory", "m0");
 }
 __device__ __forceinline__ void dma_dword_at(u32x4 rs, unsigned byte_offset, unsigned dst, int lane) {
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, %3 offen lds"
-               :: "s"(dst), "v"((unsigned)lane * 4u), "s"(rs), "s"(byte_offset) : "memory");
+               :: "s"(dst), "v"((unsigned)lane * 4u), "s"(rs), "s"(byte_offset) : "memory", "m0");
 }
 // The same transposition as transpose_tile, cut into steps that can be placed between MFMAs: read() fetches
 // this thread's 4-row x 8-column block, write(J) stores column pair member J (0..7) as 8 bytes.  Threads
@@ -610,8 +610,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         const int kvcol = wkv0 + ln;
         f32x16 s[2], dp[2];
         v8 pf[2][2], df[2][2];
-        f32x4 rowv[2][2];  // per P group: LSE of four query rows, requested two slots before use
-        f32x4 nd[4];       // -delta of the 16 rows a lane holds of a query block, requested before its dP
+        // -LSE (log2 units) and -delta of the 16 rows a lane holds of either query block.  LDS reads return in
+        // order, so each group is requested a ring depth or more before its first use: waiting for it then waits
+        // for no fragment that is not due anyway
+        f32x4 nl0[4], nl1[4], nd0[4], nd1[4];
 
         auto frag = [&](auto I) -> v8 {
           constexpr int i = decltype(I)::value;
@@ -635,6 +637,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
             } else if constexpr (ks == 0) {
               // dP starts from -delta of its rows (C layout: value v belongs to row 8 (v/4) + 4 g + v%4), so
               // that dS = P o dP needs no subtraction
+              const f32x4 (&nd)[4] = qb == 0 ? nd0 : nd1;
               const f32x16 init = {nd[0][0], nd[0][1], nd[0][2], nd[0][3], nd[1][0], nd[1][1], nd[1][2], nd[1][3],
                                    nd[2][0], nd[2][1], nd[2][2], nd[2][3], nd[3][0], nd[3][1], nd[3][2], nd[3][3]};
               dp[qb] = MT<T>::mfma32(f, vf[ks], init);
@@ -653,21 +656,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         auto valu = [&](auto I, auto START, auto QBc, auto IS_Pc) {
           constexpr int i = decltype(I)::value, st = decltype(START)::value, qb = decltype(QBc)::value;
           constexpr bool IS_P = decltype(IS_Pc)::value;
-          constexpr int GI = qb;
           constexpr int QS = 4 / EPS;  // slots per quad of rows
-          // request the LSE of quad vq two slots before its first element (slot st + QS vq)
-          if constexpr (IS_P && i + 2 >= st && i + 2 < st + VL && (i + 2 - st) % QS == 0) {
-            constexpr int vq = (i + 2 - st) / QS;
-            rowv[GI][vq & 1] = *(const f32x4*)(lsel + qb * 32 + 8 * vq + 4 * g);
-          }
           if constexpr (i >= st && i < st + VL) {
             constexpr int k = i - st, vq = k / QS;
-            const f32x4 r4 = IS_P ? rowv[GI][vq & 1] : f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int e2 = 0; e2 < EPS; e2++) {
               const int e = EPS * (k % QS) + e2, v = 4 * vq + e;
               if constexpr (IS_P) {
-                float pv = fast_exp2(__builtin_fmaf(s[qb][v], c, -r4[e]));
+                const f32x4 (&nl)[4] = qb == 0 ? nl0 : nl1;
+                float pv = fast_exp2(__builtin_fmaf(s[qb][v], c, nl[vq][e]));
                 if (MASKED) {
                   const int r = qb * 32 + 8 * vq + 4 * g + e;
                   const int qrow = qi0 + r;
@@ -727,10 +724,19 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
             else dma_dword_at(nx.rr, nx.offr, dma_r, lane);
           }
           if constexpr (COMPUTE) {
-            if constexpr (i + 2 == 2 * K || i + 2 == 3 * K) {
-              constexpr int qb = (i + 2 - 2 * K) / K;
+            if constexpr (i == 0) {
 #pragma unroll
-              for (int vq = 0; vq < 4; vq++) nd[vq] = *(const f32x4*)(deltal + qb * 32 + 8 * vq + 4 * g);
+              for (int vq = 0; vq < 4; vq++) nl0[vq] = *(const f32x4*)(lsel + 8 * vq + 4 * g);
+            }
+            if constexpr (i == K) {
+#pragma unroll
+              for (int vq = 0; vq < 4; vq++) nl1[vq] = *(const f32x4*)(lsel + 32 + 8 * vq + 4 * g);
+#pragma unroll
+              for (int vq = 0; vq < 4; vq++) nd0[vq] = *(const f32x4*)(deltal + 8 * vq + 4 * g);
+            }
+            if constexpr (i == 2 * K) {
+#pragma unroll
+              for (int vq = 0; vq < 4; vq++) nd1[vq] = *(const f32x4*)(deltal + 32 + 8 * vq + 4 * g);
             }
             if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
             mma(I, fr[i % NF]);
@@ -815,7 +821,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
           for (int vq = 0; vq < 4; vq++) {
             const f32x4 l4 = *(const f32x4*)(lsel + qb * 32 + 8 * vq + 4 * g);
 #pragma unroll
-            for (int e = 0; e < 4; e++) sacc[qb][4 * vq + e] = fast_exp2(__builtin_fmaf(sacc[qb][4 * vq + e], c, -l4[e]));
+            for (int e = 0; e < 4; e++) sacc[qb][4 * vq + e] = fast_exp2(__builtin_fmaf(sacc[qb][4 * vq + e], c, l4[e]));  // l4 = -LSE
           }
         if (need_mask) {  // separate pass: the common unmasked tile carries no per-element branches
 #pragma unroll
@@ -870,6 +876,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   // every LDS-writing load of this wave has landed before it leaves (the last ones write zeros nobody reads,
   // but they must not outlive the workgroup's LDS allocation)
   __builtin_amdgcn_s_waitcnt(0);
+  // The accumulating MFMAs are opaque assembly (mfma32_acc): the compiler does not know that dkacc / dvacc come
+  // out of a 16-pass matrix instruction and inserts no wait states before reading them.  Make the distance
+  // explicit (the longest MFMA-write -> VALU-read hazard is 18 wait states).
+  asm volatile("s_nop 15\n\ts_nop 3" ::: "memory");
   // ---- epilogue: lane = kv row, 4 consecutive head-dim values per store
   const int row = wkv0 + ln;
   if (row < Skv) {
