@@ -9,6 +9,8 @@ Pinning status (what each function is checked against in tests/test_oracle.py, w
 reference, which needs torch_xla / jax / omegaconf):
 
   rms_norm                  F.rms_norm, fp64 numpy brute force, invariants          pinned
+  rms_norm_grads_eager_order  torch autograd through rms_norm itself (bf16 and fp32), explicit
+                            sum_rows dy * round(x_hat) loop                          pinned
   default/llama3 inv_freq   closed form; llm.c loop restated from torchprime/tests/test_rope.py:83-108;
                             transformers ROPE_INIT_FUNCTIONS["llama3"] when installed   pinned
   yarn inv_freq             transformers ROPE_INIT_FUNCTIONS["yarn"] when installed; closed-form
@@ -19,6 +21,11 @@ reference, which needs torch_xla / jax / omegaconf):
   eager_attention           F.scaled_dot_product_attention, brute-force loops       pinned
   attention_ref             eager_attention (causal), block-diagonal decomposition for segments,
                             brute force incl. fully-masked rows                     pinned
+  llama_attention           the pieces above composed; HF LlamaAttention when installed    pinned
+  mixtral_attention         equals llama_attention with tables taken at position_ids; shifted ids  pinned
+  deepseek_v3_attention     brute-force per-head loops with the rotary part as a complex rotation of
+                            adjacent pairs (independent of the [evens|odds] layout); attention_ref with
+                            k_rot expanded by hand; gradient of k_rot = sum over heads       pinned
   segment masking vs the reference's TPU splash kernel numerics                     PARITY UNPINNED:
                             no reference test exercises decoder_segment_ids and the Pallas kernel is
                             not in the tree; semantics are the closed form
@@ -45,6 +52,18 @@ def rms_norm(hidden_states: torch.Tensor, weight: torch.Tensor, eps: float) -> t
   variance = h.pow(2).mean(-1, keepdim=True)
   h = h * torch.rsqrt(variance + eps)
   return weight * h.to(input_dtype)
+
+
+def rms_norm_grads_eager_order(x: torch.Tensor, weight: torch.Tensor, dy: torch.Tensor, eps: float):
+  """(dx, dw) autograd returns for ``rms_norm`` above, evaluated in fp64: the normalised value is rounded to
+  the input dtype before the weight multiply (model/llama/model.py:51-52) and the cast passes gradients
+  straight through, so ``dw = sum_rows dy * round(x_hat)`` while ``dx`` flows through the unrounded x_hat."""
+  x64 = x.double().requires_grad_(True)
+  w64 = weight.double().requires_grad_(True)
+  h = x64 * torch.rsqrt(x64.pow(2).mean(-1, keepdim=True) + eps)
+  h_rounded = h + (h.detach().to(x.dtype).double() - h.detach())  # value of the cast, gradient of the identity
+  (w64 * h_rounded).backward(dy.double())
+  return x64.grad, w64.grad
 
 
 def rms_norm_exact(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
@@ -245,3 +264,74 @@ def llama_attention_block(x, w_norm, wq, wk, wv, wo, n_heads, n_kv_heads, eps, t
   o = eager_attention(q, k, v, mask)
   o = o.transpose(1, 2).contiguous().reshape(B, S, hidden)
   return o @ wo.T
+
+
+def llama_attention(x, wq, wk, wv, wo, n_heads, n_kv_heads, cos, sin, attention_mask="causal"):
+  """``LlamaAttention.forward`` (model/llama/model.py:206-238): q/k/v projections, head split, RoPE with the
+  given (batch, seq, dim) tables, eager attention, head merge, output projection."""
+  B, S, hidden = x.shape
+  hd = hidden // n_heads
+  q = (x @ wq.T).view(B, S, n_heads, hd).transpose(1, 2)
+  k = (x @ wk.T).view(B, S, n_kv_heads, hd).transpose(1, 2)
+  v = (x @ wv.T).view(B, S, n_kv_heads, hd).transpose(1, 2)
+  q, k = apply_rotary_pos_emb(q, k, cos, sin)
+  mask = causal_additive_mask(S, x.dtype) if isinstance(attention_mask, str) else attention_mask
+  o = eager_attention(q, k, v, mask)
+  return o.transpose(1, 2).contiguous().reshape(B, S, hidden) @ wo.T
+
+
+def mixtral_attention(x, wq, wk, wv, wo, n_heads, n_kv_heads, rope_theta, max_position_embeddings, position_ids,
+                      attention_mask="causal", table_dtype=None, act_dtype=None):
+  """``MixtralAttention.forward`` (model/mixtral/model.py:208-243) with its rotary module
+  (model/mixtral/model.py:62-103): cos/sin tables of ``max_position_embeddings`` rows cached in the default
+  dtype at construction (``table_dtype``), sliced to the sequence, cast to the activations' dtype (``act_dtype``;
+  ``x.dtype`` unless the block is being evaluated in higher precision than the model runs in) and gathered by
+  ``position_ids`` (model/mixtral/model.py:136-137)."""
+  B, S, hidden = x.shape
+  hd = hidden // n_heads
+  q = (x @ wq.T).view(B, S, n_heads, hd).transpose(1, 2)
+  k = (x @ wk.T).view(B, S, n_kv_heads, hd).transpose(1, 2)
+  v = (x @ wv.T).view(B, S, n_kv_heads, hd).transpose(1, 2)
+  inv_freq = 1.0 / (rope_theta ** (torch.arange(0, hd, 2, dtype=torch.int64).float() / hd))
+  t = torch.arange(max(max_position_embeddings, S), dtype=torch.int64).type_as(inv_freq)
+  emb = torch.cat((torch.outer(t, inv_freq),) * 2, dim=-1)
+  table_dtype = x.dtype if table_dtype is None else table_dtype
+  act_dtype = x.dtype if act_dtype is None else act_dtype
+  cos = emb.cos().to(table_dtype)[:S].to(act_dtype).to(x.dtype)
+  sin = emb.sin().to(table_dtype)[:S].to(act_dtype).to(x.dtype)
+  q, k = apply_rotary_pos_emb(q, k, cos, sin, position_ids, gather=True)
+  mask = causal_additive_mask(S, x.dtype) if isinstance(attention_mask, str) else attention_mask
+  o = eager_attention(q, k, v, mask)
+  return o.transpose(1, 2).contiguous().reshape(B, S, hidden) @ wo.T
+
+
+def deepseek_v3_attention(x, w, n_heads, qk_nope_head_dim, qk_rope_head_dim, v_head_dim, kv_lora_rank, cos, sin,
+                          rope_interleave=True, eps=1e-6, attention_mask="causal"):
+  """``DeepseekV3Attention.forward`` (model/deepseek_v3/model.py:403-455), multi-headed latent attention.
+  ``w`` holds ``q_a_proj, q_a_layernorm, q_b_proj`` (or ``q_proj`` when there is no q latent),
+  ``kv_a_proj_with_mqa, kv_a_layernorm, kv_b_proj, o_proj``.  The latent norms use the class default eps 1e-6
+  (model/deepseek_v3/model.py:373, 383); the single rotated k head is expanded to every head (:444); the
+  softmax scale is 1/sqrt(v_head_dim) because AttentionModule takes it from v (attention.py:54-58)."""
+  B, S, _ = x.shape
+  qk_head_dim = qk_nope_head_dim + qk_rope_head_dim
+  if "q_proj" in w:
+    q = x @ w["q_proj"].T
+  else:
+    q = rms_norm(x @ w["q_a_proj"].T, w["q_a_layernorm"], eps) @ w["q_b_proj"].T
+  q = q.view(B, S, -1, qk_head_dim).transpose(1, 2)
+  q_pass, q_rot = torch.split(q, [qk_nope_head_dim, qk_rope_head_dim], dim=-1)
+  ckv = x @ w["kv_a_proj_with_mqa"].T
+  k_pass, k_rot = torch.split(ckv, [kv_lora_rank, qk_rope_head_dim], dim=-1)
+  k_pass = (rms_norm(k_pass, w["kv_a_layernorm"], eps) @ w["kv_b_proj"].T).view(B, S, -1, qk_nope_head_dim + v_head_dim).transpose(1, 2)
+  k_pass, v = torch.split(k_pass, [qk_nope_head_dim, v_head_dim], dim=-1)
+  k_rot = k_rot.view(B, 1, S, qk_rope_head_dim)
+  if rope_interleave:
+    q_rot, k_rot = apply_rotary_pos_emb_interleave(q_rot, k_rot, cos, sin)
+  else:
+    q_rot, k_rot = apply_rotary_pos_emb(q_rot, k_rot, cos, sin)
+  k_rot = k_rot.expand(*k_pass.shape[:-1], -1)
+  q = torch.cat((q_pass, q_rot), dim=-1)
+  k = torch.cat((k_pass, k_rot), dim=-1)
+  mask = causal_additive_mask(S, x.dtype) if isinstance(attention_mask, str) else attention_mask
+  o = eager_attention(q, k, v, mask)
+  return o.transpose(1, 2).contiguous().reshape(B, S, -1) @ w["o_proj"].T

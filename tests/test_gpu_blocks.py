@@ -1,0 +1,140 @@
+"""GPU parity of the callers: ``LlamaAttention``, ``MixtralAttention`` and ``DeepseekV3Attention`` built from the
+package (projections are stock ``nn.Linear``; RMSNorm, RoPE and attention are the HIP kernels), same weights as the
+CPU oracle's restatement of the reference's modules, forward and the gradients of the input and of every weight.
+
+bf16 modules against the oracle in fp64 on the same bf16-rounded inputs and weights.  Activations (block output,
+input gradient) meet the kernels' own bounds, relative-L2 1e-2 and 2e-2 + 2^-7 |ref| per element, through the
+three to five bf16 GEMMs a block chains around them.  Weight gradients come out of stock bf16 GEMMs that sum
+batch x seq products of already rounded operands: relative-L2 1e-2, and every element within two bf16 ulps of the
+tensor's largest value (2^-6 |ref|_inf)."""
+
+import pytest
+import torch
+
+import torchprime_amd as tpa
+from oracle import tprime_oracle as orc
+from tests.util import assert_close, randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+DT = torch.bfloat16
+
+
+def _load(module, weights):
+  """weights: name -> bf16 CPU tensor; copies into the module's parameters (state-dict names of the reference)."""
+  sd = module.state_dict()
+  assert set(sd.keys()) == set(weights.keys()), (sorted(sd.keys()), sorted(weights.keys()))
+  module.load_state_dict({k: v.to(DEV) for k, v in weights.items()})
+
+
+def _compare(y, y_ref, x, x_ref, params, refs, do, rel_l2=1e-2):
+  y.backward(do.to(DEV))
+  y_ref.backward(do.double())
+  assert_close(y, y_ref, "out", scale_abs=True, rel_l2=rel_l2)
+  assert_close(x.grad, x_ref.grad, "dx", scale_abs=True, rel_l2=rel_l2)
+  for name, p in params.items():
+    assert p.grad is not None, name
+    ref = refs[name].grad
+    assert_close(p.grad, ref, f"d{name}", max_abs=max(2e-2, 2.0**-6 * ref.abs().max().item()), rel_l2=rel_l2)
+
+
+def _cfg(**kw):
+  base = dict(attention_dropout=False, attention_bias=False)
+  base.update(kw)
+  return tpa.Config(base)
+
+
+@pytest.mark.parametrize("kernel,Hkv", [("flash_attention", 8), ("splash_attention", 2), (None, 8)])
+def test_llama_attention_module(kernel, Hkv):
+  # benchmark configuration 1's block shape (B=2, S=128, hidden 512, 8 heads of 64), plus a GQA variant
+  B, S, hidden, H, hd = 2, 128, 512, 8, 64
+  cfg = _cfg(attention_kernel=kernel, hidden_size=hidden, num_attention_heads=H, num_key_value_heads=Hkv)
+  m = tpa.LlamaAttention(cfg).to(DEV).to(DT)
+  w = {
+    "q_proj.weight": randn((hidden, hidden), 1, DT, 0.02), "k_proj.weight": randn((Hkv * hd, hidden), 2, DT, 0.02),
+    "v_proj.weight": randn((Hkv * hd, hidden), 3, DT, 0.02), "o_proj.weight": randn((hidden, hidden), 4, DT, 0.02),
+  }
+  _load(m, w)
+  x = randn((B, S, hidden), 5, DT)
+  do = randn((B, S, hidden), 6, DT)
+  pos = torch.arange(S)[None].float()
+  rot = tpa.LlamaRotaryEmbedding(hd, 500000.0).to(DEV)
+  xg = x.to(DEV).requires_grad_(True)
+  cos, sin = rot(xg, pos.to(DEV))
+  mask = orc.causal_additive_mask(S).to(DEV) if kernel is None else None
+  y = m(xg, (cos, sin), mask)
+  assert y.shape == (B, S, hidden) and y.dtype == DT
+
+  c_ref, s_ref = orc.rotary_cos_sin(orc.llama3_rope_frequencies(hd, 500000.0), pos, DT)
+  assert torch.equal(cos.cpu(), c_ref) or (cos.cpu().float() - c_ref.float()).abs().max() <= 8e-3
+  x64 = x.double().requires_grad_(True)
+  r = {k: v.double().requires_grad_(True) for k, v in w.items()}
+  y_ref = orc.llama_attention(x64, r["q_proj.weight"], r["k_proj.weight"], r["v_proj.weight"], r["o_proj.weight"], H, Hkv,
+                              cos.cpu().double(), sin.cpu().double())
+  _compare(y, y_ref, xg, x64, dict(m.named_parameters()), r, do)
+
+
+@pytest.mark.parametrize("table_default", [torch.float32, torch.bfloat16])
+def test_mixtral_attention_module(table_default):
+  B, S, hidden, H, Hkv, hd = 2, 160, 512, 8, 2, 64
+  cfg = _cfg(attention_kernel="splash_attention", hidden_size=hidden, num_attention_heads=H, num_key_value_heads=Hkv,
+             max_position_embeddings=256, rope_theta=1e6)
+  old = torch.get_default_dtype()
+  torch.set_default_dtype(table_default)  # the rotary cache takes the default dtype at construction (train.py:66 sets bf16)
+  try:
+    m = tpa.MixtralAttention(cfg)
+  finally:
+    torch.set_default_dtype(old)
+  m = m.to(DEV).to(DT)
+  w = {
+    "q_proj.weight": randn((hidden, hidden), 11, DT, 0.02), "k_proj.weight": randn((Hkv * hd, hidden), 12, DT, 0.02),
+    "v_proj.weight": randn((Hkv * hd, hidden), 13, DT, 0.02), "o_proj.weight": randn((hidden, hidden), 14, DT, 0.02),
+  }
+  _load(m, w)
+  x, do = randn((B, S, hidden), 15, DT), randn((B, S, hidden), 16, DT)
+  pos = torch.stack([torch.arange(S), torch.arange(S).flip(0)])  # per-batch ids, the second row reversed
+  xg = x.to(DEV).requires_grad_(True)
+  y = m(xg, None, pos.to(DEV))
+  x64 = x.double().requires_grad_(True)
+  r = {k: v.double().requires_grad_(True) for k, v in w.items()}
+  y_ref = orc.mixtral_attention(x64, r["q_proj.weight"], r["k_proj.weight"], r["v_proj.weight"], r["o_proj.weight"], H, Hkv,
+                                1e6, 256, pos, table_dtype=table_default, act_dtype=DT)
+  # (the oracle rotates in fp64 with the table values the model sees: cached in table_default, cast to bf16)
+  _compare(y, y_ref, xg, x64, dict(m.named_parameters()), r, do)
+
+
+@pytest.mark.parametrize("q_lora,interleave", [(1536, True), (None, True), (1536, False)])
+def test_deepseek_v3_attention_module(q_lora, interleave):
+  # head and latent dims of configs/model/deepseek-v3.yaml (128 + 64 rotated q/k dims, v 128, latents 1536 / 512);
+  # 8 heads and hidden 1024 keep the fp64 oracle quick
+  B, S, hidden, H, nope, rope, vd, kvl = 1, 256, 1024, 8, 128, 64, 128, 512
+  cfg = _cfg(attention_kernel="splash_attention", hidden_size=hidden, num_attention_heads=H, num_key_value_heads=H,
+             q_lora_rank=q_lora, kv_lora_rank=kvl, qk_rope_head_dim=rope, qk_nope_head_dim=nope, v_head_dim=vd,
+             qk_head_dim=nope + rope, head_dim=rope, rope_interleave=interleave, rope_theta=10000.0,
+             max_position_embeddings=4096, rms_norm_eps=1e-6,
+             rope_scaling=dict(beta_fast=32, beta_slow=1, factor=40, mscale=1.0, mscale_all_dim=1.0,
+                               original_max_position_embeddings=4096, rope_type="yarn", type="yarn"))
+  m = tpa.DeepseekV3Attention(cfg).to(DEV).to(DT)
+  w = {
+    "kv_a_proj_with_mqa.weight": randn((kvl + rope, hidden), 21, DT, 0.02), "kv_a_layernorm.weight": (1 + randn((kvl,), 22, torch.float32, 0.1)).to(DT),
+    "kv_b_proj.weight": randn((H * (nope + vd), kvl), 23, DT, 0.02), "o_proj.weight": randn((hidden, H * vd), 24, DT, 0.02),
+  }
+  if q_lora:
+    w.update({"q_a_proj.weight": randn((q_lora, hidden), 25, DT, 0.02), "q_a_layernorm.weight": (1 + randn((q_lora,), 26, torch.float32, 0.1)).to(DT),
+              "q_b_proj.weight": randn((H * (nope + rope), q_lora), 27, DT, 0.02)})
+  else:
+    w["q_proj.weight"] = randn((H * (nope + rope), hidden), 28, DT, 0.02)
+  _load(m, w)
+  x, do = randn((B, S, hidden), 29, DT), randn((B, S, hidden), 30, DT)
+  pos = torch.arange(S)[None].float()
+  rot = tpa.DeepseekV3RotaryEmbedding(cfg).to(DEV)
+  xg = x.to(DEV).requires_grad_(True)
+  cos, sin = rot(xg, pos.to(DEV))
+  y = m(xg, (cos, sin))
+  assert y.shape == (B, S, hidden)
+
+  x64 = x.double().requires_grad_(True)
+  r = {k: v.double().requires_grad_(True) for k, v in w.items()}
+  y_ref = orc.deepseek_v3_attention(x64, {k.replace(".weight", ""): v for k, v in r.items()}, H, nope, rope, vd, kvl,
+                                    cos.cpu().double(), sin.cpu().double(), rope_interleave=interleave)
+  _compare(y, y_ref, xg, x64, dict(m.named_parameters()), r, do)

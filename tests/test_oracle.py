@@ -43,6 +43,33 @@ def test_rms_norm_invariants_and_rounding_order():
 
 
 # ---- inverse frequencies -------------------------------------------------------------------------------
+
+def test_rms_norm_eager_order_grads_match_autograd_and_explicit_sum():
+  """The gradient the reference's autograd produces: dw sums dy * (normalised value ROUNDED to the input dtype)."""
+  g = torch.Generator().manual_seed(3)
+  for dtype in (torch.bfloat16, torch.float32):
+    x = torch.randn((6, 40, 64), generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn((64,), generator=g)).to(dtype)
+    dy = torch.randn((6, 40, 64), generator=g).to(dtype)
+    dx, dw = orc.rms_norm_grads_eager_order(x, w, dy, 1e-5)
+    # explicit form of dw
+    h = x.double() * torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + 1e-5)
+    dw_explicit = (dy.double() * h.to(dtype).double()).sum((0, 1))
+    torch.testing.assert_close(dw, dw_explicit, rtol=1e-12, atol=1e-12)
+    # torch's own autograd through the eager expression in the input dtype (its sums round, hence the tolerance)
+    xa, wa = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    orc.rms_norm(xa, wa, 1e-5).backward(dy)
+    tol = dict(rtol=2e-2, atol=0.3) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(wa.grad.double(), dw, **tol)
+    torch.testing.assert_close(xa.grad.double(), dx, **(dict(rtol=2e-2, atol=3e-2) if dtype == torch.bfloat16 else tol))
+    if dtype == torch.float32:
+      # fp32 input: the cast only rounds fp64 to fp32, so dw agrees with the exact-math gradient to fp32 precision
+      # and dx, which does not see the rounded value, exactly
+      x64, w64 = x.double().requires_grad_(True), w.double().requires_grad_(True)
+      orc.rms_norm_exact(x64, w64, 1e-5).backward(dy.double())
+      torch.testing.assert_close(dw, w64.grad, rtol=1e-5, atol=1e-5)
+      torch.testing.assert_close(dx, x64.grad, rtol=1e-12, atol=1e-12)
+
 @pytest.mark.parametrize("head_dim,theta", [(128, 500000.0), (128, 10000.0), (512, 500000.0), (64, 10000.0)])
 def test_default_frequencies_closed_form(head_dim, theta):
   f = orc.default_rope_frequencies(head_dim, theta)
@@ -315,3 +342,109 @@ def test_llama_block_matches_hf_llama_when_available():
   got = orc.llama_attention_block(x, norm.weight.detach(), attn.q_proj.weight.detach(), attn.k_proj.weight.detach(),
                                   attn.v_proj.weight.detach(), attn.o_proj.weight.detach(), 8, 8, 1e-5, 500000.0)
   torch.testing.assert_close(got, ref, rtol=1e-4, atol=1e-5)
+
+
+# ---- the callers ------------------------------------------------------------------------------------------
+def test_mixtral_attention_is_llama_attention_with_gathered_tables():
+  B, S, H, Hkv, hd = 2, 12, 4, 2, 16
+  hidden = H * hd
+  x = randn((B, S, hidden), 31).double()
+  wq, wk, wv, wo = (randn(s, 32 + i, std=0.1).double() for i, s in enumerate(((hidden, hidden), (Hkv * hd, hidden), (Hkv * hd, hidden), (hidden, hidden))))
+  theta, max_pos = 1e6, 64
+  pos = torch.arange(S)[None].expand(B, S)
+  y = orc.mixtral_attention(x, wq, wk, wv, wo, H, Hkv, theta, max_pos, pos)
+  cos, sin = orc.rotary_cos_sin(orc.default_rope_frequencies(hd, theta), torch.arange(S)[None].float(), torch.float32)
+  y_llama = orc.llama_attention(x, wq, wk, wv, wo, H, Hkv, cos.double(), sin.double())
+  torch.testing.assert_close(y, y_llama, rtol=1e-6, atol=1e-6)
+  # other per-batch position ids: the tables are read at those rows (model/mixtral/model.py:136-137).  The rotary
+  # module hands over the first S rows only (model/mixtral/model.py:100-103), so ids stay below S.
+  pos2 = torch.stack([torch.arange(S).flip(0), (torch.arange(S) * 5) % S])
+  y2 = orc.mixtral_attention(x, wq, wk, wv, wo, H, Hkv, theta, max_pos, pos2)
+  c2, s2 = orc.rotary_cos_sin(orc.default_rope_frequencies(hd, theta), pos2.float(), torch.float32)
+  torch.testing.assert_close(y2, orc.llama_attention(x, wq, wk, wv, wo, H, Hkv, c2.double(), s2.double()), rtol=1e-6, atol=1e-6)
+  assert (y2 - y).abs().max() > 1e-3
+  with pytest.raises(IndexError):  # an id beyond the rows handed over fails like the reference's cos[position_ids]
+    orc.mixtral_attention(x, wq, wk, wv, wo, H, Hkv, theta, max_pos, pos + 1)
+  # a table cached in bf16 is what reaches the rotation (trap: the default dtype at construction)
+  y_bf = orc.mixtral_attention(x, wq, wk, wv, wo, H, Hkv, theta, max_pos, pos, table_dtype=torch.bfloat16)
+  y_bf_ref = orc.llama_attention(x, wq, wk, wv, wo, H, Hkv, cos.bfloat16().double(), sin.bfloat16().double())
+  torch.testing.assert_close(y_bf, y_bf_ref, rtol=1e-6, atol=1e-6)
+
+
+def _mla_case(q_lora=True, seed=41):
+  B, S, H, nope, rope, vd, kvl, ql, hidden = 2, 10, 3, 8, 6, 8, 12, 10, 20
+  w = {
+    "kv_a_proj_with_mqa": randn((kvl + rope, hidden), seed + 1, std=0.3), "kv_a_layernorm": 1 + randn((kvl,), seed + 2, std=0.1),
+    "kv_b_proj": randn((H * (nope + vd), kvl), seed + 3, std=0.3), "o_proj": randn((hidden, H * vd), seed + 4, std=0.3),
+  }
+  if q_lora:
+    w.update({"q_a_proj": randn((ql, hidden), seed + 5, std=0.3), "q_a_layernorm": 1 + randn((ql,), seed + 6, std=0.1),
+              "q_b_proj": randn((H * (nope + rope), ql), seed + 7, std=0.3)})
+  else:
+    w["q_proj"] = randn((H * (nope + rope), hidden), seed + 8, std=0.3)
+  w = {k: v.double() for k, v in w.items()}
+  x = randn((B, S, hidden), seed).double()
+  inv = orc.default_rope_frequencies(rope, 10000.0)
+  pos = torch.arange(S)[None].float()
+  cos, sin = orc.rotary_cos_sin(inv, pos, torch.float64)
+  return x, w, (B, S, H, nope, rope, vd, kvl), cos, sin, inv
+
+
+@pytest.mark.parametrize("q_lora", [True, False])
+def test_deepseek_attention_against_brute_force_mla(q_lora):
+  """Explicit per-(batch, head, query) loops; the rotary part of the scores is computed as a complex rotation of
+  ADJACENT pairs (x_2i + i x_2i+1) e^{i p f_i}, which never builds the [evens | odds] layout."""
+  x, w, (B, S, H, nope, rope, vd, kvl), cos, sin, inv = _mla_case(q_lora)
+  y = orc.deepseek_v3_attention(x, w, H, nope, rope, vd, kvl, cos, sin, rope_interleave=True)
+
+  def rms(t, g):
+    return g * t / torch.sqrt(t.pow(2).mean(-1, keepdim=True) + 1e-6)
+
+  q = (x @ w["q_proj"].T) if not q_lora else rms(x @ w["q_a_proj"].T, w["q_a_layernorm"]) @ w["q_b_proj"].T
+  q = q.view(B, S, H, nope + rope)
+  ckv = x @ w["kv_a_proj_with_mqa"].T
+  kvb = (rms(ckv[..., :kvl], w["kv_a_layernorm"]) @ w["kv_b_proj"].T).view(B, S, H, nope + vd)
+  k_rot = ckv[..., kvl:]  # (B, S, rope), one head
+  ang = torch.arange(S)[:, None].double() * inv.double()[None]  # (S, rope/2)
+  e = torch.polar(torch.ones_like(ang), ang)
+  zq = torch.complex(q[..., nope::2], q[..., nope + 1 :: 2]) * e[None, :, None]  # (B,S,H,rope/2)
+  zk = torch.complex(k_rot[..., 0::2], k_rot[..., 1::2]) * e[None]                # (B,S,rope/2)
+  out = torch.zeros(B, S, H * vd, dtype=torch.float64)
+  for b in range(B):
+    for h in range(H):
+      for i in range(S):
+        sc = torch.empty(i + 1, dtype=torch.float64)
+        for j in range(i + 1):
+          sc[j] = (q[b, i, h, :nope] * kvb[b, j, h, :nope]).sum() + (zq[b, i, h] * zk[b, j].conj()).real.sum()
+        p = torch.softmax(sc / math.sqrt(vd), 0)  # scale from v's head dim (attention.py:54-58)
+        out[b, i, h * vd : (h + 1) * vd] = (p[:, None] * kvb[b, : i + 1, h, nope:]).sum(0)
+  # (the oracle's tables are fp32 values, the loops above use fp64 angles: agreement to fp32 precision)
+  torch.testing.assert_close(y, out @ w["o_proj"].T, rtol=1e-5, atol=5e-6)
+
+
+def test_deepseek_attention_equals_attention_ref_with_expanded_k_rot_and_k_rot_grad_sums_heads():
+  x, w, (B, S, H, nope, rope, vd, kvl), cos, sin, inv = _mla_case(True, seed=51)
+  for il in (True, False):
+    xr = x.clone().requires_grad_(True)
+    wr = {k: v.clone().requires_grad_(True) for k, v in w.items()}
+    y = orc.deepseek_v3_attention(xr, wr, H, nope, rope, vd, kvl, cos, sin, rope_interleave=il)
+    # the same pipeline by hand: k_rot copied per head (separate leaves), attention_ref instead of the eager branch
+    q = (orc.rms_norm(x @ w["q_a_proj"].T, w["q_a_layernorm"], 1e-6) @ w["q_b_proj"].T).view(B, S, H, nope + rope).transpose(1, 2)
+    ckv = x @ w["kv_a_proj_with_mqa"].T
+    kvb = (orc.rms_norm(ckv[..., :kvl], w["kv_a_layernorm"], 1e-6) @ w["kv_b_proj"].T).view(B, S, H, nope + vd).transpose(1, 2)
+    k_rot_heads = ckv[..., kvl:].view(B, 1, S, rope).repeat(1, H, 1, 1).detach().requires_grad_(True)
+    fn = orc.apply_rotary_pos_emb_interleave if il else orc.apply_rotary_pos_emb
+    q_rot, k_rot = fn(q[..., nope:], k_rot_heads, cos, sin)
+    qq, kk = torch.cat((q[..., :nope], q_rot), -1), torch.cat((kvb[..., :nope], k_rot), -1)
+    o, _ = orc.attention_ref(qq, kk, kvb[..., nope:], None, True, 1 / math.sqrt(vd), torch.float64)
+    y2 = o.transpose(1, 2).reshape(B, S, -1) @ w["o_proj"].T
+    # (the eager branch takes its softmax in fp32, attention.py:163-165: agreement to fp32 precision)
+    torch.testing.assert_close(y, y2, rtol=1e-5, atol=2e-6)
+    # gradient reaching the single rotated k head = sum over heads of the per-head gradients
+    do = randn(tuple(y.shape), 77).double()
+    y.backward(do)
+    (g_heads,) = torch.autograd.grad(y2, k_rot_heads, do)
+    g_shared = g_heads.sum(1)  # (B,S,rope): d/d(ckv[..., kvl:]) through the rotated part only
+    # route it into kv_a_proj_with_mqa's rows of the rotated dims and compare with autograd of the block
+    gw = torch.einsum("bsr,bsh->rh", g_shared, x)
+    torch.testing.assert_close(wr["kv_a_proj_with_mqa"].grad[kvl:], gw, rtol=1e-4, atol=1e-5)

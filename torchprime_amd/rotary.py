@@ -63,6 +63,10 @@ class MixtralRotaryEmbedding(nn.Module):
     self.base = base
     inv_freq = 1.0 / (self.base ** (torch.arange(0, self.dim, 2, dtype=torch.int64).float().to(device) / self.dim))
     self.register_buffer("inv_freq", inv_freq, persistent=False)
+    # The reference fills the cache here, from the fp32 frequencies, before any ``module.to(dtype)`` can round the
+    # ``inv_freq`` buffer.  This build fills it on the first GPU call, so it keeps the fp32 values out of reach of
+    # ``.to()`` (a plain attribute, not a buffer).
+    self._inv_freq_fp32 = inv_freq.detach().clone().float()
     self._cache_dtype = torch.get_default_dtype()
     self.max_seq_len_cached = 0
     self.register_buffer("cos_cached", torch.empty(0), persistent=False)
@@ -70,8 +74,8 @@ class MixtralRotaryEmbedding(nn.Module):
 
   def _set_cos_sin_cache(self, seq_len, device, dtype):
     self.max_seq_len_cached = seq_len
-    t = torch.arange(seq_len, device=device, dtype=torch.int64).type_as(self.inv_freq)[None]
-    cos, sin = ops.rope_table(self.inv_freq.to(device), t.to(device), 1.0, dtype)
+    t = torch.arange(seq_len, device=device, dtype=torch.int64).float()[None]
+    cos, sin = ops.rope_table(self._inv_freq_fp32.to(device), t, 1.0, dtype)
     self.cos_cached, self.sin_cached = cos[0], sin[0]
 
   def forward(self, x, seq_len=None):
