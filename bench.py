@@ -231,7 +231,7 @@ def bench_norm_rope(dev, iters=20):
   for name, backward in (("rope_fwd", 0), ("rope_bwd", 1)):
     ms = timed(lambda: _lib.call("tp_rope_apply", q.data_ptr(), k.data_ptr(), cos.data_ptr(), sin.data_ptr(), None,
                                  qo.data_ptr(), ko.data_ptr(), B, Hq, Hkv, S, D, _lib.strides3(q), _lib.strides3(k),
-                                 _lib.strides3(qo), _lib.strides3(ko), 0, D, 0, 0, backward, bf, st))  # fmt: skip
+                                 _lib.strides3(qo), _lib.strides3(ko), 0, D, 0, 0, 0, backward, bf, st))  # fmt: skip
     res[name] = {"ms": round(ms, 4), "GBps": round(nb / ms / 1e6, 1)}
   for v in res.values():
     v["frac_of_hbm_peak"] = round(v["GBps"] / PEAK_HBM_GBPS, 4)

@@ -89,7 +89,9 @@ int tp_rope_table(const float* inv_freq, const float* position_ids, void* cos, v
  * with each product and the sum rounded to the tensor dtype, as the eager expression does.
  *   q (B,Hq,S,D), k (B,Hkv,S,D)  strided (dim stride 1); q_out/k_out same shapes, own strides
  *   cos, sin  (Bc or T, S or T, D): row (b, s) is at  cs_b_stride*b + cs_s_stride*s  unless `pos`
- *             is given, then at  cs_s_stride * pos[b*pos_b_stride + s]  (table gather, Mixtral)
+ *             is given, then at  cs_s_stride * pos[b*pos_b_stride + s]  (table gather, Mixtral);
+ *             `table_rows` is then the number of table rows: positions are clamped to it in the
+ *             kernel (callers reject out-of-range ids first, as the reference's indexing does)
  *   interleaved != 0: x is first permuted [x0,x1,x2,...] -> [evens | odds] (DeepSeek); outputs stay
  *             in the permuted order, as in the reference
  *   backward != 0: q,k are gradients w.r.t. the outputs and q_out,k_out receive gradients w.r.t.
@@ -101,8 +103,8 @@ int tp_rope_apply(const void* q, const void* k, const void* cos, const void* sin
                   const int64_t* pos, void* q_out, void* k_out, int B, int Hq, int Hkv, int S, int D,
                   const int64_t q_strides[3], const int64_t k_strides[3],
                   const int64_t qo_strides[3], const int64_t ko_strides[3], int64_t cs_b_stride,
-                  int64_t cs_s_stride, int64_t pos_b_stride, int interleaved, int backward,
-                  int dtype, void* stream);
+                  int64_t cs_s_stride, int64_t pos_b_stride, int64_t table_rows, int interleaved,
+                  int backward, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Attention forward.  Replaces the three branches of AttentionModule.forward

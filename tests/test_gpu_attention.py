@@ -90,6 +90,20 @@ def test_segment_ids_fwd_bwd(S, lo, hi, causal):
   _check(2, 4, 2, S, 128, 128, torch.bfloat16, causal, seg=seg)
 
 
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("Dqk,Dv,dtype", [(128, 128, torch.float16), (64, 64, torch.float16), (192, 128, torch.bfloat16), (192, 128, torch.float16)])
+def test_segment_ids_other_dtypes_and_head_dims(causal, Dqk, Dv, dtype):
+  # fp16 with segment ids, and the asymmetric 192/128 heads (single-buffer dK/dV path) with segment ids / non-causal
+  seg, _ = packed_segment_ids(1, 330, 8, 120, seed=Dqk + causal)
+  _check(1, 4, 2 if Dqk != 192 else 4, 330, Dqk, Dv, dtype, causal, seg=seg)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_full_attention_wide_and_small_heads(dtype):
+  _check(1, 4, 4, 200, 192, 128, dtype, False, Skv=260)   # 192/128 non-causal, Skv != Sq
+  _check(2, 4, 2, 100, 64, 64, dtype, False, Skv=333)     # 64/64 non-causal backward, Skv != Sq
+
+
 def test_segment_ids_unsorted_and_negative_ids():
   # ids need not be sorted or non-negative: equality is all that matters
   g = torch.Generator().manual_seed(3)

@@ -191,3 +191,86 @@ def test_rotary_embedding_modules():
   cos, sin = d(x, pos)
   cr, sr = orc.rotary_cos_sin(orc.default_rope_frequencies(64, 10000.0), pos.cpu(), torch.bfloat16)
   assert (cos.cpu().float() - cr.float()).abs().max() <= 8e-3
+
+
+def test_rope_gather_rejects_positions_outside_the_table():
+  # the reference's cos[position_ids] raises IndexError (model/mixtral/model.py:136-137)
+  B, H, S, D = 1, 2, 16, 64
+  q = randn((B, S, H, D), 61, torch.bfloat16).transpose(1, 2).to(DEV)
+  inv = tpa.default_rope_frequencies(D, 1e6).to(DEV)
+  cos, sin = tpa.ops.rope_table(inv, torch.arange(S, device=DEV)[None].float(), 1.0, torch.bfloat16)
+  cos, sin = cos[0], sin[0]
+  ok = torch.arange(S, device=DEV)[None]
+  tpa.apply_rotary_pos_emb(q, q, cos, sin, ok)
+  with pytest.raises(IndexError):
+    tpa.apply_rotary_pos_emb(q, q, cos, sin, ok + 1)
+
+
+# ---- full-size cases (the benchmark's layer shape) ---------------------------------------------------------
+def test_rmsnorm_full_size_llama3_8b():
+  """x (4, 8192, 4096) bf16: 32768 rows walk the grid-stride backward with 512 partial-dw rows.  y and dx are
+  checked on a sample of rows against the oracle, dw (a sum over every row) in full."""
+  B, S, H, eps = 4, 8192, 4096, 1e-5
+  g = torch.Generator(device="cpu").manual_seed(1234 + 1)
+  x = torch.randn((B, S, H), generator=g).to(torch.bfloat16)
+  dy = torch.randn((B, S, H), generator=g).to(torch.bfloat16)
+  w = (1 + 0.1 * torch.randn((H,), generator=g)).to(torch.bfloat16)
+  xg, wg = x.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+  y = tpa.ops.rmsnorm(xg, wg, eps)
+  y.backward(dy.to(DEV))
+  rows = torch.arange(0, B * S, 97)
+  xs, dys = x.view(-1, H)[rows], dy.view(-1, H)[rows]
+  y_ref = orc.rms_norm(xs, w, eps)
+  ys = y.detach().view(-1, H)[rows.to(DEV)].cpu()
+  assert (ys != y_ref).float().mean().item() < 2e-3  # same roundings as the eager expression
+  assert_close(ys, y_ref, "y rows", rel_l2=1e-3, scale_abs=True)
+  x64 = xs.double().requires_grad_(True)
+  orc.rms_norm_exact(x64, w.double(), eps).backward(dys.double())
+  assert_close(xg.grad.view(-1, H)[rows.to(DEV)], x64.grad, "dx rows", scale_abs=True)
+  # dw over all rows, eager order (normalised value rounded to bf16), accumulated in fp64 chunk by chunk
+  dw = torch.zeros(H, dtype=torch.float64)
+  for r0 in range(0, B * S, 4096):
+    xc = x.view(-1, H)[r0 : r0 + 4096].float()
+    h = (xc * torch.rsqrt(xc.pow(2).mean(-1, keepdim=True) + eps)).to(torch.bfloat16)
+    dw += (dy.view(-1, H)[r0 : r0 + 4096].double() * h.double()).sum(0)
+  assert_close(wg.grad, dw, "dw", scale_abs=True)
+  assert torch.isfinite(y.float()).all() and torch.isfinite(xg.grad.float()).all()
+
+
+def test_rope_full_size_llama3_8b_bitwise():
+  """q (4, 32, 8192, 128) and k (4, 8, 8192, 128) bf16, (B,S,H,D) memory: identical bits to the eager expression
+  (evaluated with the oracle's function on the same device tensors, and on the host for one batch element)."""
+  B, Hq, Hkv, S, D = 4, 32, 8, 8192, 128
+  g = torch.Generator(device="cpu").manual_seed(1234 + 1)
+  q = torch.randn((B, S, Hq, D), generator=g).to(torch.bfloat16).transpose(1, 2)
+  k = torch.randn((B, S, Hkv, D), generator=g).to(torch.bfloat16).transpose(1, 2)
+  pos = torch.arange(S)[None].float()
+  cos, sin = orc.rotary_cos_sin(orc.default_rope_frequencies(D, 500000.0), pos, torch.bfloat16)
+  qd, kd, cd, sd = q.to(DEV), k.to(DEV), cos.to(DEV), sin.to(DEV)
+  qo, ko = tpa.apply_rotary_pos_emb(qd, kd, cd, sd)
+  qr, kr = orc.apply_rotary_pos_emb(qd, kd, cd, sd)
+  assert torch.equal(qo, qr) and torch.equal(ko, kr)
+  qh, kh = orc.apply_rotary_pos_emb(q[2:3], k[2:3], cos, sin)
+  assert torch.equal(qo[2:3].cpu(), qh) and torch.equal(ko[2:3].cpu(), kh)
+  # backward = the transposed rotation: also bit-identical to the eager expression with -sin
+  gq, gk = torch.ops.tprime.rope_apply(qd, kd, cd, sd, None, False, True)
+  gqr, gkr = orc.apply_rotary_pos_emb(qd, kd, cd, -sd)
+  assert torch.equal(gq, gqr) and torch.equal(gk, gkr)
+
+
+def test_rope_offsets_beyond_32_bits():
+  """A q view whose rows lie 2^18 elements apart: offsets inside one batch element pass 2^31 elements, which
+  takes the kernel instantiation with 64-bit per-lane offsets."""
+  B, H, S, D = 1, 2, 8192 + 8, 128
+  stride_s = 1 << 18
+  base = torch.empty(((S - 1) * stride_s + H * D,), dtype=torch.bfloat16, device=DEV)
+  q = base.as_strided((B, H, S, D), (0, D, stride_s, 1))
+  g = torch.Generator(device="cpu").manual_seed(5)
+  vals = torch.randn((B, H, S, D), generator=g).to(torch.bfloat16)
+  q.copy_(vals.to(DEV))
+  assert (S - 1) * stride_s >= 2**31
+  pos = torch.arange(S)[None].float()
+  cos, sin = orc.rotary_cos_sin(orc.default_rope_frequencies(D, 500000.0), pos, torch.bfloat16)
+  qo, ko = tpa.apply_rotary_pos_emb(q, q, cos.to(DEV), sin.to(DEV))
+  qr, _ = orc.apply_rotary_pos_emb(vals, vals, cos, sin)
+  assert torch.equal(qo.cpu(), qr) and torch.equal(ko.cpu(), qr)

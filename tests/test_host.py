@@ -51,8 +51,8 @@ def test_c_abi_validates_arguments_before_launching():
   assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 128, 128, z3, z3, z3, z3, 0.1, 1, 2, None) == -2  # fp32
   assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 128, 128, z3, z3, z3, z3, -1.0, 1, 0, None) == -1  # scale
   assert lib.tp_attn_fwd(p, p, p, p, p, p, 1, 2, 2, 8, 16, 128, 128, z3, z3, z3, z3, 0.1, 1, 0, None) == -1  # seg, Sq != Skv
-  assert lib.tp_rope_apply(p, None, p, p, None, p, None, 1, 2, 0, 8, 24, z3, z3, z3, z3, 0, 24, 0, 0, 0, 0, None) == -2  # D % 16
-  assert lib.tp_rope_apply(p + 2, None, p, p, None, p, None, 1, 2, 0, 8, 32, z3, z3, z3, z3, 0, 32, 0, 0, 0, 0, None) == -1  # alignment
+  assert lib.tp_rope_apply(p, None, p, p, None, p, None, 1, 2, 0, 8, 24, z3, z3, z3, z3, 0, 24, 0, 0, 0, 0, 0, None) == -2  # D % 16
+  assert lib.tp_rope_apply(p + 2, None, p, p, None, p, None, 1, 2, 0, 8, 32, z3, z3, z3, z3, 0, 32, 0, 0, 0, 0, 0, None) == -1  # alignment
   assert lib.tp_rmsnorm_bwd_workspace_bytes(32768, 4096) == 512 * 4096 * 4
   assert lib.tp_rmsnorm_bwd_workspace_bytes(10, 64) == 12 * 64 * 4
   assert lib.tp_attn_bwd_workspace_bytes(4, 32, 8192) == 2 * 4 * 32 * 8192 * 4

@@ -39,7 +39,7 @@ SIGNATURES = {
     [c_void_p] * 7
     + [c_int] * 5
     + [_I64x3] * 4
-    + [c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p],
+    + [c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p],
   ),
   "tp_attn_fwd": (
     c_int,

@@ -41,6 +41,22 @@ def _is_causal_additive_mask(mask: torch.Tensor, q_len: int, kv_len: int) -> boo
   return bool(ok.all())
 
 
+# Verdicts of the check above, keyed on the mask's storage, shape and version.  A model builds its mask once per
+# forward and hands the same tensor to every layer, so the (S x S) compare and its host sync run once per mask
+# rather than once per layer; ``kernel_config={"assume_causal_mask": True}`` skips the check altogether.
+_MASK_VERDICTS: dict = {}
+
+
+def _causal_mask_verdict(mask: torch.Tensor, q_len: int, kv_len: int) -> bool:
+  key = (mask.data_ptr(), tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask._version, q_len, kv_len)
+  hit = _MASK_VERDICTS.get(key)
+  if hit is None:
+    if len(_MASK_VERDICTS) > 16:
+      _MASK_VERDICTS.clear()
+    hit = _MASK_VERDICTS[key] = _is_causal_additive_mask(mask, q_len, kv_len)
+  return hit
+
+
 class AttentionModule(nn.Module):
   def __init__(self, config, kernel_config: dict[str, Any] | None = None):
     super().__init__()
@@ -77,7 +93,7 @@ class AttentionModule(nn.Module):
         causal = False
       else:
         assume = bool(self.kernel_config and self.kernel_config.get("assume_causal_mask"))
-        if not assume and not _is_causal_additive_mask(attention_mask, q_len, kv_seq_len):
+        if not assume and not _causal_mask_verdict(attention_mask, q_len, kv_seq_len):
           raise NotImplementedError(
             "only the causal additive mask (0 on/below the diagonal, -inf above) is supported; "
             "document masking goes through segment ids (tpu_splash_attention_jax_call_wrapper)"

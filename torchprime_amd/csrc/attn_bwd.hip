@@ -1509,6 +1509,9 @@ extern "C" int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, co
   TP_REQUIRE(sm_scale > 0.f, TP_ERR_BAD_ARG, "tp_attn_bwd: sm_scale must be positive");
   TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F16, TP_ERR_UNSUPPORTED, "tp_attn_bwd: dtype %d (bf16 and fp16 only)", dtype);
   TP_REQUIRE((int64_t)(B + 8) * Hq * ((Sq + 127) / 128 + (Skv + 127) / 128) < (1ll << 31), TP_ERR_UNSUPPORTED, "tp_attn_bwd: too many workgroups");
+  // the row-sum kernel runs one thread per 16 bytes of dO: its 1-D grid of 256-thread blocks has the same limit
+  TP_REQUIRE(Dv > 0 && ((int64_t)B * Hq * Sq * (Dv / 8) + 255) / 256 < (1ll << 31), TP_ERR_UNSUPPORTED,
+             "tp_attn_bwd: B*Hq*Sq*Dv = %lld elements of dO exceed the row-sum kernel's grid", (long long)B * Hq * Sq * Dv);
   BwdArgs a;
   a.q = q; a.k = k; a.v = v; a.out = out; a.dout = dout; a.lse = lse; a.seg = seg;
   a.dq = dq; a.dk = dk; a.dv = dv; a.delta = ws;

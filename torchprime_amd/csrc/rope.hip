@@ -65,7 +65,7 @@ struct RopeArgs {
   const void* cos;
   const void* sin;
   const int64_t* pos;
-  int64_t cs_b, cs_s, pos_b;
+  int64_t cs_b, cs_s, pos_b, table_rows;
   int B, S, D;
 };
 
@@ -95,7 +95,11 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
   T* yp = (T*)a.y[which] + b * a.ys[which][0] + (off_t)h * (off_t)a.ys[which][1] + (off_t)s * (off_t)a.ys[which][2];
   const T *cp, *sp;
   if (a.pos) {
-    const int64_t crow = a.cs_s * a.pos[b * a.pos_b + s];
+    // (positions outside the table are clamped so that no lane reads beyond it; the host side has already
+    // rejected them the way the reference's cos[position_ids] does)
+    int64_t p = a.pos[b * a.pos_b + s];
+    p = p < 0 ? 0 : (p >= a.table_rows ? a.table_rows - 1 : p);
+    const int64_t crow = a.cs_s * p;
     cp = (const T*)a.cos + crow;
     sp = (const T*)a.sin + crow;
   } else {
@@ -215,12 +219,13 @@ extern "C" int tp_rope_table(const float* inv_freq, const float* position_ids, v
 extern "C" int tp_rope_apply(const void* q, const void* k, const void* cos, const void* sin, const int64_t* pos,
                              void* q_out, void* k_out, int B, int Hq, int Hkv, int S, int D, const int64_t q_strides[3],
                              const int64_t k_strides[3], const int64_t qo_strides[3], const int64_t ko_strides[3],
-                             int64_t cs_b_stride, int64_t cs_s_stride, int64_t pos_b_stride, int interleaved,
-                             int backward, int dtype, void* stream) {
+                             int64_t cs_b_stride, int64_t cs_s_stride, int64_t pos_b_stride, int64_t table_rows,
+                             int interleaved, int backward, int dtype, void* stream) {
   TP_REQUIRE(q && q_out && cos && sin && q_strides && qo_strides, TP_ERR_BAD_ARG, "tp_rope_apply: null pointer");
   TP_REQUIRE((k == nullptr) == (Hkv == 0), TP_ERR_BAD_ARG, "tp_rope_apply: k must be NULL exactly when Hkv == 0");
   TP_REQUIRE(Hkv == 0 || (k_out && k_strides && ko_strides), TP_ERR_BAD_ARG, "tp_rope_apply: null k output/strides");
   TP_REQUIRE(B >= 0 && Hq > 0 && Hkv >= 0 && S >= 0 && D > 0, TP_ERR_BAD_ARG, "tp_rope_apply: bad shape");
+  TP_REQUIRE(!pos || table_rows > 0, TP_ERR_BAD_ARG, "tp_rope_apply: a position gather needs the table's row count");
   const int esz = dtype == TP_F32 ? 4 : 2;
   TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F16 || dtype == TP_F32, TP_ERR_UNSUPPORTED, "tp_rope_apply: unsupported dtype %d", dtype);
   const int E = 16 / esz;
@@ -238,7 +243,7 @@ extern "C" int tp_rope_apply(const void* q, const void* k, const void* cos, cons
   ok = ok && (cs_b_stride * esz) % 16 == 0 && (cs_s_stride * esz) % 16 == 0;
   TP_REQUIRE(ok, TP_ERR_BAD_ARG, "tp_rope_apply: pointers and strides must keep rows 16-byte aligned");
   a.cos = cos; a.sin = sin; a.pos = pos;
-  a.cs_b = cs_b_stride; a.cs_s = cs_s_stride; a.pos_b = pos_b_stride;
+  a.cs_b = cs_b_stride; a.cs_s = cs_s_stride; a.pos_b = pos_b_stride; a.table_rows = table_rows;
   a.B = B; a.S = S; a.D = D;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == TP_BF16) return rope_typed<bf16_t>(a, interleaved, backward, st);

@@ -154,6 +154,27 @@ def _(inv_freq, position_ids, attention_scaling, dtype):
   return c, torch.empty_like(c)
 
 
+# verdicts of the position range check, keyed on the tensor's storage, shape and version: a model hands the same
+# position_ids tensor to every layer (and to the backward of each), so the device reduction and its host sync run
+# once per tensor, not once per call
+_POS_OK: dict = {}
+
+
+def _check_positions(pos: Tensor, rows: int) -> None:
+  """``cos[position_ids]`` raises IndexError for ids outside the table (model/mixtral/model.py:136-137); so does this."""
+  key = (pos.data_ptr(), tuple(pos.shape), pos._version, rows)
+  if key in _POS_OK:
+    return
+  lo, hi = (int(v) for v in torch.stack((pos.min(), pos.max())).tolist()) if pos.numel() else (0, 0)
+  if lo < -rows or hi >= rows:
+    raise IndexError(f"position id {hi if hi >= rows else lo} is out of bounds for a rotary table of {rows} rows")
+  if lo < 0:
+    raise NotImplementedError("negative position ids (indexing the table from its end) are not supported")
+  if len(_POS_OK) > 64:
+    _POS_OK.clear()
+  _POS_OK[key] = True
+
+
 def _rope_launch(q, k, cos, sin, pos, interleaved: bool, backward: bool):
   dev = _lib.require_gpu(q, k, cos, sin, pos)
   if q.dim() != 4 or (k is not None and k.dim() != 4):
@@ -182,7 +203,8 @@ def _rope_launch(q, k, cos, sin, pos, interleaved: bool, backward: bool):
       pos = pos[None]
     if pos.shape[-1] != S or pos.shape[0] not in (1, B):
       raise ValueError(f"position_ids shape {tuple(pos.shape)} does not match (batch, seq) = ({B}, {S})")
-    cs_b, cs_s, pos_b = 0, cos.stride(0), (pos.stride(0) if pos.shape[0] == B and B > 1 else 0)
+    _check_positions(pos, cos.shape[0])
+    cs_b, cs_s, pos_b, table_rows = 0, cos.stride(0), (pos.stride(0) if pos.shape[0] == B and B > 1 else 0), cos.shape[0]
   else:
     if cos.dim() == 2:
       cos, sin = cos[None], sin[None]
@@ -190,7 +212,7 @@ def _rope_launch(q, k, cos, sin, pos, interleaved: bool, backward: bool):
       raise ValueError(f"cos/sin shape {tuple(cos.shape)} does not broadcast to (batch, seq, dim) = ({B}, {S}, {D})")
     if cos.stride(-1) != 1 or sin.stride() != cos.stride():
       cos, sin = cos.contiguous(), sin.contiguous()
-    cs_b, cs_s, pos_b = (cos.stride(0) if cos.shape[0] == B and B > 1 else 0), cos.stride(1), 0
+    cs_b, cs_s, pos_b, table_rows = (cos.stride(0) if cos.shape[0] == B and B > 1 else 0), cos.stride(1), 0, 0
   qo = _empty_like_heads(q)
   ko = _empty_like_heads(k) if k is not None else None
   z3 = _lib._I64x3(0, 0, 0)
@@ -198,7 +220,7 @@ def _rope_launch(q, k, cos, sin, pos, interleaved: bool, backward: bool):
     "tp_rope_apply", q.data_ptr(), _lib.ptr(k), cos.data_ptr(), sin.data_ptr(), _lib.ptr(pos), qo.data_ptr(),
     _lib.ptr(ko), B, Hq, 0 if k is None else k.shape[1], S, D, _lib.strides3(q),
     z3 if k is None else _lib.strides3(k), _lib.strides3(qo), z3 if k is None else _lib.strides3(ko),
-    cs_b, cs_s, pos_b, int(interleaved), int(backward), _lib.dtype_code(q.dtype), _lib.stream_ptr(dev),
+    cs_b, cs_s, pos_b, table_rows, int(interleaved), int(backward), _lib.dtype_code(q.dtype), _lib.stream_ptr(dev),
   )  # fmt: skip
   return qo, ko
 
