@@ -156,15 +156,21 @@ def bench_attention(args, dev):
     n: {"ms": round(avg[n], 4), "algorithmic_TFLOPs": round(algo[n] / (avg[n] * 1e-3) / 1e12, 2) if avg[n] > 0 else None}
     for n in names
   }
-  # HBM bytes per launch (FETCH_SIZE + WRITE_SIZE of two rocprofv3 --pmc runs of this script, each scaled by
-  # what the counter reads for the 256 MiB copy of --calib-copy); the summary with the commands is
-  # profiles/attn_fwd_bwd_llama3_8b_S8192_hbm_traffic.md.  Counters cannot be read from inside this process.
-  measured_traffic = {"attn_fwd": 9.04e8, "attn_bwd_dkdv": 9.67e9, "attn_bwd_dq": 1.2e9}
+  # HBM bytes per launch: counters cannot be read from inside this process, so the figures of the last counter
+  # runs of this script (FETCH_SIZE + WRITE_SIZE, two rocprofv3 --pmc runs, each scaled by what the counter reads
+  # for the 256 MiB copy of --calib-copy) are kept in a data file next to the summary that documents them,
+  # profiles/attn_fwd_bwd_llama3_8b_S8192_hbm_traffic.{md,json}; null when the file is absent.
+  measured_traffic = {}
+  try:
+    with open(os.path.join(ROOT, "profiles", "attn_fwd_bwd_llama3_8b_S8192_hbm_traffic.json")) as f:
+      measured_traffic = json.load(f)["hbm_bytes_per_launch"]
+  except (OSError, KeyError, ValueError):
+    pass
   dom = max(("attn_fwd", "attn_bwd_dkdv", "attn_bwd_dq"), key=lambda n: avg[n])
   achieved = algo[dom] / (avg[dom] * 1e-3) / 1e12
   roofline = {
     "bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-    "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": measured_traffic[dom], "launch_ms": round(avg[dom], 4),
+    "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": measured_traffic.get(dom), "launch_ms": round(avg[dom], 4),
     "step_frac_of_peak": round(flops_step / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
   }  # fmt: skip
   return ms_per_step, flops_step, roofline, kernels, dict(B=B, Hq=Hq, Hkv=Hkv, S=S, D=D)
@@ -238,6 +244,90 @@ def bench_norm_rope(dev, iters=20):
   return res
 
 
+def packed_segment_ids(B, S, lo, hi, seed):
+  """Rows packed with documents of uniform-random lengths lo..hi summing to S (a last piece shorter than lo joins
+  its predecessor); ids 0,1,2,... per row.  Returns the ids and the realised lengths."""
+  import torch
+
+  g = torch.Generator(device="cpu").manual_seed(seed)
+  seg = torch.empty((B, S), dtype=torch.int32)
+  lengths = []
+  for b in range(B):
+    rem, i, pos, ls = S, 0, 0, []
+    while rem > 0:
+      L = int(torch.randint(lo, hi + 1, (1,), generator=g))
+      if rem - L < lo:
+        L = rem
+      seg[b, pos : pos + L] = i
+      pos, rem, i = pos + L, rem - L, i + 1
+      ls.append(L)
+    lengths.append(ls)
+  return seg, lengths
+
+
+def bench_other_configs(dev, iters=5):
+  """The other benchmark configurations, forward + backward through the C ABI, inputs resident: packed documents
+  (configuration 3), the Llama-3-70B layer (4) and the DeepSeek-V3 head dims (5).  FLOPs are counted like the
+  headline: 3 x 2 * Hq * (dqk + dv) * (allowed query/key pairs)."""
+  import torch
+
+  from torchprime_amd import _lib
+
+  lib = _lib.load()
+  res = {}
+  cases = [
+    ("llama3_8b_packed_segments", 4, 32, 8, 8192, 128, 128, True),
+    ("llama3_70b_layer", 1, 64, 8, 8192, 128, 128, False),
+    ("deepseek_v3_heads", 1, 128, 128, 4096, 192, 128, False),
+  ]
+  for name, B, Hq, Hkv, S, Dqk, Dv, packed in cases:
+    g = torch.Generator(device="cpu").manual_seed(1236)
+
+    def mk(h, d):
+      return torch.randn((B, S, h, d), generator=g, dtype=torch.float32).to(torch.bfloat16).to(dev).transpose(1, 2)
+
+    q, k, v, do = mk(Hq, Dqk), mk(Hkv, Dqk), mk(Hkv, Dv), mk(Hq, Dv)
+    seg, pairs = None, B * S * (S + 1) // 2
+    if packed:
+      seg_cpu, lengths = packed_segment_ids(B, S, 64, 4096, 1236)
+      seg = seg_cpu.to(dev)
+      pairs = sum(L * (L + 1) // 2 for row in lengths for L in row)
+    out = torch.empty((B, S, Hq, Dv), dtype=q.dtype, device=dev).transpose(1, 2)
+    lse = torch.empty((B, Hq, S), dtype=torch.float32, device=dev)
+    dq, dk, dv = (torch.empty_like(t.transpose(1, 2)).transpose(1, 2) for t in (q, k, v))
+    ws = torch.empty((lib.tp_attn_bwd_workspace_bytes(B, Hq, S) // 4,), dtype=torch.float32, device=dev)
+    st, s3, code, sm = _lib.stream_ptr(dev), _lib.strides3, _lib.dtype_code(q.dtype), 1.0 / math.sqrt(Dv)
+
+    def fwd():
+      _lib.call("tp_attn_fwd", q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.ptr(seg), out.data_ptr(), lse.data_ptr(),
+                B, Hq, Hkv, S, S, Dqk, Dv, s3(q), s3(k), s3(v), s3(out), sm, 1, code, st)  # fmt: skip
+
+    def bwd():
+      _lib.call("tp_attn_bwd", do.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                _lib.ptr(seg), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), B, Hq, Hkv, S, S, Dqk, Dv,
+                s3(do), s3(q), s3(k), s3(v), s3(out), s3(dq), s3(dk), s3(dv), sm, 1, code, st)  # fmt: skip
+
+    def timed(fn):
+      fn()
+      torch.cuda.synchronize()
+      a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+      a.record()
+      for _ in range(iters):
+        fn()
+      b.record()
+      torch.cuda.synchronize()
+      return a.elapsed_time(b) / iters
+
+    tf, tb = timed(fwd), timed(bwd)
+    flops = 3.0 * 2.0 * Hq * (Dqk + Dv) * pairs
+    tfl = flops / ((tf + tb) * 1e-3) / 1e12
+    res[name] = {"fwd_ms": round(tf, 4), "bwd_ms": round(tb, 4), "TFLOPs": round(tfl, 1),
+                 "frac_of_bf16_mfma_peak": round(tfl / PEAK_BF16_TFLOPS, 4), "allowed_pairs": pairs,
+                 "shape": dict(B=B, Hq=Hq, Hkv=Hkv, S=S, Dqk=Dqk, Dv=Dv)}  # fmt: skip
+    del q, k, v, do, out, lse, dq, dk, dv, ws
+  return res
+
+
 def cpu_baseline(max_seconds=24.0):
   """The oracle's eager attention (attention.py:151-170 restated), fwd + bwd by autograd, bf16 inputs, on
   this host's cores: one batch element and one kv-head group (4 q heads) of the benchmark workload."""
@@ -264,10 +354,33 @@ def cpu_baseline(max_seconds=24.0):
       break
   sec = (time.perf_counter() - t0) / reps
   flops = 6.0 * 1 * n_rep * S * S * D
+  # the two HBM-bound parts of the path on the same cores: eager RMSNorm fwd+bwd on 2048 rows of 4096 and eager
+  # rotate-half on q (1, 32, 2048, 128) + k (1, 8, 2048, 128), bf16 (1/16 of the layer's tensors each)
+  rows, H = 2048, 4096
+  x = torch.randn((rows, H), generator=g).to(torch.bfloat16).requires_grad_(True)
+  w = torch.ones((H,), dtype=torch.bfloat16, requires_grad=True)
+  dy = torch.randn((rows, H), generator=g).to(torch.bfloat16)
+  t0 = time.perf_counter()
+  n = 0
+  while time.perf_counter() - t0 < 2.0:
+    orc.rms_norm(x, w, 1e-5).backward(dy)
+    x.grad = w.grad = None
+    n += 1
+  norm_gbps = 5 * rows * H * 2 / ((time.perf_counter() - t0) / n) / 1e9  # fwd 2 N + bwd 3 N elements of 2 bytes
+  qr = torch.randn((1, 2048, 32, D), generator=g).to(torch.bfloat16).transpose(1, 2)
+  kr = torch.randn((1, 2048, 8, D), generator=g).to(torch.bfloat16).transpose(1, 2)
+  cos, sin = orc.rotary_cos_sin(orc.default_rope_frequencies(D, 500000.0), torch.arange(2048)[None].float(), torch.bfloat16)
+  t0 = time.perf_counter()
+  n = 0
+  while time.perf_counter() - t0 < 2.0:
+    orc.apply_rotary_pos_emb(qr, kr, cos, sin)
+    n += 1
+  rope_gbps = 2 * (qr.numel() + kr.numel()) * 2 / ((time.perf_counter() - t0) / n) / 1e9
   return {
     "value": round(flops / sec / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
     "sample": f"oracle eager attention fwd+bwd (autograd), bf16, B=1, {n_rep} q heads / 1 kv head, S={S}, d={D}: "
               f"1/32 of one step; {reps} rep(s), {sec:.2f} s each",
+    "rmsnorm_fwd_bwd_GBps": round(norm_gbps, 2), "rope_fwd_GBps": round(rope_gbps, 2),
   }  # fmt: skip
 
 
@@ -299,6 +412,8 @@ def main():
     del src, dst
   ms_per_step, flops_step, roofline, kernels, shape = bench_attention(args, dev)
   extra = None if args.no_extra else bench_norm_rope(dev)
+  if extra is not None:
+    extra["other_configs"] = bench_other_configs(dev)
   torch.cuda.empty_cache()
   cpu = None if args.no_cpu else cpu_baseline()
   value = flops_step / (ms_per_step * 1e-3) / 1e12
