@@ -70,6 +70,19 @@ int tp_rmsnorm_bwd(const void* dy, const void* x, const void* w, const float* rs
                    int64_t x_row_stride, int64_t dx_row_stride, int x_dtype, int w_dtype,
                    void* stream);
 
+/* tp_rmsnorm_bwd without a workspace argument and without any allocation.  No counterpart in the
+ * reference: it is for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  The partial-dw rows go to an array built into the library, 16 MiB of
+ * device memory per GPU the library runs on, held until the process ends; shapes whose workspace
+ * (tp_rmsnorm_bwd_workspace_bytes) exceeds it, i.e. hidden > 8192 at 512 partial rows, return
+ * TP_ERR_UNSUPPORTED.  Calls on one GPU share the array: calls that overlap in time on one GPU race.
+ * The first call on a device looks the array's address up (no allocation, but make it outside a graph
+ * capture).  Same results as tp_rmsnorm_bwd, bit for bit. */
+int tp_rmsnorm_bwd_noalloc(const void* dy, const void* x, const void* w, const float* rstd, void* dx,
+                           void* dw, int64_t rows, int hidden, int64_t dy_row_stride,
+                           int64_t x_row_stride, int64_t dx_row_stride, int x_dtype, int w_dtype,
+                           void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Rotary tables.  Replaces LlamaRotaryEmbedding.forward (model/llama/model.py:68-88) and
  * DeepseekV3RotaryEmbedding.forward (model/deepseek_v3/model.py:57-75):

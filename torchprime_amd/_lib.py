@@ -33,6 +33,10 @@ SIGNATURES = {
     c_int,
     [c_void_p] * 7 + [c_int64, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p],
   ),
+  "tp_rmsnorm_bwd_noalloc": (
+    c_int,
+    [c_void_p] * 6 + [c_int64, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p],
+  ),
   "tp_rope_table": (c_int, [c_void_p] * 4 + [c_int, c_int, c_int, c_float, c_int, c_void_p]),
   "tp_rope_apply": (
     c_int,

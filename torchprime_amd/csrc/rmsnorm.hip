@@ -5,6 +5,8 @@
 // same body at model/mixtral/model.py:53-59 and model/deepseek_v3/model.py:38-44):
 //   h = x.float(); var = mean(h*h, -1); h = h * rsqrt(var + eps); return weight * h.to(x.dtype)
 // i.e. the normalised value is rounded to the input dtype BEFORE the weight multiply.
+#include <mutex>
+
 #include "common.hpp"
 
 namespace tp {
@@ -349,4 +351,55 @@ extern "C" int tp_rmsnorm_bwd(const void* dy, const void* x, const void* w, cons
   if (x_dtype == TP_F32 && w_dtype == TP_F32) TP_GO(float, float, float);
 #undef TP_GO
   TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_rmsnorm_bwd: unsupported dtypes x=%d w=%d", x_dtype, w_dtype);
+}
+
+// ------------------------------------------------------------------------------------------------
+// The backward once more for callers that must not allocate (code under HIP graph capture, serving loops,
+// harnesses that forbid hipMalloc): the partial-dw rows live in a file-scope device array instead of a
+// caller-provided workspace.  Every GPU the library runs on holds its own copy of the array until the process
+// ends.  In host code the array's name is only a stand-in for the symbol, not a device address: the address is
+// looked up once per device (with that device current) and the kernels are given that pointer.
+// Nothing in the array has to start at zero: every partial row that the fold reads is written in full by the
+// same call first.  All calls on one GPU share the array, so calls that overlap on one GPU (two streams) race.
+// ------------------------------------------------------------------------------------------------
+namespace tp {
+constexpr int RMS_NOALLOC_MAX_HIDDEN = 8192;
+constexpr size_t RMS_NOALLOC_BYTES = (size_t)RMS_MAX_PARTS * RMS_NOALLOC_MAX_HIDDEN * sizeof(float);  // 16 MiB
+static __device__ __align__(256) unsigned char scratch[RMS_NOALLOC_BYTES];
+
+constexpr int RMS_MAX_DEVICES = 64;
+static void* g_scratch_ptr[RMS_MAX_DEVICES];  // per device, filled on the first call on that device
+static std::mutex g_scratch_mu;
+
+static int scratch_for_current_device(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  TP_REQUIRE(e == hipSuccess && dev >= 0 && dev < RMS_MAX_DEVICES, TP_ERR_LAUNCH, "tp_rmsnorm_bwd_noalloc: hipGetDevice: %s",
+             hipGetErrorString(e));
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    TP_REQUIRE(e == hipSuccess && p, TP_ERR_LAUNCH, "tp_rmsnorm_bwd_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = (float*)g_scratch_ptr[dev];
+  return TP_OK;
+}
+}  // namespace tp
+
+extern "C" int tp_rmsnorm_bwd_noalloc(const void* dy, const void* x, const void* w, const float* rstd, void* dx, void* dw,
+                                      int64_t rows, int hidden, int64_t dy_row_stride, int64_t x_row_stride,
+                                      int64_t dx_row_stride, int x_dtype, int w_dtype, void* stream) {
+  TP_REQUIRE(rows > 0 && hidden > 0, TP_ERR_BAD_ARG, "tp_rmsnorm_bwd_noalloc: bad shape rows=%lld hidden=%d", (long long)rows, hidden);
+  const size_t need = tp_rmsnorm_bwd_workspace_bytes(rows, hidden);
+  TP_REQUIRE(need <= RMS_NOALLOC_BYTES, TP_ERR_UNSUPPORTED,
+             "tp_rmsnorm_bwd_noalloc: rows=%lld hidden=%d need %zu bytes of scratch, the built-in array holds %zu "
+             "(hidden up to %d); use tp_rmsnorm_bwd with a caller-provided workspace",
+             (long long)rows, hidden, need, (size_t)RMS_NOALLOC_BYTES, RMS_NOALLOC_MAX_HIDDEN);
+  float* ws = nullptr;
+  const int rc = scratch_for_current_device(&ws);
+  if (rc) return rc;
+  return tp_rmsnorm_bwd(dy, x, w, rstd, dx, dw, ws, rows, hidden, dy_row_stride, x_row_stride, dx_row_stride, x_dtype, w_dtype,
+                        stream);
 }
