@@ -239,6 +239,60 @@ def bench_norm_rope(dev, iters=20):
                                  qo.data_ptr(), ko.data_ptr(), B, Hq, Hkv, S, D, _lib.strides3(q), _lib.strides3(k),
                                  _lib.strides3(qo), _lib.strides3(ko), 0, D, 0, 0, 0, backward, bf, st))  # fmt: skip
     res[name] = {"ms": round(ms, 4), "GBps": round(nb / ms / 1e6, 1)}
+  # Llama-4 adjacent-pair rotary on the same tensors presented as (B, S, N, D)
+  ms = timed(lambda: _lib.call("tp_rope_apply", q.data_ptr(), k.data_ptr(), cos.data_ptr(), sin.data_ptr(), None,
+                               qo.data_ptr(), ko.data_ptr(), B, Hq, Hkv, S, D, _lib.strides3(q), _lib.strides3(k),
+                               _lib.strides3(qo), _lib.strides3(ko), 0, D, 0, 0, 2, 0, bf, st))  # fmt: skip
+  res["rope_llama4_pairs_fwd"] = {"ms": round(ms, 4), "GBps": round(nb / ms / 1e6, 1)}
+  # Llama-4 qk L2 norm over the head dim of q: rows = B * S * Hq of 128
+  qrows = B * S * Hq
+  rstd_q = torch.empty((qrows,), dtype=torch.float32, device=dev)
+  ms = timed(lambda: _lib.call("tp_l2norm_fwd", q.data_ptr(), qo.data_ptr(), rstd_q.data_ptr(), qrows, D, D, D, 1e-6, bf, st))
+  res["l2norm_fwd"] = {"ms": round(ms, 4), "GBps": round(2 * q.numel() * 2 / ms / 1e6, 1)}
+  ms = timed(lambda: _lib.call("tp_l2norm_bwd", qo.data_ptr(), q.data_ptr(), rstd_q.data_ptr(), qo.data_ptr(), qrows, D, D, D, D, bf, st))
+  res["l2norm_bwd"] = {"ms": round(ms, 4), "GBps": round(3 * q.numel() * 2 / ms / 1e6, 1)}
+  del q, k, qo, ko, rstd_q
+
+  # residual add + RMSNorm in one pass: reads x and the residual, writes their sum and the normalised row
+  x2 = torch.randn((B, S, H), generator=g).to(torch.bfloat16).to(dev)
+  r2 = torch.randn((B, S, H), generator=g).to(torch.bfloat16).to(dev)
+  h2, y2, dx2 = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+  ws2 = torch.empty((_lib.load().tp_rmsnorm_bwd_workspace_bytes(rows, H),), dtype=torch.uint8, device=dev)
+  ms = timed(lambda: _lib.call("tp_add_rmsnorm_fwd", x2.data_ptr(), r2.data_ptr(), w.data_ptr(), h2.data_ptr(), y2.data_ptr(),
+                               rstd.data_ptr(), rows, H, H, H, H, H, 1e-5, bf, bf, st))  # fmt: skip
+  res["add_rmsnorm_fwd"] = {"ms": round(ms, 4), "GBps": round(4 * n * 2 / ms / 1e6, 1)}
+  ms = timed(lambda: _lib.call("tp_add_rmsnorm_bwd", x2.data_ptr(), r2.data_ptr(), h2.data_ptr(), w.data_ptr(), rstd.data_ptr(),
+                               dx2.data_ptr(), dw.data_ptr(), ws2.data_ptr(), rows, H, H, H, H, H, bf, bf, st))  # fmt: skip
+  res["add_rmsnorm_bwd"] = {"ms": round(ms, 4), "GBps": round(4 * n * 2 / ms / 1e6, 1)}
+  del x2, r2, h2, y2, dx2, ws2
+
+  # SwiGLU at the Llama-3-8B MLP width (32768 tokens x 14336): fwd reads gate, up, writes out; bwd reads three, writes two
+  I = 14336
+  gt, up, ot = (torch.randn((rows, I), generator=None, device=dev, dtype=torch.bfloat16) for _ in range(3))
+  dgt, dup = torch.empty_like(gt), torch.empty_like(gt)
+  ms = timed(lambda: _lib.call("tp_swiglu_fwd", gt.data_ptr(), up.data_ptr(), ot.data_ptr(), rows, I, I, I, I, bf, st))
+  res["swiglu_fwd"] = {"ms": round(ms, 4), "GBps": round(3 * rows * I * 2 / ms / 1e6, 1)}
+  ms = timed(lambda: _lib.call("tp_swiglu_bwd", ot.data_ptr(), gt.data_ptr(), up.data_ptr(), dgt.data_ptr(), dup.data_ptr(),
+                               rows, I, I, I, I, I, I, bf, st))  # fmt: skip
+  res["swiglu_bwd"] = {"ms": round(ms, 4), "GBps": round(5 * rows * I * 2 / ms / 1e6, 1)}
+  del gt, up, ot, dgt, dup
+
+  # shifted cross entropy over a 128256-entry vocabulary, fp32 logits of one 8192-token sequence: fwd reads the logits
+  # once, bwd reads them and writes their gradient
+  V, Sx = 128256, 8192
+  logits = torch.randn((1, Sx, V), device=dev, dtype=torch.float32)
+  labels = torch.randint(0, V, (1, Sx), device=dev)
+  lse, rl, lc = (torch.empty((n_,), dtype=torch.float32, device=dev) for n_ in (Sx, Sx, 2))
+  dl = torch.ones((1,), dtype=torch.float32, device=dev)
+  dlog = torch.empty_like(logits)
+  f32 = _lib.dtype_code(torch.float32)
+  ms = timed(lambda: _lib.call("tp_cross_entropy_fwd", logits.data_ptr(), labels.data_ptr(), lse.data_ptr(), rl.data_ptr(),
+                               lc.data_ptr(), 1, Sx, V, Sx * V, V, Sx, -100, f32, st))  # fmt: skip
+  res["cross_entropy_fwd"] = {"ms": round(ms, 4), "GBps": round(Sx * V * 4 / ms / 1e6, 1)}
+  ms = timed(lambda: _lib.call("tp_cross_entropy_bwd", logits.data_ptr(), labels.data_ptr(), lse.data_ptr(), lc.data_ptr(),
+                               dl.data_ptr(), dlog.data_ptr(), 1, Sx, V, Sx * V, V, Sx, Sx * V, V, -100, f32, st))  # fmt: skip
+  res["cross_entropy_bwd"] = {"ms": round(ms, 4), "GBps": round(2 * Sx * V * 4 / ms / 1e6, 1)}
+  del logits, dlog
   for v in res.values():
     v["frac_of_hbm_peak"] = round(v["GBps"] / PEAK_HBM_GBPS, 4)
   return res

@@ -105,8 +105,10 @@ int tp_rope_table(const float* inv_freq, const float* position_ids, void* cos, v
  *             is given, then at  cs_s_stride * pos[b*pos_b_stride + s]  (table gather, Mixtral);
  *             `table_rows` is then the number of table rows: positions are clamped to it in the
  *             kernel (callers reject out-of-range ids first, as the reference's indexing does)
- *   interleaved != 0: x is first permuted [x0,x1,x2,...] -> [evens | odds] (DeepSeek); outputs stay
+ *   interleaved == 1: x is first permuted [x0,x1,x2,...] -> [evens | odds] (DeepSeek); outputs stay
  *             in the permuted order, as in the reference
+ *   interleaved == 2: adjacent pairs (x[2i], x[2i+1]) are rotated by angle i, taken from the first half
+ *             of the cos/sin row, and stay in place (Llama-4 apply_rotary_emb, model/llama4/model.py:364-409)
  *   backward != 0: q,k are gradients w.r.t. the outputs and q_out,k_out receive gradients w.r.t.
  *             the inputs (transpose of the rotation, then the inverse permutation if interleaved)
  *   k may be NULL (Hkv = 0) to rotate a single tensor.
@@ -169,6 +171,70 @@ int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, const void* v
                    const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
                    const int64_t dv_strides[3], float sm_scale, int causal, int dtype, void* stream,
                    void* const* events);
+
+/* ------------------------------------------------------------------------------------------------
+ * The steps either side of the attention path (HBM-bound, one pass over each tensor).
+ * ---------------------------------------------------------------------------------------------- */
+
+/* Residual add fused with the RMSNorm that follows it in a decoder layer
+ * (torchprime/torch_xla_models/model/llama/model.py:288-291:
+ *     hidden_states = residual + hidden_states; residual = hidden_states;
+ *     hidden_states = self.post_attention_layernorm(hidden_states)):
+ *     h = (residual + x) rounded to x_dtype;  y = weight * (h.float() * rsqrt(mean(h^2) + eps)).to(x_dtype)
+ *   x, residual, h (rows, hidden) of x_dtype with their own row strides; y, rstd, dtypes as tp_rmsnorm_fwd */
+int tp_add_rmsnorm_fwd(const void* x, const void* residual, const void* w, void* h, void* y,
+                       float* rstd, int64_t rows, int hidden, int64_t x_row_stride,
+                       int64_t res_row_stride, int64_t h_row_stride, int64_t y_row_stride, float eps,
+                       int x_dtype, int w_dtype, void* stream);
+
+/* Its backward: dx = d(residual) = (RMSNorm backward of dy at h) rounded to x_dtype + dh, where dh is the
+ * gradient that reaches h through the residual path; dw as tp_rmsnorm_bwd.  ws: tp_rmsnorm_bwd_workspace_bytes. */
+int tp_add_rmsnorm_bwd(const void* dy, const void* dh, const void* h, const void* w, const float* rstd,
+                       void* dx, void* dw, float* ws, int64_t rows, int hidden, int64_t dy_row_stride,
+                       int64_t dh_row_stride, int64_t h_row_stride, int64_t dx_row_stride, int x_dtype,
+                       int w_dtype, void* stream);
+
+/* Llama4TextL2Norm.forward (model/llama4/model.py:104-116): y = (x.float() * rsqrt(mean(x^2, -1) + eps)).type_as(x)
+ * over rows of `dim` elements (a head dim: 16 bytes times a power of two up to 64 lanes); rstd (rows) fp32 out. */
+int tp_l2norm_fwd(const void* x, void* y, float* rstd, int64_t rows, int dim, int64_t x_row_stride,
+                  int64_t y_row_stride, float eps, int dtype, void* stream);
+/* dx = rstd * (dy - n * mean(dy * n, -1)),  n = x * rstd */
+int tp_l2norm_bwd(const void* dy, const void* x, const float* rstd, void* dx, int64_t rows, int dim,
+                  int64_t dy_row_stride, int64_t x_row_stride, int64_t dx_row_stride, int dtype,
+                  void* stream);
+
+/* Temperature scale of the Llama-4 NoPE layers (model/llama4/model.py:513-525):
+ * y[r, :] = (x[r, :] * scale[(r / heads) % seq]).to(dtype) for rows numbered (batch, position, head);
+ * `scale` (seq) fp32.  The backward is the same call on the gradient. */
+int tp_scale_rows(const void* x, const float* scale, void* y, int64_t rows, int dim, int64_t x_row_stride,
+                  int64_t y_row_stride, int heads, int seq, int dtype, void* stream);
+
+/* act_fn(gate) * up of LlamaMLP.forward (model/llama/model.py:137-139) for act_fn = SiLU:
+ * out = (silu(gate).to(dtype) * up).to(dtype), (rows, cols) tensors with their own row strides. */
+int tp_swiglu_fwd(const void* gate, const void* up, void* out, int64_t rows, int cols,
+                  int64_t gate_row_stride, int64_t up_row_stride, int64_t out_row_stride, int dtype,
+                  void* stream);
+/* dup = dout * silu(gate).to(dtype);  dgate = (dout * up).to(dtype) * silu'(gate) */
+int tp_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dgate, void* dup, int64_t rows,
+                  int cols, int64_t dout_row_stride, int64_t gate_row_stride, int64_t up_row_stride,
+                  int64_t dgate_row_stride, int64_t dup_row_stride, int dtype, void* stream);
+
+/* cross_entropy_loss (torchprime/torch_xla_models/loss.py:5-20): logits (B,S,V), labels (B,S) int64; position s
+ * of a sequence is scored against labels[b, s+1], the last position has no target, labels equal to ignore_index
+ * are skipped, the loss is the mean over the scored positions.  The shift is done by indexing (no copies).
+ *   lse, row_loss  (B*S) fp32 out: logsumexp of every row, and its loss (0 where there is no target)
+ *   loss_and_count (2) fp32 out: the mean loss, and the number of scored positions
+ *   dtype          TP_F32 or TP_BF16 logits (the models cast to fp32 first, model/llama/model.py:393) */
+int tp_cross_entropy_fwd(const void* logits, const int64_t* labels, float* lse, float* row_loss,
+                         float* loss_and_count, int B, int S, int V, int64_t logits_b_stride,
+                         int64_t logits_s_stride, int64_t labels_b_stride, int ignore_index, int dtype,
+                         void* stream);
+/* dlogits = dloss / count * (softmax(logits) - onehot(label)) on scored rows, 0 elsewhere; dloss (1) fp32 */
+int tp_cross_entropy_bwd(const void* logits, const int64_t* labels, const float* lse,
+                         const float* loss_and_count, const float* dloss, void* dlogits, int B, int S,
+                         int V, int64_t logits_b_stride, int64_t logits_s_stride,
+                         int64_t labels_b_stride, int64_t dlogits_b_stride, int64_t dlogits_s_stride,
+                         int ignore_index, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -26,6 +26,11 @@ reference, which needs torch_xla / jax / omegaconf):
   deepseek_v3_attention     brute-force per-head loops with the rotary part as a complex rotation of
                             adjacent pairs (independent of the [evens|odds] layout); attention_ref with
                             k_rot expanded by hand; gradient of k_rot = sum over heads       pinned
+  add_rms_norm, l2_norm     F.rms_norm without a weight, explicit fp64 loops                pinned
+  apply_rotary_emb_llama4   complex rotation of adjacent pairs (torch.polar), norm preservation      pinned
+  attn temperature          closed form log(floor((p+1)/f)+1) a + 1 at hand-computed positions       pinned
+  swiglu                    x * sigmoid(x) * u in fp64 loops                                          pinned
+  cross_entropy_loss        explicit per-token -log softmax loops incl. ignored labels; F.cross_entropy   pinned
   segment masking vs the reference's TPU splash kernel numerics                     PARITY UNPINNED:
                             no reference test exercises decoder_segment_ids and the Pallas kernel is
                             not in the tree; semantics are the closed form
@@ -335,3 +340,58 @@ def deepseek_v3_attention(x, w, n_heads, qk_nope_head_dim, qk_rope_head_dim, v_h
   mask = causal_additive_mask(S, x.dtype) if isinstance(attention_mask, str) else attention_mask
   o = eager_attention(q, k, v, mask)
   return o.transpose(1, 2).contiguous().reshape(B, S, -1) @ w["o_proj"].T
+
+
+# ------------------------------------------------------------------------------------------------
+# the steps either side of the attention path
+# ------------------------------------------------------------------------------------------------
+def add_rms_norm(x, residual, weight, eps):
+  """model/llama/model.py:288-291: ``h = residual + x`` (in the activation dtype), then ``rms_norm(h)``;
+  returns ``(y, h)``."""
+  h = residual + x
+  return rms_norm(h, weight, eps), h
+
+
+def l2_norm(x, eps):
+  """Llama4TextL2Norm.forward, model/llama4/model.py:104-116."""
+  xf = x.float() if x.dtype != torch.float64 else x
+  return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)).type_as(x)
+
+
+def apply_rotary_emb_llama4(q, k, cos_full, sin_full, unsqueeze_dim=2):
+  """apply_rotary_emb, model/llama4/model.py:364-409: q, k (B, S, N, D); pairs (x[2i], x[2i+1]) rotated by the
+  angle whose cos/sin are entry i of the (B, S, D) tables; results interleaved back."""
+  hd = q.size(-1)
+  c = cos_full.unsqueeze(unsqueeze_dim)[..., : hd // 2]
+  s = sin_full.unsqueeze(unsqueeze_dim)[..., : hd // 2]
+
+  def rot(t):
+    x, y = t[..., ::2], t[..., 1::2]
+    xo, yo = x * c - y * s, y * c + x * s
+    return torch.stack([xo, yo], dim=-1).reshape(t.shape).type_as(t)
+
+  return rot(q), rot(k)
+
+
+def attn_temperature_scales(seq_len, floor_scale, attn_scale):
+  """model/llama4/model.py:515-521."""
+  pos = torch.arange(seq_len).float()
+  return torch.log(torch.floor((pos + 1.0) / floor_scale) + 1.0) * attn_scale + 1.0
+
+
+def apply_attn_temperature(q, floor_scale, attn_scale):
+  """model/llama4/model.py:522-525: q (B, S, N, D) times the per-position scale, cast back to q's dtype."""
+  sc = attn_temperature_scales(q.shape[1], floor_scale, attn_scale).view(1, -1, 1, 1)
+  return (q * (sc.double() if q.dtype == torch.float64 else sc)).to(q.dtype)
+
+
+def swiglu(gate, up):
+  """``act_fn(gate_proj(x)) * up_proj(x)`` of LlamaMLP.forward (model/llama/model.py:137-139), act_fn = SiLU."""
+  return F.silu(gate) * up
+
+
+def cross_entropy_loss(logits, labels, vocab_size):
+  """loss.py:5-20."""
+  shift_logits = logits[..., :-1, :].contiguous().view(-1, vocab_size)
+  shift_labels = labels[..., 1:].contiguous().view(-1)
+  return torch.nn.CrossEntropyLoss()(shift_logits, shift_labels)

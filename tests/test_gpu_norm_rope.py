@@ -253,7 +253,7 @@ def test_rope_full_size_llama3_8b_bitwise():
   qh, kh = orc.apply_rotary_pos_emb(q[2:3], k[2:3], cos, sin)
   assert torch.equal(qo[2:3].cpu(), qh) and torch.equal(ko[2:3].cpu(), kh)
   # backward = the transposed rotation: also bit-identical to the eager expression with -sin
-  gq, gk = torch.ops.tprime.rope_apply(qd, kd, cd, sd, None, False, True)
+  gq, gk = torch.ops.tprime.rope_apply(qd, kd, cd, sd, None, 0, True)
   gqr, gkr = orc.apply_rotary_pos_emb(qd, kd, cd, -sd)
   assert torch.equal(gq, gqr) and torch.equal(gk, gkr)
 

@@ -448,3 +448,70 @@ def test_deepseek_attention_equals_attention_ref_with_expanded_k_rot_and_k_rot_g
     # route it into kv_a_proj_with_mqa's rows of the rotated dims and compare with autograd of the block
     gw = torch.einsum("bsr,bsh->rh", g_shared, x)
     torch.testing.assert_close(wr["kv_a_proj_with_mqa"].grad[kvl:], gw, rtol=1e-4, atol=1e-5)
+
+
+# ---- the steps either side of the path ----------------------------------------------------------------------
+def test_l2_norm_and_add_rms_norm_reduce_to_library_routines():
+  x = randn((3, 5, 4, 32), 61)
+  torch.testing.assert_close(orc.l2_norm(x, 1e-6), F.rms_norm(x, (32,), None, 1e-6), rtol=1e-6, atol=1e-6)
+  xb = x.bfloat16()
+  ref = torch.empty_like(x)
+  for idx in np.ndindex(3, 5, 4):
+    row = xb[idx].double()
+    ref[idx] = (row / math.sqrt((row * row).mean().item() + 1e-6)).float()
+  assert torch.equal(orc.l2_norm(xb, 1e-6), ref.bfloat16())  # fp32 math, one rounding at the end
+  h, r, w = randn((4, 7, 64), 62).bfloat16(), randn((4, 7, 64), 63).bfloat16(), (1 + randn((64,), 64, std=0.1)).bfloat16()
+  y, s = orc.add_rms_norm(h, r, w, 1e-5)
+  assert torch.equal(s, (r.float() + h.float()).bfloat16()) and torch.equal(y, orc.rms_norm(s, w, 1e-5))
+
+
+def test_llama4_rotary_is_adjacent_pair_complex_rotation():
+  B, S, N, D = 2, 9, 3, 16
+  q, k = randn((B, S, N, D), 65).double(), randn((B, S, 2, D), 66).double()
+  inv = orc.default_rope_frequencies(D, 500000.0)
+  pos = torch.arange(S)[None].float() * 5
+  cos, sin = orc.rotary_cos_sin(inv, pos, torch.float32)
+  qo, ko = orc.apply_rotary_emb_llama4(q, k, cos.double(), sin.double())
+  ang = pos[0, :, None].double() * inv.double()[None]
+  e = torch.polar(torch.ones_like(ang), ang)[None, :, None]  # (1, S, 1, D/2)
+  for x, xo in ((q, qo), (k, ko)):
+    z = torch.complex(x[..., 0::2], x[..., 1::2]) * e
+    torch.testing.assert_close(xo[..., 0::2], z.real, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(xo[..., 1::2], z.imag, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(xo.norm(dim=-1), x.norm(dim=-1), rtol=1e-6, atol=1e-6)
+
+
+def test_attn_temperature_closed_form():
+  sc = orc.attn_temperature_scales(20000, 8192.0, 0.1)
+  assert sc[0].item() == 1.0 and sc[8190].item() == 1.0  # floor((p+1)/8192) = 0 below position 8191
+  assert sc[8191].item() == pytest.approx(math.log(2.0) * 0.1 + 1.0, rel=1e-6)
+  assert sc[16383].item() == pytest.approx(math.log(3.0) * 0.1 + 1.0, rel=1e-6)
+  q = randn((2, 6, 2, 8), 67).bfloat16()
+  out = orc.apply_attn_temperature(q, 2.0, 0.5)
+  s6 = orc.attn_temperature_scales(6, 2.0, 0.5)
+  assert torch.equal(out, (q.float() * s6.view(1, 6, 1, 1)).bfloat16())
+
+
+def test_swiglu_and_cross_entropy_explicit_forms():
+  g, u = randn((5, 24), 68).double(), randn((5, 24), 69).double()
+  ref = torch.empty_like(g)
+  for i, j in np.ndindex(5, 24):
+    x = g[i, j].item()
+    ref[i, j] = x / (1.0 + math.exp(-x)) * u[i, j].item()
+  torch.testing.assert_close(orc.swiglu(g, u), ref, rtol=1e-12, atol=1e-12)
+  B, S, V = 2, 7, 11
+  logits = randn((B, S, V), 70).double()
+  labels = torch.randint(0, V, (B, S), generator=torch.Generator().manual_seed(71))
+  labels[0, 3] = -100
+  labels[1, 0] = -100  # position 0's label is never a target: no effect
+  total, n = 0.0, 0
+  for b in range(B):
+    for s in range(S - 1):
+      lab = labels[b, s + 1].item()
+      if lab == -100:
+        continue
+      row = logits[b, s]
+      total += math.log(sum(math.exp(v) for v in row.tolist())) - row[lab].item()
+      n += 1
+  assert n == B * (S - 1) - 1
+  assert orc.cross_entropy_loss(logits, labels, V).item() == pytest.approx(total / n, rel=1e-12)

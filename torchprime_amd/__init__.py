@@ -22,7 +22,16 @@ from .attention import AttentionModule, repeat_kv
 from .blocks import DeepseekV3Attention, LlamaAttention, MixtralAttention
 from .config import Config
 from .kernel_utils import SplashAttentionConfig, splash_attention_jax_wrapper, tpu_splash_attention_jax_call_wrapper
-from .norm import DeepseekV3RMSNorm, LlamaRMSNorm, MixtralRMSNorm
+from .llama4 import (
+  Llama4TextL2Norm,
+  Llama4TextRotaryEmbedding,
+  apply_attn_temperature,
+  apply_rotary_emb,
+  attn_temperature_scales,
+)
+from .loss import cross_entropy_loss
+from .mlp import LlamaMLP
+from .norm import DeepseekV3RMSNorm, LlamaRMSNorm, MixtralRMSNorm, add_rms_norm
 from .rope import RopeScaling, default_rope_frequencies, deepseek_v3_rope_init_fn, llama3_rope_frequencies
 from .rotary import (
   DeepseekV3RotaryEmbedding,
@@ -39,4 +48,6 @@ __all__ = [
   "default_rope_frequencies", "llama3_rope_frequencies", "deepseek_v3_rope_init_fn", "LlamaRotaryEmbedding",
   "MixtralRotaryEmbedding", "DeepseekV3RotaryEmbedding", "rotate_half", "apply_rotary_pos_emb",
   "apply_rotary_pos_emb_interleave", "LlamaAttention", "MixtralAttention", "DeepseekV3Attention", "Config",
+  "Llama4TextL2Norm", "Llama4TextRotaryEmbedding", "apply_rotary_emb", "attn_temperature_scales", "apply_attn_temperature",
+  "cross_entropy_loss", "LlamaMLP", "add_rms_norm",
 ]  # fmt: skip

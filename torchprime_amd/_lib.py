@@ -37,6 +37,21 @@ SIGNATURES = {
     c_int,
     [c_void_p] * 6 + [c_int64, c_int, c_int64, c_int64, c_int64, c_int, c_int, c_void_p],
   ),
+  "tp_add_rmsnorm_fwd": (
+    c_int,
+    [c_void_p] * 6 + [c_int64, c_int, c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_int, c_void_p],
+  ),
+  "tp_add_rmsnorm_bwd": (
+    c_int,
+    [c_void_p] * 8 + [c_int64, c_int, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_void_p],
+  ),
+  "tp_l2norm_fwd": (c_int, [c_void_p] * 3 + [c_int64, c_int, c_int64, c_int64, c_float, c_int, c_void_p]),
+  "tp_l2norm_bwd": (c_int, [c_void_p] * 4 + [c_int64, c_int, c_int64, c_int64, c_int64, c_int, c_void_p]),
+  "tp_scale_rows": (c_int, [c_void_p] * 3 + [c_int64, c_int, c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
+  "tp_swiglu_fwd": (c_int, [c_void_p] * 3 + [c_int64, c_int, c_int64, c_int64, c_int64, c_int, c_void_p]),
+  "tp_swiglu_bwd": (c_int, [c_void_p] * 5 + [c_int64, c_int] + [c_int64] * 5 + [c_int, c_void_p]),
+  "tp_cross_entropy_fwd": (c_int, [c_void_p] * 5 + [c_int] * 3 + [c_int64] * 3 + [c_int, c_int, c_void_p]),
+  "tp_cross_entropy_bwd": (c_int, [c_void_p] * 6 + [c_int] * 3 + [c_int64] * 5 + [c_int, c_int, c_void_p]),
   "tp_rope_table": (c_int, [c_void_p] * 4 + [c_int, c_int, c_int, c_float, c_int, c_void_p]),
   "tp_rope_apply": (
     c_int,

@@ -40,7 +40,8 @@ template <typename XT, typename WT, typename OT, int NV, int WAVES>
 __global__ __launch_bounds__(256) void rmsnorm_fwd_vec(const XT* __restrict__ x, const WT* __restrict__ w,
                                                        OT* __restrict__ y, float* __restrict__ rstd,
                                                        int64_t rows, int hidden, int64_t xs, int64_t ys,
-                                                       float eps) {
+                                                       float eps, const XT* __restrict__ res, XT* __restrict__ hsum,
+                                                       int64_t rss, int64_t hss) {
   constexpr int E = 16 / sizeof(XT);
   constexpr int RPB = 4 / WAVES, TPR = 64 * WAVES;
   __shared__ float red[4];
@@ -60,6 +61,21 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_vec(const XT* __restrict__ x,
   for (int i = 0; i < NV; i++) {
     const int v = t + TPR * i;
     load_f_nt<XT, E>(xr + (int64_t)(v < nvec ? v : nvec - 1) * E, xv[i]);
+  }
+  if (res) {
+    // fused residual add (model/llama/model.py:288-291): h = residual + x, rounded to the activation dtype as the
+    // eager add does; h is written out (it is the next residual) and normalised in place of x
+    const XT* rr = res + row * rss;
+    XT* hr = hsum + row * hss;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      const int v = t + TPR * i;
+      float rv[E];
+      load_f_nt<XT, E>(rr + (int64_t)(v < nvec ? v : nvec - 1) * E, rv);
+#pragma unroll
+      for (int e = 0; e < E; e++) xv[i][e] = round_to<XT>(rv[e] + xv[i][e]);
+      if (v < nvec) store_f_nt<XT, E>(hr + (int64_t)v * E, xv[i]);
+    }
   }
 #pragma unroll
   for (int i = 0; i < NV; i++) {
@@ -89,12 +105,18 @@ template <typename XT, typename WT, typename OT>
 __global__ __launch_bounds__(256) void rmsnorm_fwd_generic(const XT* __restrict__ x, const WT* __restrict__ w,
                                                            OT* __restrict__ y, float* __restrict__ rstd,
                                                            int64_t rows, int hidden, int64_t xs, int64_t ys,
-                                                           float eps) {
+                                                           float eps, const XT* __restrict__ res, XT* __restrict__ hsum,
+                                                           int64_t rss, int64_t hss) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const XT* xr = x + row * xs;
   OT* yr = y + row * ys;
+  if (res) {  // h = residual + x first; the wave then normalises the row it has just written
+    XT* hr = hsum + row * hss;
+    for (int c = lane; c < hidden; c += 64) hr[c] = Elem<XT>::from_f(Elem<XT>::to_f(res[row * rss + c]) + Elem<XT>::to_f(xr[c]));
+    xr = hr;
+  }
   float ss = 0.f;
   for (int c = lane; c < hidden; c += 64) {
     const float f = Elem<XT>::to_f(xr[c]);
@@ -116,7 +138,8 @@ template <typename XT, typename WT, typename OT, int NV, int WAVES>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_vec(const OT* __restrict__ dy, const XT* __restrict__ x,
                                                        const WT* __restrict__ w, const float* __restrict__ rstd,
                                                        XT* __restrict__ dx, float* __restrict__ ws, int64_t rows,
-                                                       int hidden, int64_t dys, int64_t xs, int64_t dxs) {
+                                                       int hidden, int64_t dys, int64_t xs, int64_t dxs,
+                                                       const XT* __restrict__ dres, int64_t drs) {
   constexpr int E = 16 / sizeof(XT);
   constexpr int RPB = 4 / WAVES, TPR = 64 * WAVES;
   __shared__ float red[2][4];
@@ -142,7 +165,7 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_vec(const OT* __restrict__ dy
     const XT* xr = x + row * xs;
     const OT* gr = dy + row * dys;
     XT* dr = dx + row * dxs;
-    float n[NV][E], g[NV][E];
+    float n[NV][E], g[NV][E], a[NV][E];
     float c = 0.f;
     // all loads first (out-of-range vectors re-read the row's last one), then the arithmetic
 #pragma unroll
@@ -151,6 +174,7 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_vec(const OT* __restrict__ dy
       const int64_t o = (int64_t)(v < nvec ? v : nvec - 1) * E;
       load_f_nt<XT, E>(xr + o, n[i]);
       load_f_nt<OT, E>(gr + o, g[i]);
+      if (dres) load_f_nt<XT, E>(dres + row * drs + o, a[i]);
     }
 #pragma unroll
     for (int i = 0; i < NV; i++) {
@@ -173,6 +197,12 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_vec(const OT* __restrict__ dy
         float o[E];
 #pragma unroll
         for (int e = 0; e < E; e++) o[e] = r * (g[i][e] - n[i][e] * c);
+        if (dres) {
+          // fused residual: the gradient that reached h through the residual path joins here, each addend rounded
+          // to the activation dtype first, as autograd's accumulation of two bf16 gradients does
+#pragma unroll
+          for (int e = 0; e < E; e++) o[e] = round_to<XT>(o[e]) + a[i][e];
+        }
         store_f_nt<XT, E>(dr + (int64_t)v * E, o);
       }
     }
@@ -190,7 +220,8 @@ template <typename XT, typename WT, typename OT>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_dx_generic(const OT* __restrict__ dy, const XT* __restrict__ x,
                                                               const WT* __restrict__ w, const float* __restrict__ rstd,
                                                               XT* __restrict__ dx, int64_t rows, int hidden,
-                                                              int64_t dys, int64_t xs, int64_t dxs) {
+                                                              int64_t dys, int64_t xs, int64_t dxs,
+                                                              const XT* __restrict__ dres, int64_t drs) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
@@ -205,7 +236,9 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_dx_generic(const OT* __restri
   for (int j = lane; j < hidden; j += 64) {
     const float n = Elem<XT>::to_f(xr[j]) * r;
     const float g = Elem<OT>::to_f(gr[j]) * Elem<WT>::to_f(w[j]);
-    dr[j] = Elem<XT>::from_f(r * (g - n * c));
+    float o = r * (g - n * c);
+    if (dres) o = round_to<XT>(o) + Elem<XT>::to_f(dres[row * drs + j]);
+    dr[j] = Elem<XT>::from_f(o);
   }
 }
 // backward dw partials, any hidden: thread = column, rows p, p+P, ...
@@ -249,17 +282,20 @@ __global__ __launch_bounds__(256) void rmsnorm_dw_reduce(const float* __restrict
 // ------------------------------------------------------------------------------------------------
 template <typename XT, typename WT, typename OT>
 static int fwd_typed(const void* x, const void* w, void* y, float* rstd, int64_t rows, int hidden, int64_t xs,
-                     int64_t ys, float eps, hipStream_t st) {
+                     int64_t ys, float eps, hipStream_t st, const void* res = nullptr, void* hsum = nullptr,
+                     int64_t rss = 0, int64_t hss = 0) {
   constexpr int E = 16 / sizeof(XT);
   const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
   const XT* xp = (const XT*)x; const WT* wp = (const WT*)w; OT* yp = (OT*)y;
+  const XT* rp = (const XT*)res; XT* hp = (XT*)hsum;
   const bool vec = hidden % E == 0 && aligned16(x) && aligned16(w) && aligned16(y) && (xs * sizeof(XT)) % 16 == 0 &&
+                   aligned16(res) && aligned16(hsum) && (rss * sizeof(XT)) % 16 == 0 && (hss * sizeof(XT)) % 16 == 0 &&
                    (ys * sizeof(OT)) % 16 == 0 && hidden / E <= 256 * 8;
   if (vec) {
     const int nvec = hidden / E;
 #define TP_RMS_FWD(NV, WAVES)                                                                                  \
   rmsnorm_fwd_vec<XT, WT, OT, NV, WAVES><<<dim3((unsigned)((rows + 4 / WAVES - 1) / (4 / WAVES))), block, 0, st>>>( \
-      xp, wp, yp, rstd, rows, hidden, xs, ys, eps)
+      xp, wp, yp, rstd, rows, hidden, xs, ys, eps, rp, hp, rss, hss)
     // two vectors per thread over a whole block measured fastest at hidden 4096 (against one vector over
     // 512 threads, or a wave per row)
     if (nvec <= 64) TP_RMS_FWD(1, 1);
@@ -270,26 +306,28 @@ static int fwd_typed(const void* x, const void* w, void* y, float* rstd, int64_t
     else TP_RMS_FWD(8, 4);
 #undef TP_RMS_FWD
   } else {
-    rmsnorm_fwd_generic<XT, WT, OT><<<grid, block, 0, st>>>(xp, wp, yp, rstd, rows, hidden, xs, ys, eps);
+    rmsnorm_fwd_generic<XT, WT, OT><<<grid, block, 0, st>>>(xp, wp, yp, rstd, rows, hidden, xs, ys, eps, rp, hp, rss, hss);
   }
   return check_launch("tp_rmsnorm_fwd");
 }
 
 template <typename XT, typename WT, typename OT>
 static int bwd_typed(const void* dy, const void* x, const void* w, const float* rstd, void* dx, void* dw, float* ws,
-                     int64_t rows, int hidden, int64_t dys, int64_t xs, int64_t dxs, hipStream_t st) {
+                     int64_t rows, int hidden, int64_t dys, int64_t xs, int64_t dxs, hipStream_t st,
+                     const void* dres = nullptr, int64_t drs = 0) {
   constexpr int E = 16 / sizeof(XT);
   const OT* gp = (const OT*)dy; const XT* xp = (const XT*)x; const WT* wp = (const WT*)w; XT* dxp = (XT*)dx;
+  const XT* drp = (const XT*)dres;
   const int parts = rms_parts(rows);
   const int nvec = hidden / E;
   const bool vec = hidden % E == 0 && aligned16(dy) && aligned16(x) && aligned16(w) && aligned16(dx) &&
                    (dys * sizeof(OT)) % 16 == 0 && (xs * sizeof(XT)) % 16 == 0 && (dxs * sizeof(XT)) % 16 == 0 &&
-                   nvec <= 256 * 8;
+                   aligned16(dres) && (drs * sizeof(XT)) % 16 == 0 && nvec <= 256 * 8;
   if (vec) {
     const dim3 block(256);
 #define TP_RMS_BWD(NV, WAVES)                                                                             \
   rmsnorm_bwd_vec<XT, WT, OT, NV, WAVES><<<dim3(parts / (4 / WAVES)), block, 0, st>>>(gp, xp, wp, rstd, dxp, ws, rows, \
-                                                                                     hidden, dys, xs, dxs)
+                                                                                     hidden, dys, xs, dxs, drp, drs)
     if (nvec <= 64) TP_RMS_BWD(1, 1);
     else if (nvec <= 128) TP_RMS_BWD(2, 1);
     else if (nvec <= 256) TP_RMS_BWD(1, 4);
@@ -299,7 +337,7 @@ static int bwd_typed(const void* dy, const void* x, const void* w, const float* 
 #undef TP_RMS_BWD
   } else {
     rmsnorm_bwd_dx_generic<XT, WT, OT><<<dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st>>>(gp, xp, wp, rstd, dxp, rows,
-                                                                                              hidden, dys, xs, dxs);
+                                                                                              hidden, dys, xs, dxs, drp, drs);
     rmsnorm_bwd_dw_generic<XT, OT><<<dim3((hidden + 255) / 256, parts), dim3(256), 0, st>>>(gp, xp, rstd, ws, rows, hidden,
                                                                                           dys, xs);
   }
@@ -351,6 +389,52 @@ extern "C" int tp_rmsnorm_bwd(const void* dy, const void* x, const void* w, cons
   if (x_dtype == TP_F32 && w_dtype == TP_F32) TP_GO(float, float, float);
 #undef TP_GO
   TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_rmsnorm_bwd: unsupported dtypes x=%d w=%d", x_dtype, w_dtype);
+}
+
+// ------------------------------------------------------------------------------------------------
+// RMSNorm fused with the residual add that precedes it in a decoder layer
+// ------------------------------------------------------------------------------------------------
+extern "C" int tp_add_rmsnorm_fwd(const void* x, const void* residual, const void* w, void* h, void* y, float* rstd,
+                                  int64_t rows, int hidden, int64_t x_row_stride, int64_t res_row_stride,
+                                  int64_t h_row_stride, int64_t y_row_stride, float eps, int x_dtype, int w_dtype,
+                                  void* stream) {
+  TP_REQUIRE(x && residual && w && h && y && rstd, TP_ERR_BAD_ARG, "tp_add_rmsnorm_fwd: null pointer");
+  TP_REQUIRE(rows >= 0 && hidden > 0, TP_ERR_BAD_ARG, "tp_add_rmsnorm_fwd: bad shape rows=%lld hidden=%d", (long long)rows, hidden);
+  TP_REQUIRE(x_row_stride >= hidden && res_row_stride >= hidden && h_row_stride >= hidden && y_row_stride >= hidden,
+             TP_ERR_BAD_ARG, "tp_add_rmsnorm_fwd: row stride smaller than hidden");
+  if (rows == 0) return TP_OK;
+  hipStream_t st = (hipStream_t)stream;
+#define TP_GO(XT, WT, OT)                                                                                          \
+  return fwd_typed<XT, WT, OT>(x, w, y, rstd, rows, hidden, x_row_stride, y_row_stride, eps, st, residual, h, \
+                               res_row_stride, h_row_stride)
+  if (x_dtype == TP_BF16 && w_dtype == TP_BF16) TP_GO(bf16_t, bf16_t, bf16_t);
+  if (x_dtype == TP_BF16 && w_dtype == TP_F32) TP_GO(bf16_t, float, float);
+  if (x_dtype == TP_F16 && w_dtype == TP_F16) TP_GO(f16_t, f16_t, f16_t);
+  if (x_dtype == TP_F16 && w_dtype == TP_F32) TP_GO(f16_t, float, float);
+  if (x_dtype == TP_F32 && w_dtype == TP_F32) TP_GO(float, float, float);
+#undef TP_GO
+  TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_add_rmsnorm_fwd: unsupported dtypes x=%d w=%d", x_dtype, w_dtype);
+}
+
+extern "C" int tp_add_rmsnorm_bwd(const void* dy, const void* dh, const void* h, const void* w, const float* rstd,
+                                  void* dx, void* dw, float* ws, int64_t rows, int hidden, int64_t dy_row_stride,
+                                  int64_t dh_row_stride, int64_t h_row_stride, int64_t dx_row_stride, int x_dtype,
+                                  int w_dtype, void* stream) {
+  TP_REQUIRE(dy && dh && h && w && rstd && dx && dw && ws, TP_ERR_BAD_ARG, "tp_add_rmsnorm_bwd: null pointer");
+  TP_REQUIRE(rows > 0 && hidden > 0, TP_ERR_BAD_ARG, "tp_add_rmsnorm_bwd: bad shape rows=%lld hidden=%d", (long long)rows, hidden);
+  TP_REQUIRE(dy_row_stride >= hidden && dh_row_stride >= hidden && h_row_stride >= hidden && dx_row_stride >= hidden,
+             TP_ERR_BAD_ARG, "tp_add_rmsnorm_bwd: row stride smaller than hidden");
+  hipStream_t st = (hipStream_t)stream;
+#define TP_GO(XT, WT, OT)                                                                                        \
+  return bwd_typed<XT, WT, OT>(dy, h, w, rstd, dx, dw, ws, rows, hidden, dy_row_stride, h_row_stride, dx_row_stride, st, \
+                               dh, dh_row_stride)
+  if (x_dtype == TP_BF16 && w_dtype == TP_BF16) TP_GO(bf16_t, bf16_t, bf16_t);
+  if (x_dtype == TP_BF16 && w_dtype == TP_F32) TP_GO(bf16_t, float, float);
+  if (x_dtype == TP_F16 && w_dtype == TP_F16) TP_GO(f16_t, f16_t, f16_t);
+  if (x_dtype == TP_F16 && w_dtype == TP_F32) TP_GO(f16_t, float, float);
+  if (x_dtype == TP_F32 && w_dtype == TP_F32) TP_GO(float, float, float);
+#undef TP_GO
+  TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_add_rmsnorm_bwd: unsupported dtypes x=%d w=%d", x_dtype, w_dtype);
 }
 
 // ------------------------------------------------------------------------------------------------

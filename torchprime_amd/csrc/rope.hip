@@ -75,8 +75,14 @@ struct RopeArgs {
 // in (B,S,H,D) memory.  Which tensor, the batch offset and all strides are wave-uniform, so they stay
 // on the scalar unit; WIDE = false keeps the per-lane offsets in 32 bits (every offset inside a batch
 // element below 2^31 elements, checked on the host).
-template <typename T, bool INTERLEAVED, bool BACKWARD, bool WIDE>
+// MODE 0: rotate-half on [first half | second half] (Llama, Mixtral).  MODE 1: the input is first permuted
+// [x0,x1,x2,...] -> [evens | odds] and the output stays in that order (DeepSeek).  MODE 2: adjacent pairs
+// (x[2i], x[2i+1]) are rotated by angle i and written back in place, using the first half of the cos/sin row for both
+// members of a pair (Llama-4 apply_rotary_emb, model/llama4/model.py:364-409).
+template <typename T, int MODE, bool BACKWARD, bool WIDE>
 __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
+  constexpr bool LOAD_PAIRS = MODE == 1 && !BACKWARD;   // de-interleave while loading
+  constexpr bool STORE_PAIRS = MODE == 1 && BACKWARD;   // re-interleave while storing
   constexpr int E = 16 / sizeof(T);
   typedef typename std::conditional<WIDE, int64_t, unsigned>::type off_t;
   const int half = a.D / 2;
@@ -108,6 +114,33 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
     sp = (const T*)a.sin + a.cs_b * b + crow;
   }
 
+  if constexpr (MODE == 2) {
+    // A 16-byte chunk holds E/2 whole pairs, so the thread's two chunks (same addresses as in the other modes)
+    // are rotated independently: chunk at j*E covers pairs j*E/2.., chunk at half + j*E pairs D/4 + j*E/2..,
+    // and pair p takes entry p of the cos / sin row.
+    constexpr int P = E / 2;
+#pragma unroll
+    for (int ch = 0; ch < 2; ch++) {
+      const int eoff = ch * half + j * E, poff = ch * (half / 2) + j * P;
+      float v[E], c[P], sn[P], o[E];
+      load_f_nt<T, E>(xp + eoff, v);
+      load_f<T, P>(cp + poff, c);
+      load_f<T, P>(sp + poff, sn);
+#pragma unroll
+      for (int e = 0; e < P; e++) {
+        const float x = v[2 * e], y = v[2 * e + 1];
+        if (!BACKWARD) {
+          o[2 * e] = round_to<T>(round_to<T>(x * c[e]) + round_to<T>(-y * sn[e]));
+          o[2 * e + 1] = round_to<T>(round_to<T>(y * c[e]) + round_to<T>(x * sn[e]));
+        } else {
+          o[2 * e] = round_to<T>(x * c[e]) + round_to<T>(y * sn[e]);
+          o[2 * e + 1] = round_to<T>(y * c[e]) + round_to<T>(-x * sn[e]);
+        }
+      }
+      store_f_nt<T, E>(yp + eoff, o);
+    }
+    return;
+  }
   float c1[E], c2[E], s1[E], s2[E];
   load_f<T, E>(cp + j * E, c1);
   load_f<T, E>(cp + half + j * E, c2);
@@ -115,7 +148,7 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
   load_f<T, E>(sp + half + j * E, s2);
 
   float x1[E], x2[E], o1[E], o2[E];
-  if (!INTERLEAVED || BACKWARD) {
+  if (!LOAD_PAIRS) {
     load_f_nt<T, E>(xp + j * E, x1);
     load_f_nt<T, E>(xp + half + j * E, x2);
   } else {
@@ -144,7 +177,7 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
       o2[e] = round_to<T>(x2[e] * c2[e]) + round_to<T>(-x1[e] * s1[e]);
     }
   }
-  if (!INTERLEAVED || !BACKWARD) {
+  if (!STORE_PAIRS) {
     store_f_nt<T, E>(yp + j * E, o1);
     store_f_nt<T, E>(yp + half + j * E, o2);
   } else {
@@ -165,10 +198,12 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
 template <typename T, bool WIDE>
 static void rope_launch(const RopeArgs& a, int interleaved, int backward, dim3 grid, hipStream_t st) {
   const dim3 block(256);
-  if (!interleaved && !backward) rope_apply_kernel<T, false, false, WIDE><<<grid, block, 0, st>>>(a);
-  else if (!interleaved && backward) rope_apply_kernel<T, false, true, WIDE><<<grid, block, 0, st>>>(a);
-  else if (interleaved && !backward) rope_apply_kernel<T, true, false, WIDE><<<grid, block, 0, st>>>(a);
-  else rope_apply_kernel<T, true, true, WIDE><<<grid, block, 0, st>>>(a);
+  if (interleaved == 0 && !backward) rope_apply_kernel<T, 0, false, WIDE><<<grid, block, 0, st>>>(a);
+  else if (interleaved == 0 && backward) rope_apply_kernel<T, 0, true, WIDE><<<grid, block, 0, st>>>(a);
+  else if (interleaved == 1 && !backward) rope_apply_kernel<T, 1, false, WIDE><<<grid, block, 0, st>>>(a);
+  else if (interleaved == 1 && backward) rope_apply_kernel<T, 1, true, WIDE><<<grid, block, 0, st>>>(a);
+  else if (!backward) rope_apply_kernel<T, 2, false, WIDE><<<grid, block, 0, st>>>(a);
+  else rope_apply_kernel<T, 2, true, WIDE><<<grid, block, 0, st>>>(a);
 }
 
 template <typename T>
@@ -225,6 +260,7 @@ extern "C" int tp_rope_apply(const void* q, const void* k, const void* cos, cons
   TP_REQUIRE((k == nullptr) == (Hkv == 0), TP_ERR_BAD_ARG, "tp_rope_apply: k must be NULL exactly when Hkv == 0");
   TP_REQUIRE(Hkv == 0 || (k_out && k_strides && ko_strides), TP_ERR_BAD_ARG, "tp_rope_apply: null k output/strides");
   TP_REQUIRE(B >= 0 && Hq > 0 && Hkv >= 0 && S >= 0 && D > 0, TP_ERR_BAD_ARG, "tp_rope_apply: bad shape");
+  TP_REQUIRE(interleaved >= 0 && interleaved <= 2, TP_ERR_BAD_ARG, "tp_rope_apply: interleaved must be 0, 1 or 2");
   TP_REQUIRE(!pos || table_rows > 0, TP_ERR_BAD_ARG, "tp_rope_apply: a position gather needs the table's row count");
   const int esz = dtype == TP_F32 ? 4 : 2;
   TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F16 || dtype == TP_F32, TP_ERR_UNSUPPORTED, "tp_rope_apply: unsupported dtype %d", dtype);

@@ -27,6 +27,12 @@ class _RMSNorm(nn.Module):
     return f"{tuple(self.weight.shape)}, eps={self.variance_epsilon}"
 
 
+def add_rms_norm(hidden_states: torch.Tensor, residual: torch.Tensor, norm: "_RMSNorm"):
+  """The residual add and the norm after it of a decoder layer (model/llama/model.py:288-291) in one pass:
+  returns ``(norm(residual + hidden_states), residual + hidden_states)``; the second value is the next residual."""
+  return ops.add_rmsnorm(hidden_states, residual, norm.weight, norm.variance_epsilon)
+
+
 class LlamaRMSNorm(_RMSNorm):
   """LlamaRMSNorm is equivalent to T5LayerNorm (model/llama/model.py:38-52)."""
 

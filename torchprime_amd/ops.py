@@ -22,6 +22,11 @@ __all__ = [
   "rope_table",
   "rope_apply",
   "attention",
+  "add_rmsnorm",
+  "l2norm",
+  "scale_rows",
+  "swiglu",
+  "cross_entropy_fwd",
 ]
 
 
@@ -175,7 +180,7 @@ def _check_positions(pos: Tensor, rows: int) -> None:
   _POS_OK[key] = True
 
 
-def _rope_launch(q, k, cos, sin, pos, interleaved: bool, backward: bool):
+def _rope_launch(q, k, cos, sin, pos, interleaved: int, backward: bool):
   dev = _lib.require_gpu(q, k, cos, sin, pos)
   if q.dim() != 4 or (k is not None and k.dim() != 4):
     raise ValueError("rotary apply expects (batch, heads, seq, dim) tensors")
@@ -227,8 +232,9 @@ def _rope_launch(q, k, cos, sin, pos, interleaved: bool, backward: bool):
 
 @torch.library.custom_op("tprime::rope_apply", mutates_args=(), device_types="cuda")
 def rope_apply_op(
-  q: Tensor, k: Tensor, cos: Tensor, sin: Tensor, pos: Tensor | None, interleaved: bool, backward: bool
+  q: Tensor, k: Tensor, cos: Tensor, sin: Tensor, pos: Tensor | None, interleaved: int, backward: bool
 ) -> tuple[Tensor, Tensor]:
+  """``interleaved``: 0 rotate-half, 1 DeepSeek ([evens | odds] output), 2 adjacent pairs in place (Llama-4)."""
   return _rope_launch(q, k, cos, sin, pos, interleaved, backward)
 
 
@@ -258,10 +264,10 @@ def _rope_backward(ctx, dq, dk):
 rope_apply_op.register_autograd(_rope_backward, setup_context=_rope_setup)
 
 
-def rope_apply(q: Tensor, k: Tensor, cos: Tensor, sin: Tensor, pos: Tensor | None = None, interleaved: bool = False):
+def rope_apply(q: Tensor, k: Tensor, cos: Tensor, sin: Tensor, pos: Tensor | None = None, interleaved: int = 0):
   """``(q*cos + rotate_half(q)*sin, k*cos + rotate_half(k)*sin)`` for (B,H,S,D) q and k in one launch."""
   _lib.require_gpu(q, k, cos, sin, pos)
-  return rope_apply_op(q, k, cos, sin, pos, interleaved, False)
+  return rope_apply_op(q, k, cos, sin, pos, int(interleaved), False)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -384,3 +390,306 @@ def attention(
   if sm_scale is None:
     sm_scale = 1.0 / math.sqrt(v.shape[-1])
   return attn_fwd(q, k, v, segment_ids, sm_scale, causal)[0]
+
+
+# ------------------------------------------------------------------------------------------------
+# the steps either side of the attention path: residual add + RMSNorm, L2 norm, temperature scale,
+# SwiGLU, cross entropy
+# ------------------------------------------------------------------------------------------------
+@torch.library.custom_op("tprime::add_rmsnorm_fwd", mutates_args=(), device_types="cuda")
+def add_rmsnorm_fwd(x: Tensor, residual: Tensor, weight: Tensor, eps: float) -> tuple[Tensor, Tensor, Tensor]:
+  """(y, h, rstd): h = residual + x, y = RMSNorm(h) * weight, in one pass."""
+  _lib.require_gpu(x, residual, weight)
+  hidden = x.shape[-1]
+  if residual.shape != x.shape or residual.dtype != x.dtype:
+    raise ValueError(f"residual {tuple(residual.shape)}/{residual.dtype} must match x {tuple(x.shape)}/{x.dtype}")
+  if weight.shape != (hidden,):
+    raise ValueError(f"weight shape {tuple(weight.shape)} does not match hidden size {hidden}")
+  x2, r2, w = _rows(x), _rows(residual), weight.contiguous()
+  rows = x2.shape[0]
+  out_dtype = torch.result_type(weight, x)
+  y = torch.empty((rows, hidden), dtype=out_dtype, device=x.device)
+  h = torch.empty((rows, hidden), dtype=x.dtype, device=x.device)
+  rstd = torch.empty((rows,), dtype=torch.float32, device=x.device)
+  if rows:
+    _lib.call(
+      "tp_add_rmsnorm_fwd", x2.data_ptr(), r2.data_ptr(), w.data_ptr(), h.data_ptr(), y.data_ptr(), rstd.data_ptr(),
+      rows, hidden, x2.stride(0) if rows > 1 else hidden, r2.stride(0) if rows > 1 else hidden, hidden, hidden,
+      float(eps), _lib.dtype_code(x.dtype), _lib.dtype_code(w.dtype), _lib.stream_ptr(x.device),
+    )  # fmt: skip
+  return y.view(*x.shape[:-1], hidden), h.view(x.shape), rstd
+
+
+@add_rmsnorm_fwd.register_fake
+def _(x, residual, weight, eps):
+  rows = x.numel() // max(x.shape[-1], 1)
+  return (x.new_empty(x.shape, dtype=torch.result_type(weight, x)), torch.empty_like(x, memory_format=torch.contiguous_format),
+          x.new_empty((rows,), dtype=torch.float32))
+
+
+@torch.library.custom_op("tprime::add_rmsnorm_bwd", mutates_args=(), device_types="cuda")
+def add_rmsnorm_bwd(dy: Tensor, dh: Tensor, h: Tensor, weight: Tensor, rstd: Tensor) -> tuple[Tensor, Tensor]:
+  _lib.require_gpu(dy, dh, h, weight, rstd)
+  hidden = h.shape[-1]
+  h2, g2, d2, w = _rows(h), _rows(dy), _rows(dh), weight.contiguous()
+  rows = h2.shape[0]
+  dx = torch.empty((rows, hidden), dtype=h.dtype, device=h.device)
+  dw = torch.empty((hidden,), dtype=w.dtype, device=h.device)
+  if rows == 0:
+    return dx.view(h.shape), dw.zero_()
+  lib = _lib.load()
+  ws = torch.empty((lib.tp_rmsnorm_bwd_workspace_bytes(rows, hidden) // 4,), dtype=torch.float32, device=h.device)
+  st = lambda t: t.stride(0) if rows > 1 else hidden  # noqa: E731
+  _lib.call(
+    "tp_add_rmsnorm_bwd", g2.data_ptr(), d2.data_ptr(), h2.data_ptr(), w.data_ptr(), rstd.data_ptr(), dx.data_ptr(),
+    dw.data_ptr(), ws.data_ptr(), rows, hidden, st(g2), st(d2), st(h2), hidden, _lib.dtype_code(h.dtype),
+    _lib.dtype_code(w.dtype), _lib.stream_ptr(h.device),
+  )  # fmt: skip
+  return dx.view(h.shape), dw
+
+
+@add_rmsnorm_bwd.register_fake
+def _(dy, dh, h, weight, rstd):
+  return torch.empty_like(h, memory_format=torch.contiguous_format), torch.empty_like(weight)
+
+
+def _add_rmsnorm_setup(ctx, inputs, output):
+  _x, _res, weight, _eps = inputs
+  _y, h, rstd = output
+  ctx.save_for_backward(h, weight, rstd)
+
+
+def _add_rmsnorm_backward(ctx, dy, dh, _drstd):
+  h, weight, rstd = ctx.saved_tensors
+  out_dtype = torch.result_type(weight, h)
+  if dy is None:
+    dy = torch.zeros_like(h, dtype=out_dtype)
+  if dh is None:
+    dx, dw = rmsnorm_bwd(dy.to(out_dtype), h, weight, rstd)
+  else:
+    dx, dw = add_rmsnorm_bwd(dy.to(out_dtype), dh.to(h.dtype), h, weight, rstd)
+  return dx, dx, dw, None
+
+
+add_rmsnorm_fwd.register_autograd(_add_rmsnorm_backward, setup_context=_add_rmsnorm_setup)
+
+
+def add_rmsnorm(x: Tensor, residual: Tensor, weight: Tensor, eps: float) -> tuple[Tensor, Tensor]:
+  """``h = residual + x; y = rms_norm(h, weight, eps)`` in one pass; returns ``(y, h)``."""
+  y, h, _ = add_rmsnorm_fwd(x, residual, weight, eps)
+  return y, h
+
+
+def _head_rows(x: Tensor) -> Tensor:
+  d = x.shape[-1]
+  x2 = x.reshape(-1, d)
+  if x2.stride(-1) != 1 or (x2.stride(0) * x2.element_size()) % 16 or x2.data_ptr() % 16:
+    x2 = x2.contiguous()
+  return x2
+
+
+@torch.library.custom_op("tprime::l2norm_fwd", mutates_args=(), device_types="cuda")
+def l2norm_fwd(x: Tensor, eps: float) -> tuple[Tensor, Tensor]:
+  _lib.require_gpu(x)
+  x2 = _head_rows(x)
+  rows, dim = x2.shape
+  y = torch.empty((rows, dim), dtype=x.dtype, device=x.device)
+  rstd = torch.empty((rows,), dtype=torch.float32, device=x.device)
+  if rows:
+    _lib.call("tp_l2norm_fwd", x2.data_ptr(), y.data_ptr(), rstd.data_ptr(), rows, dim, x2.stride(0) if rows > 1 else dim, dim,
+              float(eps), _lib.dtype_code(x.dtype), _lib.stream_ptr(x.device))  # fmt: skip
+  return y.view(x.shape), rstd
+
+
+@l2norm_fwd.register_fake
+def _(x, eps):
+  return torch.empty_like(x, memory_format=torch.contiguous_format), x.new_empty((x.numel() // max(x.shape[-1], 1),), dtype=torch.float32)
+
+
+@torch.library.custom_op("tprime::l2norm_bwd", mutates_args=(), device_types="cuda")
+def l2norm_bwd(dy: Tensor, x: Tensor, rstd: Tensor) -> Tensor:
+  _lib.require_gpu(dy, x, rstd)
+  x2, g2 = _head_rows(x), _head_rows(dy)
+  rows, dim = x2.shape
+  dx = torch.empty((rows, dim), dtype=x.dtype, device=x.device)
+  if rows:
+    st = lambda t: t.stride(0) if rows > 1 else dim  # noqa: E731
+    _lib.call("tp_l2norm_bwd", g2.data_ptr(), x2.data_ptr(), rstd.data_ptr(), dx.data_ptr(), rows, dim, st(g2), st(x2), dim,
+              _lib.dtype_code(x.dtype), _lib.stream_ptr(x.device))  # fmt: skip
+  return dx.view(x.shape)
+
+
+@l2norm_bwd.register_fake
+def _(dy, x, rstd):
+  return torch.empty_like(x, memory_format=torch.contiguous_format)
+
+
+def _l2norm_setup(ctx, inputs, output):
+  ctx.save_for_backward(inputs[0], output[1])
+
+
+def _l2norm_backward(ctx, dy, _drstd):
+  x, rstd = ctx.saved_tensors
+  return l2norm_bwd(dy.to(x.dtype), x, rstd), None
+
+
+l2norm_fwd.register_autograd(_l2norm_backward, setup_context=_l2norm_setup)
+
+
+def l2norm(x: Tensor, eps: float) -> Tensor:
+  """``(x.float() * rsqrt(mean(x.float()**2, -1) + eps)).type_as(x)`` over the last dim."""
+  return l2norm_fwd(x, eps)[0]
+
+
+@torch.library.custom_op("tprime::scale_rows", mutates_args=(), device_types="cuda")
+def scale_rows(x: Tensor, scale: Tensor) -> Tensor:
+  """x (B, S, N, D) times scale (S) fp32 per position, rounded to x's dtype."""
+  _lib.require_gpu(x, scale)
+  if x.dim() != 4 or scale.shape != (x.shape[1],):
+    raise ValueError(f"expected x (batch, seq, heads, dim) and scale (seq,), got {tuple(x.shape)} and {tuple(scale.shape)}")
+  B, S, N, D = x.shape
+  x2 = _head_rows(x)
+  y = torch.empty((B * S * N, D), dtype=x.dtype, device=x.device)
+  if y.numel():
+    _lib.call("tp_scale_rows", x2.data_ptr(), scale.to(torch.float32).contiguous().data_ptr(), y.data_ptr(), B * S * N, D,
+              x2.stride(0) if B * S * N > 1 else D, D, N, S, _lib.dtype_code(x.dtype), _lib.stream_ptr(x.device))  # fmt: skip
+  return y.view(x.shape)
+
+
+@scale_rows.register_fake
+def _(x, scale):
+  return torch.empty_like(x, memory_format=torch.contiguous_format)
+
+
+def _scale_rows_setup(ctx, inputs, output):
+  ctx.save_for_backward(inputs[1])
+
+
+def _scale_rows_backward(ctx, dy):
+  (scale,) = ctx.saved_tensors
+  return scale_rows(dy, scale), None
+
+
+scale_rows.register_autograd(_scale_rows_backward, setup_context=_scale_rows_setup)
+
+
+@torch.library.custom_op("tprime::swiglu_fwd", mutates_args=(), device_types="cuda")
+def swiglu_fwd(gate: Tensor, up: Tensor) -> Tensor:
+  _lib.require_gpu(gate, up)
+  if gate.shape != up.shape or gate.dtype != up.dtype:
+    raise ValueError(f"gate {tuple(gate.shape)}/{gate.dtype} and up {tuple(up.shape)}/{up.dtype} must match")
+  g2, u2 = _head_rows(gate), _head_rows(up)
+  rows, cols = g2.shape
+  out = torch.empty((rows, cols), dtype=gate.dtype, device=gate.device)
+  if out.numel():
+    st = lambda t: t.stride(0) if rows > 1 else cols  # noqa: E731
+    _lib.call("tp_swiglu_fwd", g2.data_ptr(), u2.data_ptr(), out.data_ptr(), rows, cols, st(g2), st(u2), cols,
+              _lib.dtype_code(gate.dtype), _lib.stream_ptr(gate.device))  # fmt: skip
+  return out.view(gate.shape)
+
+
+@swiglu_fwd.register_fake
+def _(gate, up):
+  return torch.empty_like(gate, memory_format=torch.contiguous_format)
+
+
+@torch.library.custom_op("tprime::swiglu_bwd", mutates_args=(), device_types="cuda")
+def swiglu_bwd(dout: Tensor, gate: Tensor, up: Tensor) -> tuple[Tensor, Tensor]:
+  _lib.require_gpu(dout, gate, up)
+  d2, g2, u2 = _head_rows(dout), _head_rows(gate), _head_rows(up)
+  rows, cols = g2.shape
+  dg = torch.empty((rows, cols), dtype=gate.dtype, device=gate.device)
+  du = torch.empty_like(dg)
+  if dg.numel():
+    st = lambda t: t.stride(0) if rows > 1 else cols  # noqa: E731
+    _lib.call("tp_swiglu_bwd", d2.data_ptr(), g2.data_ptr(), u2.data_ptr(), dg.data_ptr(), du.data_ptr(), rows, cols, st(d2),
+              st(g2), st(u2), cols, cols, _lib.dtype_code(gate.dtype), _lib.stream_ptr(gate.device))  # fmt: skip
+  return dg.view(gate.shape), du.view(gate.shape)
+
+
+@swiglu_bwd.register_fake
+def _(dout, gate, up):
+  return torch.empty_like(gate, memory_format=torch.contiguous_format), torch.empty_like(up, memory_format=torch.contiguous_format)
+
+
+def _swiglu_setup(ctx, inputs, output):
+  ctx.save_for_backward(*inputs)
+
+
+def _swiglu_backward(ctx, dout):
+  gate, up = ctx.saved_tensors
+  return swiglu_bwd(dout.to(gate.dtype), gate, up)
+
+
+swiglu_fwd.register_autograd(_swiglu_backward, setup_context=_swiglu_setup)
+
+
+def swiglu(gate: Tensor, up: Tensor) -> Tensor:
+  """``silu(gate) * up`` with the eager roundings, one pass."""
+  return swiglu_fwd(gate, up)
+
+
+@torch.library.custom_op("tprime::cross_entropy_fwd", mutates_args=(), device_types="cuda")
+def cross_entropy_fwd(logits: Tensor, labels: Tensor, ignore_index: int) -> tuple[Tensor, Tensor, Tensor]:
+  """(loss (scalar fp32), lse (B*S), loss_and_count (2)) of the shifted next-token cross entropy."""
+  _lib.require_gpu(logits, labels)
+  if logits.dim() != 3 or labels.shape != logits.shape[:2]:
+    raise ValueError(f"expected logits (batch, seq, vocab) and labels (batch, seq), got {tuple(logits.shape)} and {tuple(labels.shape)}")
+  if logits.dtype not in (torch.float32, torch.bfloat16):
+    raise TypeError(f"cross entropy takes float32 or bfloat16 logits, got {logits.dtype}")
+  B, S, V = logits.shape
+  if logits.stride(2) != 1:
+    logits = logits.contiguous()
+  labels = labels.to(torch.int64)
+  if labels.stride(1) != 1:
+    labels = labels.contiguous()
+  lse = torch.empty((B * S,), dtype=torch.float32, device=logits.device)
+  row_loss = torch.empty_like(lse)
+  lc = torch.empty((2,), dtype=torch.float32, device=logits.device)
+  _lib.call("tp_cross_entropy_fwd", logits.data_ptr(), labels.data_ptr(), lse.data_ptr(), row_loss.data_ptr(), lc.data_ptr(),
+            B, S, V, logits.stride(0), logits.stride(1), labels.stride(0), int(ignore_index), _lib.dtype_code(logits.dtype),
+            _lib.stream_ptr(logits.device))  # fmt: skip
+  return lc[0].clone(), lse, lc
+
+
+@cross_entropy_fwd.register_fake
+def _(logits, labels, ignore_index):
+  B, S, _ = logits.shape
+  return logits.new_empty((), dtype=torch.float32), logits.new_empty((B * S,), dtype=torch.float32), logits.new_empty((2,), dtype=torch.float32)
+
+
+@torch.library.custom_op("tprime::cross_entropy_bwd", mutates_args=(), device_types="cuda")
+def cross_entropy_bwd(dloss: Tensor, logits: Tensor, labels: Tensor, lse: Tensor, loss_and_count: Tensor, ignore_index: int) -> Tensor:
+  _lib.require_gpu(dloss, logits, labels, lse, loss_and_count)
+  B, S, V = logits.shape
+  if logits.stride(2) != 1:
+    logits = logits.contiguous()
+  labels = labels.to(torch.int64)
+  if labels.stride(1) != 1:
+    labels = labels.contiguous()
+  dlogits = torch.empty((B, S, V), dtype=logits.dtype, device=logits.device)
+  _lib.call("tp_cross_entropy_bwd", logits.data_ptr(), labels.data_ptr(), lse.data_ptr(), loss_and_count.data_ptr(),
+            dloss.to(torch.float32).reshape(1).contiguous().data_ptr(), dlogits.data_ptr(), B, S, V, logits.stride(0),
+            logits.stride(1), labels.stride(0), dlogits.stride(0), dlogits.stride(1), int(ignore_index),
+            _lib.dtype_code(logits.dtype), _lib.stream_ptr(logits.device))  # fmt: skip
+  return dlogits
+
+
+@cross_entropy_bwd.register_fake
+def _(dloss, logits, labels, lse, loss_and_count, ignore_index):
+  return torch.empty_like(logits, memory_format=torch.contiguous_format)
+
+
+def _xent_setup(ctx, inputs, output):
+  logits, labels, ignore_index = inputs
+  _loss, lse, lc = output
+  ctx.save_for_backward(logits, labels, lse, lc)
+  ctx.ignore_index = ignore_index
+
+
+def _xent_backward(ctx, dloss, _dlse, _dlc):
+  logits, labels, lse, lc = ctx.saved_tensors
+  return cross_entropy_bwd(dloss, logits, labels, lse, lc, ctx.ignore_index), None, None
+
+
+cross_entropy_fwd.register_autograd(_xent_backward, setup_context=_xent_setup)
