@@ -63,8 +63,9 @@ def test_hip_attention_matches_golden():
 
 @pytest.mark.gpu
 def test_hip_llama_block_matches_golden_c1():
-  """benchmark configuration 1 on the GPU: RMSNorm (fp32 kernel) -> projections -> RoPE -> attention -> o_proj.
-  The attention kernels are 16-bit, so q/k/v are cast to bf16 around the attention call only."""
+  """benchmark configuration 1 on the GPU in fp32 end to end: RMSNorm -> projections -> RoPE -> fp32 attention ->
+  o_proj, at the fp32 tolerance class of the reference's own test of this shape
+  (torchprime/torch_xla_models/tests/test_llama.py:143-188)."""
   import torchprime_amd as tpa
 
   dev = "cuda"
@@ -81,7 +82,17 @@ def test_hip_llama_block_matches_golden_c1():
   q, k = tpa.apply_rotary_pos_emb(q, k, cos, sin)
   cfg = tpa.Config(attention_kernel=None, num_attention_heads=H, num_key_value_heads=H, attention_dropout=False)
   mask = orc.causal_additive_mask(S).to(dev)
-  o = tpa.AttentionModule(cfg)(q.bfloat16(), k.bfloat16(), v.bfloat16(), mask).float()
-  y = o.transpose(1, 2).contiguous().reshape(B, S, hid) @ w["wo"].T
+  old = torch.backends.cuda.matmul.allow_tf32
+  torch.backends.cuda.matmul.allow_tf32 = False
+  try:
+    o = tpa.AttentionModule(cfg)(q, k, v, mask)
+    assert o.dtype == torch.float32
+    y = o.transpose(1, 2).contiguous().reshape(B, S, hid) @ w["wo"].T
+  finally:
+    torch.backends.cuda.matmul.allow_tf32 = old
   ref = _load("c1_llama_block.npz")["out_rows"]
-  assert_close(y[:, ::8], ref, "C1 block", max_abs=2e-2, rel_l2=1e-2)
+  assert_close(y[:, ::8], ref, "C1 block", max_abs=2e-5, rel_l2=2e-5)
+  # and with 16-bit attention, as the production configurations run it
+  o16 = tpa.AttentionModule(cfg)(q.bfloat16(), k.bfloat16(), v.bfloat16(), mask).float()
+  y16 = o16.transpose(1, 2).contiguous().reshape(B, S, hid) @ w["wo"].T
+  assert_close(y16[:, ::8], ref, "C1 block, bf16 attention", max_abs=2e-2, rel_l2=1e-2)

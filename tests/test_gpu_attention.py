@@ -239,13 +239,39 @@ def test_splash_wrapper_signature_and_segments():
     tpa.tpu_splash_attention_jax_call_wrapper(None, qs.to(DEV), k.to(DEV), v.to(DEV), slide, None, True)
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,S,Skv,D,causal,use_seg", [
+  (2, 8, 8, 128, 128, 64, True, False),    # benchmark configuration 1's attention
+  (1, 4, 2, 200, 200, 128, True, False),   # GQA, ragged
+  (2, 4, 1, 77, 300, 64, False, False),    # full attention, Skv != Sq
+  (2, 4, 2, 260, 260, 128, True, True),    # segment ids
+  (1, 2, 2, 1, 1, 64, True, False),
+])
+def test_fp32_attention_forward(B, Hq, Hkv, S, Skv, D, causal, use_seg):
+  """fp32 operands (v_mfma_f32_32x32x2_f32): the fp32 tolerance class of the reference's CPU tests, atol 1e-5."""
+  q, k, v = heads_view(B, Hq, S, D, 1, torch.float32), heads_view(B, Hkv, Skv, D, 2, torch.float32), heads_view(B, Hkv, Skv, D, 3, torch.float32)
+  seg = packed_segment_ids(B, S, 5, 90, seed=8)[0] if use_seg else None
+  out, lse = torch.ops.tprime.attn_fwd(q.to(DEV), k.to(DEV), v.to(DEV), None if seg is None else seg.to(DEV), D**-0.5, causal)
+  o_ref, lse_ref = orc.attention_ref(q, k, v, seg, causal, D**-0.5, torch.float64)
+  assert out.dtype == torch.float32
+  assert_close(out, o_ref, "out", max_abs=1e-5, rel_l2=1e-5)
+  assert_close(lse, lse_ref, "lse", max_abs=1e-5, rel_l2=1e-6)
+  if use_seg is False and causal:
+    m = tpa.AttentionModule(_cfg(None, Hq, Hkv))
+    o2 = m(q.to(DEV), k.to(DEV), v.to(DEV), orc.causal_additive_mask(S).to(DEV)) if S == Skv else None
+    if o2 is not None:
+      assert_close(o2, orc.eager_attention(q, k, v, orc.causal_additive_mask(S)), "module, fp32 eager branch", max_abs=1e-5, rel_l2=1e-5)
+
+
 def test_unsupported_inputs_raise():
   q = torch.zeros((1, 2, 16, 96), dtype=torch.bfloat16, device=DEV)
   with pytest.raises(NotImplementedError):
     tpa.ops.attention(q, q, q)
-  q32 = torch.zeros((1, 2, 16, 64), dtype=torch.float32, device=DEV)
+  q64 = torch.zeros((1, 2, 16, 64), dtype=torch.float64, device=DEV)
   with pytest.raises(TypeError):
-    tpa.ops.attention(q32, q32, q32)
+    tpa.ops.attention(q64, q64, q64)
+  q32 = torch.zeros((1, 2, 16, 64), dtype=torch.float32, device=DEV, requires_grad=True)
+  with pytest.raises(NotImplementedError):  # fp32 attention is forward-only
+    tpa.ops.attention(q32, q32, q32).sum().backward()
   with pytest.raises(RuntimeError):
     tpa.ops.attention(q.cpu(), q.cpu(), q.cpu())
 

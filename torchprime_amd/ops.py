@@ -274,6 +274,7 @@ def rope_apply(q: Tensor, k: Tensor, cos: Tensor, sin: Tensor, pos: Tensor | Non
 # attention
 # ------------------------------------------------------------------------------------------------
 _SUPPORTED_HEAD_DIMS = ((64, 64), (128, 128), (192, 128))
+_SUPPORTED_HEAD_DIMS_F32 = ((64, 64), (128, 128))  # fp32 operands: forward only (the small fp32 configurations)
 
 
 def _check_attn(q, k, v, seg):
@@ -285,11 +286,12 @@ def _check_attn(q, k, v, seg):
     raise ValueError(f"q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)} are inconsistent")
   if Hkv == 0 or Hq % Hkv != 0:
     raise ValueError(f"num query heads {Hq} must be a multiple of num kv heads {Hkv}")
-  if q.dtype not in (torch.bfloat16, torch.float16) or k.dtype != q.dtype or v.dtype != q.dtype:
-    raise TypeError(f"attention kernels take bfloat16 or float16 q/k/v of one dtype, got {q.dtype}/{k.dtype}/{v.dtype}")
+  if q.dtype not in (torch.bfloat16, torch.float16, torch.float32) or k.dtype != q.dtype or v.dtype != q.dtype:
+    raise TypeError(f"attention kernels take bfloat16, float16 or float32 q/k/v of one dtype, got {q.dtype}/{k.dtype}/{v.dtype}")
   Dv = v.shape[-1]
-  if (Dqk, Dv) not in _SUPPORTED_HEAD_DIMS:
-    raise NotImplementedError(f"head dims (qk={Dqk}, v={Dv}) not built; supported: {_SUPPORTED_HEAD_DIMS}")
+  dims = _SUPPORTED_HEAD_DIMS_F32 if q.dtype == torch.float32 else _SUPPORTED_HEAD_DIMS
+  if (Dqk, Dv) not in dims:
+    raise NotImplementedError(f"head dims (qk={Dqk}, v={Dv}) not built for {q.dtype}; supported: {dims}")
   if seg is not None:
     # kernel_utils.py:238-241: segment ids must cover the whole (unsharded) sequence
     assert seg.shape == (B, Skv) and Sq == Skv, "Sharding along sequence dimension not allowed in tpu kernel attention"
@@ -297,7 +299,8 @@ def _check_attn(q, k, v, seg):
 
 
 def _prep_heads(t: Tensor) -> Tensor:
-  ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all((s * 2) % 16 == 0 for s in t.stride()[:3])
+  esz = t.element_size()
+  ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all((s * esz) % 16 == 0 for s in t.stride()[:3])
   return t if ok else t.contiguous()
 
 
@@ -330,6 +333,8 @@ def attn_bwd(
   dout: Tensor, q: Tensor, k: Tensor, v: Tensor, out: Tensor, lse: Tensor, seg: Tensor | None, sm_scale: float, causal: bool
 ) -> tuple[Tensor, Tensor, Tensor]:
   dev = _lib.require_gpu(dout, q, k, v, out, lse, seg)
+  if q.dtype == torch.float32:
+    raise NotImplementedError("fp32 attention is forward-only; run the backward in bfloat16 or float16")
   B, Hq, Hkv, Sq, Skv, Dqk, Dv = _check_attn(q, k, v, seg)
   q, k, v, out, dout = _prep_heads(q), _prep_heads(k), _prep_heads(v), _prep_heads(out), _prep_heads(dout)
   lse = lse.contiguous()
