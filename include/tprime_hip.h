@@ -173,6 +173,36 @@ int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, const void* v
                    void* const* events);
 
 /* ------------------------------------------------------------------------------------------------
+ * Mask extensions of the functional API (torchprime/utils/kernel_utils.py:259-294,
+ * torchprime/utils/parallelism_utils.py:87-152, call site torchprime/torch_xla_models/attention.py:75-119).
+ * tp_attn_fwd / tp_attn_bwd with, on top of `causal` and `seg`:
+ *   q_positions     NULL or (Sq) int32: query row i stands for position q_positions[i] of the key order
+ *                   (LoadBalancedCausalMask.q_sequence); NULL: position i
+ *   causal_offset   with causal != 0, key j is allowed iff j <= position + causal_offset (the mask's `offset`)
+ *   window_left / window_right   >= 0: key j is allowed only if position - window_left <= j <= position +
+ *                   window_right (LocalMask, kernel_utils.py:266-275); < 0: unbounded on that side
+ *   logits_soft_cap > 0: scores become cap * tanh(sm_scale * q.k / cap) before masking and softmax
+ *                   (attn_logits_soft_cap, kernel_utils.py:292); <= 0: none
+ * Tiles outside every row's band are skipped.  Rows left without any allowed key give out = 0, lse = -inf and
+ * zero gradients.  Head dims 64 and 128, bf16 / fp16.  With none of the extensions in use the calls are
+ * tp_attn_fwd / tp_attn_bwd.
+ * ---------------------------------------------------------------------------------------------- */
+int tp_attn_fwd_masked(const void* q, const void* k, const void* v, const int32_t* seg,
+                       const int32_t* q_positions, void* out, float* lse, int B, int Hq, int Hkv, int Sq,
+                       int Skv, int Dqk, int Dv, const int64_t q_strides[3], const int64_t k_strides[3],
+                       const int64_t v_strides[3], const int64_t o_strides[3], float sm_scale, int causal,
+                       int causal_offset, int window_left, int window_right, float logits_soft_cap,
+                       int dtype, void* stream);
+int tp_attn_bwd_masked(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                       const float* lse, const int32_t* seg, const int32_t* q_positions, void* dq,
+                       void* dk, void* dv, float* ws, int B, int Hq, int Hkv, int Sq, int Skv, int Dqk,
+                       int Dv, const int64_t do_strides[3], const int64_t q_strides[3],
+                       const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
+                       const int64_t dq_strides[3], const int64_t dk_strides[3],
+                       const int64_t dv_strides[3], float sm_scale, int causal, int causal_offset,
+                       int window_left, int window_right, float logits_soft_cap, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * The steps either side of the attention path (HBM-bound, one pass over each tensor).
  * ---------------------------------------------------------------------------------------------- */
 

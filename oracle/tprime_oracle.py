@@ -31,6 +31,10 @@ reference, which needs torch_xla / jax / omegaconf):
   attn temperature          closed form log(floor((p+1)/f)+1) a + 1 at hand-computed positions       pinned
   swiglu                    x * sigmoid(x) * u in fp64 loops                                          pinned
   cross_entropy_loss        explicit per-token -log softmax loops incl. ignored labels; F.cross_entropy   pinned
+  allowed_mask extensions   window = band matrix (torch.tril/triu); permuted causal = causal on the un-permuted
+                            order (reorder o attention o reorder^-1); soft cap = explicit loops         pinned
+                            (exact inclusivity of jax's LocalMask bounds: restated from its published source,
+                            jax is not installed and pinned to no version by the reference: PARITY UNPINNED)
   segment masking vs the reference's TPU splash kernel numerics                     PARITY UNPINNED:
                             no reference test exercises decoder_segment_ids and the Pallas kernel is
                             not in the tree; semantics are the closed form
@@ -193,12 +197,25 @@ def eager_attention(q, k, v, attention_mask=None):
   return torch.matmul(w, v)
 
 
-def allowed_mask(segment_ids, q_len: int, kv_len: int, causal: bool) -> torch.Tensor:
+def allowed_mask(segment_ids, q_len: int, kv_len: int, causal: bool, window=None, q_positions=None,
+                 causal_offset: int = 0) -> torch.Tensor:
   """Boolean (B or 1, q_len, kv_len): (j <= i if causal) AND same segment.  Closed form of
-  CausalMask/FullMask (kernel_utils.py:259-263) combined with SegmentIds(q=ids, kv=ids) (:215-220)."""
-  i = torch.arange(q_len)[:, None]
+  CausalMask/FullMask (kernel_utils.py:259-263) combined with SegmentIds(q=ids, kv=ids) (:215-220).
+
+  Extensions: ``window=(left, right)`` ANDs in jax's LocalMask as kernel_utils.py:271-275 builds it (offset 0;
+  its mask function is ``q - left <= kv`` and ``kv <= q + right``, either side optional);
+  ``q_positions`` replaces the row index i by the position the row stands for and ``causal_offset`` shifts the
+  causal bound, ``q_positions[i] + offset >= j``: LoadBalancedCausalMask (parallelism_utils.py:109-132)."""
+  i = torch.arange(q_len) if q_positions is None else torch.as_tensor(q_positions).to(torch.int64).cpu()
+  i = i[:, None]
   j = torch.arange(kv_len)[None, :]
-  m = (j <= i) if causal else torch.ones((q_len, kv_len), dtype=torch.bool)
+  m = (j <= i + causal_offset) if causal else torch.ones((q_len, kv_len), dtype=torch.bool)
+  if window is not None:
+    left, right = window
+    if left is not None:
+      m = m & (i - left <= j)
+    if right is not None:
+      m = m & (j <= i + right)
   m = m[None]
   if segment_ids is not None:
     seg = segment_ids.to("cpu")
@@ -206,17 +223,21 @@ def allowed_mask(segment_ids, q_len: int, kv_len: int, causal: bool) -> torch.Te
   return m
 
 
-def attention_ref(q, k, v, segment_ids=None, causal=True, sm_scale=None, dtype=torch.float32):
+def attention_ref(q, k, v, segment_ids=None, causal=True, sm_scale=None, dtype=torch.float32, window=None, soft_cap=None,
+                  q_positions=None, causal_offset=0):
   """softmax(sm_scale * q k^T | allowed) v in ``dtype`` with no intermediate rounding; returns
   (out, lse).  Rows with no allowed key give out = 0, lse = -inf (the eager formula gives NaN there;
-  tests assert that divergence explicitly)."""
+  tests assert that divergence explicitly).  ``soft_cap``: logits <- cap * tanh(logits / cap) before masking, the
+  published definition of the splash kernel's ``attn_logits_soft_cap`` (kernel_utils.py:292)."""
   q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
   n_rep = q.shape[1] // k.shape[1]
   k, v = repeat_kv(k, n_rep), repeat_kv(v, n_rep)
   if sm_scale is None:
     sm_scale = 1.0 / math.sqrt(v.shape[-1])
   s = torch.matmul(q, k.transpose(2, 3)) * sm_scale
-  m = allowed_mask(segment_ids, q.shape[2], k.shape[2], causal)[:, None]
+  if soft_cap is not None:
+    s = soft_cap * torch.tanh(s / soft_cap)
+  m = allowed_mask(segment_ids, q.shape[2], k.shape[2], causal, window, q_positions, causal_offset)[:, None]
   s = s.masked_fill(~m, NEG_INF)
   lse = torch.logsumexp(s, dim=-1)
   any_allowed = m.any(-1)
@@ -240,12 +261,12 @@ def attention_ref_chunked(q, k, v, segment_ids=None, causal=True, sm_scale=None,
   return torch.cat(outs, 1), torch.cat(lses, 1)
 
 
-def attention_grads_ref(q, k, v, dout, segment_ids=None, causal=True, sm_scale=None, dtype=torch.float32):
+def attention_grads_ref(q, k, v, dout, segment_ids=None, causal=True, sm_scale=None, dtype=torch.float32, **mask_kw):
   """(out, dq, dk, dv) by autograd through attention_ref."""
   q = q.detach().to(dtype).requires_grad_(True)
   k = k.detach().to(dtype).requires_grad_(True)
   v = v.detach().to(dtype).requires_grad_(True)
-  out, _ = attention_ref(q, k, v, segment_ids, causal, sm_scale, dtype)
+  out, _ = attention_ref(q, k, v, segment_ids, causal, sm_scale, dtype, **mask_kw)
   dq, dk, dv = torch.autograd.grad(out, (q, k, v), dout.to(dtype))
   return out.detach(), dq, dk, dv
 

@@ -1,0 +1,151 @@
+"""GPU parity of the mask extensions (sliding window, logits soft cap, load-balanced causal mask with query rows in
+the striped order) through the ops, the functional wrapper and AttentionModule, against the CPU oracle: forward,
+gradients and the exact support of P."""
+
+import math
+
+import pytest
+import torch
+
+import torchprime_amd as tpa
+from oracle import tprime_oracle as orc
+from tests.util import assert_close, heads_view, packed_segment_ids
+from torchprime_amd import parallelism_utils as pu
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _check(B, Hq, Hkv, S, D, dtype=torch.bfloat16, causal=True, seg=None, window=None, soft_cap=None, q_positions=None,
+           causal_offset=0, Skv=None, seed=0):
+  Skv = S if Skv is None else Skv
+  q, k, v, do = (heads_view(B, h, s_, D, seed + i, dtype) for i, (h, s_) in enumerate(((Hq, S), (Hkv, Skv), (Hkv, Skv), (Hq, S))))
+  sm = 1.0 / math.sqrt(D)
+  qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+  qp = None if q_positions is None else torch.as_tensor(q_positions).to(DEV)
+  out = tpa.ops.attention(qd, kd, vd, None if seg is None else seg.to(DEV), sm, causal, window=window, soft_cap=soft_cap,
+                          q_positions=qp, causal_offset=causal_offset)
+  out.backward(do.to(DEV))
+  kw = dict(window=window, soft_cap=soft_cap, q_positions=q_positions, causal_offset=causal_offset)
+  o_ref, dq_ref, dk_ref, dv_ref = orc.attention_grads_ref(q, k, v, do, seg, causal, sm, torch.float64, **kw)
+  assert_close(out, o_ref, "out")
+  assert_close(qd.grad, dq_ref, "dq", scale_abs=True)
+  assert_close(kd.grad, dk_ref, "dk", scale_abs=True)
+  assert_close(vd.grad, dv_ref, "dv", scale_abs=True)
+
+
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("causal,window", [(True, (100, 100)), (True, (17, None)), (False, (64, 64)), (False, (0, 200)), (False, (300, None)),
+                                            (True, (1000, 1000))])
+def test_sliding_window_fwd_bwd(D, causal, window):
+  _check(2, 4, 2, 520, D, causal=causal, window=window)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_sliding_window_with_segments_and_ragged_kv(dtype):
+  seg, _ = packed_segment_ids(2, 333, 10, 150, seed=2)
+  _check(2, 4, 2, 333, 128, dtype=dtype, causal=True, seg=seg, window=(40, 40))
+  _check(1, 2, 1, 130, 64, dtype=dtype, causal=False, window=(50, 20), Skv=300)
+
+
+@pytest.mark.parametrize("D,causal", [(128, True), (64, True), (128, False)])
+def test_soft_cap_fwd_bwd(D, causal):
+  _check(1, 4, 2, 300, D, causal=causal, soft_cap=2.0)       # caps visibly: |logit| reaches ~3 with N(0,1) inputs
+  _check(1, 2, 2, 200, D, causal=causal, soft_cap=30.0, window=(64, 64) if not causal else None)
+
+
+@pytest.mark.parametrize("cp_size,D", [(2, 128), (4, 128), (4, 64)])
+def test_load_balanced_causal_mask_fwd_bwd(cp_size, D):
+  S = 512
+  mask = pu.LoadBalancedCausalMask(shape=(S, S), cp_size=cp_size)
+  _check(2, 4, 2, S, D, causal=True, q_positions=mask.q_sequence)
+  _check(1, 2, 2, S, D, causal=True, q_positions=mask.q_sequence, causal_offset=5)
+
+
+def test_rows_without_any_allowed_key_give_zero_output_and_gradients():
+  """A negative causal offset leaves the first rows with no key at all: the kernels' convention for such rows,
+  out = 0, lse = -inf, no gradient through them (where the eager formula would give NaN), executed on the device."""
+  B, H, S, D, off = 1, 2, 200, 128, -7
+  q, k, v, do = (heads_view(B, H, S, D, i, torch.bfloat16) for i in range(4))
+  qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+  out, lse = torch.ops.tprime.attn_fwd_masked(qd, kd, vd, None, None, D**-0.5, True, off, -1, -1, 0.0)
+  out.backward(do.to(DEV))
+  assert out[:, :, : -off].abs().max().item() == 0 and (lse[:, :, : -off] == float("-inf")).all()
+  assert torch.isfinite(out.float()).all() and torch.isfinite(lse[:, :, -off:]).all()
+  assert qd.grad[:, :, : -off].abs().max().item() == 0
+  o_ref, dq_ref, dk_ref, dv_ref = orc.attention_grads_ref(q, k, v, do, None, True, D**-0.5, torch.float64, causal_offset=off)
+  assert_close(out, o_ref, "out")
+  assert_close(qd.grad, dq_ref, "dq", scale_abs=True)
+  assert_close(kd.grad, dk_ref, "dk", scale_abs=True)
+  assert_close(vd.grad, dv_ref, "dv", scale_abs=True)
+
+
+@pytest.mark.parametrize("kind", ["window_causal", "window_full", "load_balanced", "window_segments"])
+def test_mask_pattern_exact_extensions(kind):
+  """The support of P, recovered through the public op with one-hot V blocks, equals the closed-form mask."""
+  B, H, S, D = 1, 2, 192, 64
+  kw, seg, causal = {}, None, True
+  if kind == "window_causal":
+    kw = dict(window=(37, 37))
+  elif kind == "window_full":
+    kw, causal = dict(window=(20, 45)), False
+  elif kind == "load_balanced":
+    kw = dict(q_positions=pu.LoadBalancedCausalMask(shape=(S, S), cp_size=4).q_sequence)
+  else:
+    kw, seg = dict(window=(50, 50)), packed_segment_ids(B, S, 5, 70, seed=4)[0]
+  q = heads_view(B, H, S, D, 1, torch.bfloat16, 0.3).to(DEV)
+  k = heads_view(B, H, S, D, 2, torch.bfloat16, 0.3).to(DEV)
+  allowed = orc.allowed_mask(seg, S, S, causal, **kw)[0]
+  dkw = {n: (torch.as_tensor(x).to(DEV) if n == "q_positions" else x) for n, x in kw.items()}
+  P = torch.zeros((H, S, S))
+  for j0 in range(0, S, D):
+    v = torch.zeros((B, H, S, D), dtype=torch.bfloat16)
+    for j in range(j0, min(j0 + D, S)):
+      v[:, :, j, j - j0] = 1
+    o = tpa.ops.attention(q, k, v.to(DEV), None if seg is None else seg.to(DEV), None, causal, **dkw)
+    P[:, :, j0 : j0 + D] = o[0, :, :, : min(D, S - j0)].float().cpu()
+  assert torch.equal(P > 0, allowed[None].expand_as(P)), "support of P differs from the mask"
+  assert_close(P.sum(-1), torch.ones(H, S), "rows sum to 1", max_abs=2e-2)
+
+
+def test_wrapper_and_module_paths():
+  B, Hq, Hkv, S, D, cp = 2, 4, 2, 256, 128, 4
+  q, k, v = (heads_view(B, h, S, D, s, torch.bfloat16) for h, s in ((Hq, 1), (Hkv, 2), (Hkv, 3)))
+  qs = (q.float() / math.sqrt(D)).to(torch.bfloat16)  # callers pre-scale q (attention.py:107)
+  # sliding window through the config JSON, soft cap through the argument (kernel_utils.py:266-275, 292)
+  cfg = tpa.SplashAttentionConfig(attentiontype_local_sliding=True, slide_window_size=48).to_json()
+  res = tpa.tpu_splash_attention_jax_call_wrapper(None, qs.to(DEV), k.to(DEV), v.to(DEV), cfg, None, True, attn_logits_soft_cap=20.0)
+  ref, _ = orc.attention_ref(qs, k, v, None, True, 1.0, torch.float64, window=(48, 48), soft_cap=20.0)
+  assert_close(res[0], ref, "window + soft cap via wrapper")
+  # load-balanced causal mask object, causal=False as the reference passes it (attention.py:110-119)
+  mask = pu.LoadBalancedCausalMask(shape=(S, S), cp_size=cp)
+  res = tpa.tpu_splash_attention_jax_call_wrapper(mask, qs.to(DEV), k.to(DEV), v.to(DEV), None, None, False, q_seq_shards=cp)
+  ref, _ = orc.attention_ref(qs, k, v, None, True, 1.0, torch.float64, q_positions=mask.q_sequence)
+  assert_close(res[0], ref, "LoadBalancedCausalMask via wrapper")
+  # AttentionModule with load_balance_cp: inputs in the striped order; equals plain causal attention on the original
+  # order, re-striped
+  cfgm = tpa.Config(attention_kernel="splash_attention", num_attention_heads=Hq, num_key_value_heads=Hkv, attention_dropout=False,
+                    load_balance_cp=True, context=cp)
+  striped = [pu.reorder_sequence(t, cp, seq_dim=2) for t in (q, k, v)]
+  out = tpa.AttentionModule(cfgm)(*(t.to(DEV) for t in striped))
+  plain, _ = orc.attention_ref(q, k, v, None, True, 1 / math.sqrt(D), torch.float64)
+  assert_close(out, pu.reorder_sequence(plain, cp, seq_dim=2), "AttentionModule, load_balance_cp")
+  plain_dev = tpa.AttentionModule(tpa.Config(attention_kernel="splash_attention"))(q.to(DEV), k.to(DEV), v.to(DEV))
+  assert_close(out, pu.reorder_sequence(plain_dev.float().cpu(), cp, seq_dim=2), "vs the plain causal kernel")
+
+
+def test_full_size_sliding_window_slice():
+  """Llama-3-8B layer shape with a 1024-token causal window: one (batch, kv group) slice against the oracle."""
+  B, Hq, Hkv, S, D, W = 2, 32, 8, 8192, 128, 1024
+  q, k, v, do = (heads_view(B, h, S, D, 40 + i, torch.bfloat16) for i, h in enumerate((Hq, Hkv, Hkv, Hq)))
+  qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+  out = tpa.ops.attention(qd, kd, vd, None, None, True, window=(W, W))
+  out.backward(do.to(DEV))
+  b, g = 1, 3
+  hs = slice(g * 4, g * 4 + 4)
+  o_ref, dq_ref, dk_ref, dv_ref = orc.attention_grads_ref(q[b : b + 1, hs], k[b : b + 1, g : g + 1], v[b : b + 1, g : g + 1], do[b : b + 1, hs],
+                                                          None, True, None, torch.float32, window=(W, W))
+  assert_close(out[b : b + 1, hs], o_ref, "out")
+  assert_close(qd.grad[b : b + 1, hs], dq_ref, "dq", scale_abs=True)
+  assert_close(kd.grad[b : b + 1, g : g + 1], dk_ref, "dk", scale_abs=True)
+  assert_close(vd.grad[b : b + 1, g : g + 1], dv_ref, "dv", scale_abs=True)

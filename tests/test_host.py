@@ -48,7 +48,11 @@ def test_c_abi_validates_arguments_before_launching():
   s96 = _lib._I64x3(8 * 2 * 96, 96, 2 * 96)
   assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 96, 96, s96, s96, s96, s96, 0.1, 1, 0, None) == -2  # head dim
   assert b"not built" in lib.tp_last_error()
-  assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 128, 128, z3, z3, z3, z3, 0.1, 1, 2, None) == -2  # fp32
+  assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 128, 128, z3, z3, z3, z3, 0.1, 1, 7, None) == -2  # unknown dtype
+  s192, s128 = _lib._I64x3(8 * 2 * 192, 192, 2 * 192), _lib._I64x3(8 * 2 * 128, 128, 2 * 128)
+  assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 192, 128, s192, s192, s128, s128, 0.1, 1, 2, None) == -2  # fp32: dims 64 / 128 only
+  assert lib.tp_attn_fwd_masked(p, p, p, None, None, p, p, 1, 2, 2, 8, 8, 192, 128, s192, s192, s128, s128, 0.1, 1, 0, 4, -1, 0.0, 0, None) == -2  # window at 192/128
+  assert lib.tp_attn_fwd_masked(p, p, p, None, None, p, p, 1, 2, 2, 8, 8, 128, 128, s128, s128, s128, s128, 0.1, 1, 0, 4, -1, 0.0, 2, None) == -2  # window in fp32
   assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 128, 128, z3, z3, z3, z3, -1.0, 1, 0, None) == -1  # scale
   assert lib.tp_attn_fwd(p, p, p, p, p, p, 1, 2, 2, 8, 16, 128, 128, z3, z3, z3, z3, 0.1, 1, 0, None) == -1  # seg, Sq != Skv
   assert lib.tp_rope_apply(p, None, p, p, None, p, None, 1, 2, 0, 8, 24, z3, z3, z3, z3, 0, 24, 0, 0, 0, 0, 0, None) == -2  # D % 16
@@ -151,16 +155,21 @@ def test_config_and_splash_config():
 
 def test_attention_module_cpu_side_errors():
   q = torch.zeros(1, 2, 8, 64, dtype=torch.bfloat16)
+  # load-balanced context parallelism reorders K / V on the host side and then needs the GPU kernels like any other call
   m = tpa.AttentionModule(tpa.Config(attention_kernel="splash_attention", load_balance_cp=True, context=2))
-  with pytest.raises(NotImplementedError, match="context parallelism"):
+  with pytest.raises(RuntimeError, match="no CPU path"):
     m(q, q, q)
+  with pytest.raises(ValueError, match="not a multiple"):
+    m(q[:, :, :6], q[:, :, :6], q[:, :, :6])  # 6 rows do not split into 2 * cp_size chunks
   m = tpa.AttentionModule(tpa.Config(attention_kernel="flash_attention", num_attention_heads=2, num_key_value_heads=2))
   with pytest.raises(RuntimeError, match="no CPU path"):
     m(q, q, q)
-  with pytest.raises(NotImplementedError, match="custom mask"):
+  with pytest.raises(NotImplementedError, match="mask objects of type"):
     tpa.tpu_splash_attention_jax_call_wrapper(object(), q, q, q, "{}", None, True)
-  with pytest.raises(NotImplementedError, match="soft_cap"):
-    tpa.tpu_splash_attention_jax_call_wrapper(None, q, q, q, "{}", None, True, attn_logits_soft_cap=30.0)
+  with pytest.raises(ValueError, match="mask shape"):
+    tpa.tpu_splash_attention_jax_call_wrapper(tpa.parallelism_utils.LoadBalancedCausalMask((16, 16), cp_size=2), q, q, q, "{}", None, False)
+  with pytest.raises(ValueError, match="soft_cap must be positive"):
+    tpa.tpu_splash_attention_jax_call_wrapper(None, q, q, q, "{}", None, True, attn_logits_soft_cap=-1.0)
 
 
 def test_ops_trace_with_fake_tensors():

@@ -289,7 +289,7 @@ def test_attention_ref_fully_masked_row_convention():
   s = torch.full((1, 1, 3, 3), float("-inf"))
   assert torch.isnan(torch.softmax(s, -1)).all()
   import unittest.mock as um
-  with um.patch.object(orc, "allowed_mask", lambda seg, ql, kl, c: torch.tensor([[[True, False, False], [False, False, False], [True, True, True]]])):
+  with um.patch.object(orc, "allowed_mask", lambda seg, ql, kl, c, *rest: torch.tensor([[[True, False, False], [False, False, False], [True, True, True]]])):
     out, lse = orc.attention_ref(q, q, q, None, True, None, torch.float64)
   assert out[0, 0, 1].abs().max() == 0 and lse[0, 0, 1] == float("-inf")
   assert torch.isfinite(out).all() and torch.isfinite(lse[0, 0, [0, 2]]).all()
@@ -515,3 +515,42 @@ def test_swiglu_and_cross_entropy_explicit_forms():
       n += 1
   assert n == B * (S - 1) - 1
   assert orc.cross_entropy_loss(logits, labels, V).item() == pytest.approx(total / n, rel=1e-12)
+
+
+# ---- mask extensions ---------------------------------------------------------------------------------------
+def test_window_is_a_band_matrix_and_soft_cap_explicit():
+  S = 23
+  ones = torch.ones(S, S, dtype=torch.bool)
+  for left, right in ((4, 0), (3, 5), (None, 2), (6, None), (0, 0)):
+    band = ones.clone()
+    if left is not None:
+      band &= torch.triu(ones, diagonal=-left)
+    if right is not None:
+      band &= torch.tril(ones, diagonal=right)
+    assert torch.equal(orc.allowed_mask(None, S, S, False, window=(left, right))[0], band)
+    assert torch.equal(orc.allowed_mask(None, S, S, True, window=(left, right))[0], band & torch.tril(ones))
+  q, k, v = randn((1, 2, 5, 8), 81).double(), randn((1, 2, 5, 8), 82).double(), randn((1, 2, 5, 8), 83).double()
+  out, _ = orc.attention_ref(q, k, v, None, True, 0.4, torch.float64, soft_cap=1.5)
+  for h in range(2):
+    for i in range(5):
+      sc = [1.5 * math.tanh(0.4 * float((q[0, h, i] * k[0, h, j]).sum()) / 1.5) for j in range(i + 1)]
+      p = torch.softmax(torch.tensor(sc, dtype=torch.float64), 0)
+      torch.testing.assert_close(out[0, h, i], (p[:, None] * v[0, h, : i + 1]).sum(0), rtol=1e-10, atol=1e-12)
+
+
+@pytest.mark.parametrize("cp_size", [2, 4])
+def test_load_balanced_causal_mask_is_causal_attention_in_the_original_order(cp_size):
+  """Queries in the striped order against keys in the original order under LoadBalancedCausalMask == plain causal
+  attention on the original order, re-striped: reorder o attention o reorder^-1."""
+  from torchprime_amd import parallelism_utils as pu
+
+  B, H, S, D = 1, 2, 32, 8
+  q, k, v = randn((B, H, S, D), 91).double(), randn((B, H, S, D), 92).double(), randn((B, H, S, D), 93).double()
+  plain, _ = orc.attention_ref(q, k, v, None, True, None, torch.float64)
+  mask = pu.LoadBalancedCausalMask(shape=(S, S), cp_size=cp_size)
+  q_striped = pu.reorder_sequence(q, cp_size, seq_dim=2)
+  out, _ = orc.attention_ref(q_striped, k, v, None, True, None, torch.float64, q_positions=mask.q_sequence)
+  torch.testing.assert_close(out, pu.reorder_sequence(plain, cp_size, seq_dim=2), rtol=1e-12, atol=1e-12)
+  assert torch.equal(orc.allowed_mask(None, S, S, True, q_positions=mask.q_sequence)[0], torch.from_numpy(mask.dense()))
+  off = pu.LoadBalancedCausalMask(shape=(S, S), cp_size=cp_size, offset=-3)
+  assert torch.equal(orc.allowed_mask(None, S, S, True, q_positions=off.q_sequence, causal_offset=-3)[0], torch.from_numpy(off.dense()))

@@ -17,7 +17,7 @@ Compute runs only in ``libtprime_hip.so`` (hand-written HIP kernels reached thro
 ops in :mod:`torchprime_amd.ops`); there is no CPU or torch-math fallback.
 """
 
-from . import kernel_utils, ops, rope  # noqa: F401
+from . import kernel_utils, ops, parallelism_utils, rope  # noqa: F401
 from .attention import AttentionModule, repeat_kv
 from .blocks import DeepseekV3Attention, LlamaAttention, MixtralAttention
 from .config import Config

@@ -16,7 +16,7 @@ from typing import Any
 import torch
 from torch import nn
 
-from . import ops
+from . import kernel_utils, ops, parallelism_utils
 from .config import has_key
 
 
@@ -78,8 +78,23 @@ class AttentionModule(nn.Module):
     kv_seq_len = key_states.shape[-2]
     self.partition_spec = None  # no mesh on one GPU (attention.py:61-67)
 
-    if has_key(self.config, "load_balance_cp") and self.config.load_balance_cp:
-      raise NotImplementedError("load-balanced context parallelism needs a device mesh; this build is single-GPU")
+    if kernel == "splash_attention" and has_key(self.config, "load_balance_cp") and self.config.load_balance_cp:
+      # Load-balanced context parallelism (attention.py:75-119), the part one GPU sees: the sequence arrives in the
+      # striped order, K / V are put back into the original order, and a causal mask whose query rows are in the
+      # striped order (LoadBalancedCausalMask) relates the two.  The kernel evaluates that mask from q_sequence.
+      cp_size = self.config.context
+      key_states = parallelism_utils.reorder_sequence(tensor=key_states, cp_size=cp_size, seq_dim=2, to_contiguous=True)
+      value_states = parallelism_utils.reorder_sequence(tensor=value_states, cp_size=cp_size, seq_dim=2, to_contiguous=True)
+      custom_mask = parallelism_utils.LoadBalancedCausalMask(shape=(q_len, q_len), cp_size=cp_size)
+      attn_output = kernel_utils.tpu_splash_attention_jax_call_wrapper(
+        mask=custom_mask, query=query_states, key=key_states, value=value_states, config=None, decoder_segment_ids=None,
+        causal=False, q_seq_shards=cp_size, sm_scale=1.0 / math.sqrt(head_dim),
+      )[0]  # fmt: skip
+      if attn_output.size() != (bsz, num_heads, q_len, head_dim):
+        raise ValueError(
+          f"`attn_output` should be of size {(bsz, num_heads, q_len, head_dim)}, but is {attn_output.size()}"
+        )
+      return attn_output
 
     if kernel in ("splash_attention", "flash_attention"):
       # both kernel branches are causal and never see attention_mask (attention.py:121-123, 144-150)

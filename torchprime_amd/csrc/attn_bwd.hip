@@ -61,6 +61,7 @@ struct BwdArgs {
   int64_t qs[3], ks[3], vs[3], os[3], dos[3], dqs[3], dks[3], dvs[3];
   float scale_log2;  // sm_scale * log2(e)
   float sm_scale;
+  MaskExt mx;
 };
 
 // ------------------------------------------------------------------------------------------------
@@ -363,7 +364,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   const int kv0 = tile * BNK;  // low kv tiles see the most queries: they start first
   const int wkv0 = kv0 + wave * 32;
   const int Sq = a.Sq, Skv = a.Skv;
-  const int32_t* segb = SEG ? a.seg + (int64_t)b * Skv : nullptr;
+  // GEN: the instantiation that also evaluates the mask extensions (and then may run without segment ids)
+  constexpr bool GEN = !CAUSAL && SEG;
+  const bool has_seg = SEG && (!GEN || a.seg != nullptr);
+  const bool ext = GEN && a.mx.on;
+  const bool capped = GEN && a.mx.cap_in != 0.f;
+  const bool has_pos = ext && a.mx.qpos != nullptr;
+  const int32_t* segb = has_seg ? a.seg + (int64_t)b * Skv : nullptr;
 
   // ---- K, V fragments of this wave's 32 kv rows (B operands: lane = kv column)
   v8 kf[KS_QK], vf[KS_DV];
@@ -376,7 +383,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
 #pragma unroll
     for (int ks = 0; ks < KS_DV; ks++) vf[ks] = *(const v8*)(vp + 16 * ks);
   }
-  const int segk = SEG ? segb[kvrow] : 0;
+  const int segk = has_seg ? segb[kvrow] : 0;
 
   // ---- query tiles to visit: causal => tiles that reach the first kv row; segments => id ranges overlap
   const int nqt_all = (Sq + BMQ - 1) / BMQ;
@@ -386,6 +393,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   int* qmax = qmin + nqt;
   int* active = qmax + nqt;
   int* bk = active + nqt;  // 8 ints: per-wave (min,max) of kv ids
+  int* pmin = bk + 8;      // per query tile: (min,max) of the rows' positions in the key order (mask extensions)
+  int* pmax = pmin + nqt;
   int nact = nqt;
   int wkmin = 0, wkmax = 0;
   if (SEG) {
@@ -398,14 +407,27 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     wkmin = __builtin_amdgcn_readfirstlane(wkmin);
     wkmax = __builtin_amdgcn_readfirstlane(wkmax);
     if (lane == 0) { bk[2 * wave] = wkmin; bk[2 * wave + 1] = wkmax; }
-    seg_tile_ranges(segb, Sq, qt_first, nqt_all, qmin, qmax, tid, 256);
+    if (has_seg) {
+      seg_tile_ranges(segb, Sq, qt_first, nqt_all, qmin, qmax, tid, 256);
+    } else {
+      for (int t = tid; t < nqt; t += 256) { qmin[t] = 0; qmax[t] = 0; }
+    }
+    if (ext) {
+      if (has_pos) {
+        seg_tile_ranges(a.mx.qpos, Sq, qt_first, nqt_all, pmin, pmax, tid, 256);
+      } else {
+        for (int t = tid; t < nqt; t += 256) { pmin[t] = (qt_first + t) * BMQ; pmax[t] = min((qt_first + t) * BMQ + BMQ - 1, Sq - 1); }
+      }
+    }
     __syncthreads();
     const int bkmin = min(min(bk[0], bk[2]), min(bk[4], bk[6]));
     const int bkmax = max(max(bk[1], bk[3]), max(bk[5], bk[7]));
     int cnt = 0;
     for (int base = 0; base < nqt; base += 64) {
       const int t = base + lane;
-      const bool act = t < nqt && !(qmax[t] < bkmin || qmin[t] > bkmax);
+      bool act = t < nqt && !(qmax[t] < bkmin || qmin[t] > bkmax);
+      // (band: some row of the tile must reach into this workgroup's 128 kv rows)
+      if (ext && act) act = kv0 <= pmax[t] + a.mx.hi_off && kv0 + BNK - 1 >= pmin[t] - a.mx.lo_off;
       const unsigned long long m = __ballot(act);
       if (act && wave == 0) active[cnt + __popcll(m & ((1ull << lane) - 1ull))] = t;
       cnt += __popcll(m);
@@ -435,8 +457,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
                 smem + DO_AT + buf * DO_BYTES, wave);
     // waves 0..2 fetch one 64-entry row vector each: 4 bytes per lane, rows past Sq arrive as zeros
     const int64_t ro = ((int64_t)b * a.Hq + hq) * Sq;
-    const void* src = wave == 0 ? (const void*)(lse2 + ro) : wave == 1 ? (const void*)(a.delta + ro) : (const void*)segb;
-    if (wave < 2 || (SEG && wave == 2))
+    const void* src = wave == 0 ? (const void*)(lse2 + ro) : wave == 1 ? (const void*)(a.delta + ro)
+                    : wave == 2 ? (const void*)segb : (const void*)a.mx.qpos;
+    if (wave < 2 || (wave == 2 && has_seg) || (wave == 3 && has_pos))
       dma_dword(make_rsrc_words(src, (unsigned)Sq * 4u), (unsigned)(qt * BMQ) * 4u, rows_base + rslot * ROW_BYTES + wave * BMQ * 4, lane);
   };
 
@@ -475,6 +498,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       const int lo = qmin[active[idx]], hi = qmax[active[idx]];
       skip = skip || hi < wkmin || lo > wkmax;
       need_mask = need_mask || !(lo == hi && wkmin == wkmax && lo == wkmin);
+    }
+    if (ext) {
+      const int plo = pmin[active[idx]], phi = pmax[active[idx]];
+      skip = skip || wkv0 > phi + a.mx.hi_off || wkv0 + 31 < plo - a.mx.lo_off;
+      need_mask = need_mask || capped || !(wkv0 >= phi - a.mx.lo_off && wkv0 + 31 <= plo + a.mx.hi_off);
     }
     return skip ? 0 : (need_mask ? 2 : 1);
   };
@@ -555,6 +583,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       const float* lsel = (const float*)(rows_base + rslot * ROW_BYTES);
       const float* deltal = lsel + BMQ;
       const int* segl = (const int*)(deltal + BMQ);
+      const int* posl = segl + BMQ;  // query positions of the tile's rows (mask extensions)
       const int rnext = rslot >= 1 ? rslot - 1 : 2;  // (it + 2) % 3, the slot tile t-1 used
       // LDS destinations of this wave's loads of tile t+2 (scalar byte addresses)
       const unsigned dma_q = lds_base + (unsigned)(Q_AT + buf * Q_BYTES) + wave_q;
@@ -567,9 +596,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         nx.rq = make_rsrc_words((const T*)a.q + b * a.qs[0] + hq * a.qs[1], issue_next ? q_span : 0u);
         nx.ro = make_rsrc_words((const T*)a.dout + b * a.dos[0] + hq * a.dos[1], issue_next ? do_span : 0u);
         const int64_t ro = ((int64_t)b * a.Hq + hq) * Sq;
-        const void* src = wave == 0 ? (const void*)(lse2 + ro) : wave == 1 ? (const void*)(a.delta + ro) : (const void*)segb;
-        // wave 3 (and wave 2 without segment ids) fetches nothing: size 0
-        nx.rr = make_rsrc_words(src, (issue_next && (wave < 2 || (SEG && wave == 2))) ? (unsigned)Sq * 4u : 0u);
+        const void* src = wave == 0 ? (const void*)(lse2 + ro) : wave == 1 ? (const void*)(a.delta + ro)
+                        : wave == 2 ? (const void*)segb : (const void*)a.mx.qpos;
+        // a wave with no row vector to fetch (wave 2 without segment ids, wave 3 without query positions): size 0
+        nx.rr = make_rsrc_words(src, (issue_next && (wave < 2 || (wave == 2 && has_seg) || (wave == 3 && has_pos))) ? (unsigned)Sq * 4u : 0u);
       }
       {
         const int qt = issue_next ? qtile_of(n_idx) : 0;
@@ -614,6 +644,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         // order, so each group is requested a ring depth or more before its first use: waiting for it then waits
         // for no fragment that is not due anyway
         f32x4 nl0[4], nl1[4], nd0[4], nd1[4];
+        float fc[2][16];  // soft cap: 1 - tanh^2 of every score, kept from P to dS
 
         auto frag = [&](auto I) -> v8 {
           constexpr int i = decltype(I)::value;
@@ -664,17 +695,34 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
               const int e = EPS * (k % QS) + e2, v = 4 * vq + e;
               if constexpr (IS_P) {
                 const f32x4 (&nl)[4] = qb == 0 ? nl0 : nl1;
-                float pv = fast_exp2(__builtin_fmaf(s[qb][v], c, nl[vq][e]));
+                float sval = s[qb][v];
+                if (GEN && MASKED) {
+                  if (capped) {
+                    const float th = fast_tanh(sval * a.mx.cap_in);
+                    fc[qb][v] = 1.f - th * th;
+                    sval = a.mx.cap_out * th;
+                  }
+                }
+                float pv = fast_exp2(__builtin_fmaf(sval, c, nl[vq][e]));
                 if (MASKED) {
                   const int r = qb * 32 + 8 * vq + 4 * g + e;
                   const int qrow = qi0 + r;
-                  const bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || segl[r] == segk);
+                  bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || !has_seg || segl[r] == segk);
+                  if (GEN) {
+                    if (ext) {
+                      const int qp = has_pos ? posl[r] : qrow;
+                      ok = ok && kvcol >= qp - a.mx.lo_off && kvcol <= qp + a.mx.hi_off;
+                    }
+                  }
                   pv = ok ? pv : 0.f;
                 }
                 asm volatile("" : "+v"(pv));  // anchors the computation in this slot (it would sink past the barrier)
                 s[qb][v] = pv;
               } else {
                 float dsv = s[qb][v] * dp[qb][v];
+                if (GEN && MASKED) {
+                  if (capped) dsv *= fc[qb][v];  // derivative of the capped score with respect to the raw one
+                }
                 asm volatile("" : "+v"(dsv));
                 dp[qb][v] = dsv;
               }
@@ -937,7 +985,11 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   const int Sq = a.Sq, Skv = a.Skv;
   const T* kb = (const T*)a.k + b * a.ks[0] + hk * a.ks[1];
   const T* vb = (const T*)a.v + b * a.vs[0] + hk * a.vs[1];
-  const int32_t* segb = SEG ? a.seg + (int64_t)b * Skv : nullptr;
+  constexpr bool GEN = !CAUSAL && SEG;  // also evaluates the mask extensions (and may then run without segment ids)
+  const bool has_seg = SEG && (!GEN || a.seg != nullptr);
+  const bool ext = GEN && a.mx.on;
+  const bool capped = GEN && a.mx.cap_in != 0.f;
+  const int32_t* segb = has_seg ? a.seg + (int64_t)b * Skv : nullptr;
 
   const int kv_end = CAUSAL ? min(Skv, q0 + BM) : Skv;
   const int ntiles = (kv_end + BN - 1) / BN;
@@ -957,7 +1009,22 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   const float lraw = a.lse[ro];
   const float lse_s = (lraw == -INFINITY) ? INFINITY : lraw * LOG2E;
   const float ndelta_s = a.delta[ro];  // -rowsum(dO o O)
-  const int segq = SEG ? segb[qrow_c] : 0;
+  const int segq = has_seg ? segb[qrow_c] : 0;
+  // band of allowed keys of this lane's query row, and the positions' extent over the wave
+  int lo_q = -BAND_INF, hi_q = BAND_INF, wpmin = 0, wpmax = 0;
+  if (ext) {
+    const int qp = a.mx.qpos ? a.mx.qpos[qrow_c] : qrow_c;
+    lo_q = qp - a.mx.lo_off;
+    hi_q = qp + a.mx.hi_off;
+    wpmin = qp; wpmax = qp;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) {
+      wpmin = min(wpmin, __shfl_xor(wpmin, o, 64));
+      wpmax = max(wpmax, __shfl_xor(wpmax, o, 64));
+    }
+    wpmin = __builtin_amdgcn_readfirstlane(wpmin);
+    wpmax = __builtin_amdgcn_readfirstlane(wpmax);
+  }
 
   int* kvmin = (int*)(smem + META_AT);
   int* kvmax = kvmin + ntiles;
@@ -974,16 +1041,24 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
     }
     wqmin = __builtin_amdgcn_readfirstlane(wqmin);
     wqmax = __builtin_amdgcn_readfirstlane(wqmax);
-    if (lane == 0) { bq[2 * wave] = wqmin; bq[2 * wave + 1] = wqmax; }
-    seg_tile_ranges(segb, Skv, 0, ntiles, kvmin, kvmax, tid, 64 * NW);
+    if (lane == 0) { bq[2 * wave] = wqmin; bq[2 * wave + 1] = wqmax; bq[2 * NW + 2 * wave] = wpmin; bq[2 * NW + 2 * wave + 1] = wpmax; }
+    if (has_seg) {
+      seg_tile_ranges(segb, Skv, 0, ntiles, kvmin, kvmax, tid, 64 * NW);
+    } else {
+      for (int t = tid; t < ntiles; t += 64 * NW) { kvmin[t] = 0; kvmax[t] = 0; }
+    }
     __syncthreads();
-    int bqmin = bq[0], bqmax = bq[1];
+    int bqmin = bq[0], bqmax = bq[1], bpmin = bq[2 * NW], bpmax = bq[2 * NW + 1];
 #pragma unroll
-    for (int w = 1; w < NW; w++) { bqmin = min(bqmin, bq[2 * w]); bqmax = max(bqmax, bq[2 * w + 1]); }
+    for (int w = 1; w < NW; w++) {
+      bqmin = min(bqmin, bq[2 * w]); bqmax = max(bqmax, bq[2 * w + 1]);
+      bpmin = min(bpmin, bq[2 * NW + 2 * w]); bpmax = max(bpmax, bq[2 * NW + 2 * w + 1]);
+    }
+    const int b_lo = ext ? bpmin - a.mx.lo_off : -BAND_INF, b_hi = ext ? bpmax + a.mx.hi_off : BAND_INF;
     int cnt = 0;
     for (int base = 0; base < ntiles; base += 64) {
       const int t = base + lane;
-      const bool act = t < ntiles && !(kvmax[t] < bqmin || kvmin[t] > bqmax);
+      const bool act = t < ntiles && !(kvmax[t] < bqmin || kvmin[t] > bqmax) && t * BN <= b_hi && t * BN + BN - 1 >= b_lo;
       const unsigned long long m = __ballot(act);
       if (act && wave == 0) active[cnt + __popcll(m & ((1ull << lane) - 1ull))] = t;
       cnt += __popcll(m);
@@ -1019,7 +1094,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
 #pragma unroll
       for (int ii = 0; ii < 4; ii++) kst.r[0][ii] = buf_load16(rs, kst.vo[0][ii], off);
     }
-    if (SEG && tid < BN) sreg = segb[min(t * BN + tid, Skv - 1)];
+    if (has_seg && tid < BN) sreg = segb[min(t * BN + tid, Skv - 1)];
   };
   // (kslot: which transposed tile; the row-major buffer is buf)
   auto store_tile = [&](int buf, int kslot, int it) {
@@ -1133,6 +1208,10 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
         skip = skip || hi < wqmin || lo > wqmax;
         need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
       }
+      if (ext) {
+        skip = skip || kv0 > wpmax + a.mx.hi_off || kv0 + BN - 1 < wpmin - a.mx.lo_off;
+        need_mask = need_mask || capped || !(kv0 >= wpmax - a.mx.lo_off && kv0 + BN - 1 <= wpmin + a.mx.hi_off);
+      }
       auto body = [&](auto masked_c) {
         constexpr bool MASKED = decltype(masked_c)::value;
         v8 fr[NF];
@@ -1174,11 +1253,23 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
             constexpr int k = i - st, lo = (k * 16 + len - 1) / len, hi = ((k + 1) * 16 + len - 1) / len;
 #pragma unroll
             for (int v = lo; v < hi; v++) {
-              float pv = fast_exp2(__builtin_fmaf(sv[v], c, -lse_s));
+              float sval = sv[v], dcap = 1.f;
+              if (GEN && MASKED) {
+                if (capped) {
+                  const float th = fast_tanh(sval * a.mx.cap_in);
+                  dcap = 1.f - th * th;  // derivative of the capped score; P only feeds dS here, so it rides on P
+                  sval = a.mx.cap_out * th;
+                }
+              }
+              float pv = fast_exp2(__builtin_fmaf(sval, c, -lse_s));
               if (MASKED) {
                 const int kvl = nb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
                 const int kv = kv0 + kvl;
-                const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
+                bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
+                if (GEN) {
+                  ok = ok && kv >= lo_q && kv <= hi_q;
+                  pv *= dcap;
+                }
                 pv = ok ? pv : 0.f;
               }
               asm volatile("" : "+v"(pv));
@@ -1239,6 +1330,10 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
         skip = skip || hi < wqmin || lo > wqmax;
         need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
       }
+      if (ext) {
+        skip = skip || kv0 > wpmax + a.mx.hi_off || kv0 + BN - 1 < wpmin - a.mx.lo_off;
+        need_mask = need_mask || capped || !(kv0 >= wpmax - a.mx.lo_off && kv0 + BN - 1 <= wpmin + a.mx.hi_off);
+      }
       // The tile body is laid out slot by slot (one MFMA each, a scheduling barrier after every slot): the
       // LDS fragment of a slot is requested AHEAD slots earlier, and the element-wise work that turns
       // S^T, dP^T into the 16-bit operand dS^T is spread under the MFMAs of the following slots.
@@ -1294,11 +1389,23 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
             constexpr int k = i - st, lo = e0 + (k * n + len - 1) / len, hi = e0 + ((k + 1) * n + len - 1) / len;
   #pragma unroll
             for (int v = lo; v < hi; v++) {
-              float pv = fast_exp2(__builtin_fmaf(s[nb][v], c, -lse_s));
+              float sval = s[nb][v], dcap = 1.f;
+              if (GEN && MASKED) {
+                if (capped) {
+                  const float th = fast_tanh(sval * a.mx.cap_in);
+                  dcap = 1.f - th * th;
+                  sval = a.mx.cap_out * th;
+                }
+              }
+              float pv = fast_exp2(__builtin_fmaf(sval, c, -lse_s));
               if (MASKED) {
                 const int kvl = nb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
                 const int kv = kv0 + kvl;
-                const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
+                bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
+                if (GEN) {
+                  ok = ok && kv >= lo_q && kv <= hi_q;
+                  pv *= dcap;
+                }
                 pv = ok ? pv : 0.f;
               }
               float dsv = pv * (dp[nb][v] + ndelta_s);
@@ -1407,7 +1514,7 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
     constexpr int ROWS = 3 * BMQ * 16;
     constexpr int NBUF = (2 * BUF + ROWS + 4096 <= 160 * 1024) ? 2 : 1;
     const int nqt = (a.Sq + BMQ - 1) / BMQ;
-    const size_t smem = (size_t)NBUF * BUF + ROWS + (SEG ? (size_t)(3 * nqt + 8) * 4 : 0);
+    const size_t smem = (size_t)NBUF * BUF + ROWS + (SEG ? (size_t)(5 * nqt + 8) * 4 : 0);
     TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_bwd: Sq=%d needs %zu bytes of LDS (max 163840)", a.Sq, smem);
     auto kern = attn_bwd_dkdv_kernel<T, DQK, DV, NBUF, CAUSAL, SEG>;
     static bool attr_set = false;
@@ -1430,7 +1537,7 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
     constexpr int BUF = BN * RowTile<DQK>::STRIDE + BN * RowTile<DV>::STRIDE + DQK * TrTile64::ROW_BYTES + BN * 4;
     const int nt = (a.Skv + BN - 1) / BN;
     // (8 waves: a third transposed K tile)
-    const size_t smem = 2 * (size_t)BUF + (NW == 8 ? (size_t)DQK * TrTile64::ROW_BYTES : 0) + (SEG ? (size_t)(3 * nt + 2 * NW) * 4 : 0);
+    const size_t smem = 2 * (size_t)BUF + (NW == 8 ? (size_t)DQK * TrTile64::ROW_BYTES : 0) + (SEG ? (size_t)(3 * nt + 4 * NW) * 4 : 0);
     TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_bwd: Skv=%d needs %zu bytes of LDS (max 163840)", a.Skv, smem);
     auto kern = attn_bwd_dq_kernel<T, DQK, DV, NW, CAUSAL, SEG>;
     static bool attr_set = false;
@@ -1449,6 +1556,11 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
 
 template <typename T, int DQK, int DV>
 static int dispatch_bwd(const BwdArgs& a, int causal, hipStream_t st, void* const* ev) {
+  if (a.mx.on) {
+    // mask extensions: the general instantiation (causality is part of the band then)
+    if constexpr (DQK == DV && DQK <= 128) return launch_bwd<T, DQK, DV, false, true>(a, st, ev);
+    else TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_attn_bwd_masked: windows, soft cap and query positions are built for head dims 64 and 128");
+  }
   if (causal) {
     if (a.seg) return launch_bwd<T, DQK, DV, true, true>(a, st, ev);
     return launch_bwd<T, DQK, DV, true, false>(a, st, ev);
@@ -1493,13 +1605,13 @@ extern "C" size_t tp_attn_bwd_workspace_bytes(int B, int Hq, int Sq) {
   return 2 * (size_t)B * Hq * Sq * sizeof(float);  // delta and the log2-scaled LSE, one float per query row each
 }
 
-extern "C" int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, const void* v, const void* out,
-                              const float* lse, const int32_t* seg, void* dq, void* dk, void* dv, float* ws, int B, int Hq,
-                              int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t do_strides[3],
-                              const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
-                              const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
-                              const int64_t dv_strides[3], float sm_scale, int causal, int dtype, void* stream,
-                              void* const* events) {
+static int attn_bwd_impl(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                         const float* lse, const int32_t* seg, void* dq, void* dk, void* dv, float* ws, int B, int Hq,
+                         int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t do_strides[3],
+                         const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                         const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                         const int64_t dv_strides[3], float sm_scale, int causal, int dtype, void* stream,
+                         void* const* events, const MaskExt& mx) {
   TP_REQUIRE(dout && q && k && v && out && lse && dq && dk && dv && ws, TP_ERR_BAD_ARG, "tp_attn_bwd: null pointer");
   TP_REQUIRE(do_strides && q_strides && k_strides && v_strides && o_strides && dq_strides && dk_strides && dv_strides,
              TP_ERR_BAD_ARG, "tp_attn_bwd: null stride array");
@@ -1536,10 +1648,39 @@ extern "C" int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, co
   }
   a.scale_log2 = sm_scale * LOG2E;
   a.sm_scale = sm_scale;
+  a.mx = mx;
   hipStream_t st = (hipStream_t)stream;
   const int rc = dtype == TP_BF16 ? bwd_by_dims_bf16(a, Dqk, Dv, causal, st, events) : bwd_by_dims_f16(a, Dqk, Dv, causal, st, events);
   TP_REQUIRE(rc != TP_DIMS_NOT_BUILT, TP_ERR_UNSUPPORTED, "tp_attn_bwd: head dims (qk=%d, v=%d) not built", Dqk, Dv);
   return rc;
+}
+
+extern "C" int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                              const float* lse, const int32_t* seg, void* dq, void* dk, void* dv, float* ws, int B, int Hq,
+                              int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t do_strides[3],
+                              const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                              const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                              const int64_t dv_strides[3], float sm_scale, int causal, int dtype, void* stream,
+                              void* const* events) {
+  return attn_bwd_impl(dout, q, k, v, out, lse, seg, dq, dk, dv, ws, B, Hq, Hkv, Sq, Skv, Dqk, Dv, do_strides, q_strides,
+                       k_strides, v_strides, o_strides, dq_strides, dk_strides, dv_strides, sm_scale, causal, dtype, stream,
+                       events, no_mask_ext());
+}
+
+extern "C" int tp_attn_bwd_masked(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                                  const float* lse, const int32_t* seg, const int32_t* q_positions, void* dq, void* dk,
+                                  void* dv, float* ws, int B, int Hq, int Hkv, int Sq, int Skv, int Dqk, int Dv,
+                                  const int64_t do_strides[3], const int64_t q_strides[3], const int64_t k_strides[3],
+                                  const int64_t v_strides[3], const int64_t o_strides[3], const int64_t dq_strides[3],
+                                  const int64_t dk_strides[3], const int64_t dv_strides[3], float sm_scale, int causal,
+                                  int causal_offset, int window_left, int window_right, float logits_soft_cap, int dtype,
+                                  void* stream) {
+  TP_REQUIRE(sm_scale > 0.f, TP_ERR_BAD_ARG, "tp_attn_bwd_masked: sm_scale must be positive");
+  TP_REQUIRE(window_left < BAND_INF && window_right < BAND_INF && causal_offset > -BAND_INF && causal_offset < BAND_INF, TP_ERR_BAD_ARG,
+             "tp_attn_bwd_masked: window or offset out of range");
+  return attn_bwd_impl(dout, q, k, v, out, lse, seg, dq, dk, dv, ws, B, Hq, Hkv, Sq, Skv, Dqk, Dv, do_strides, q_strides,
+                       k_strides, v_strides, o_strides, dq_strides, dk_strides, dv_strides, sm_scale, causal, dtype, stream,
+                       nullptr, make_mask_ext(q_positions, causal, causal_offset, window_left, window_right, logits_soft_cap, sm_scale));
 }
 
 extern "C" int tp_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,

@@ -103,6 +103,47 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
 
+// tanh(x) = 1 - 2 / (exp(2x) + 1); saturates cleanly (exp -> inf gives 1, exp -> 0 gives -1)
+__device__ __forceinline__ float fast_tanh(float x) {
+  const float e = fast_exp2(x * (2.f * LOG2E));
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
+}
+
+// ---- mask extensions -------------------------------------------------------------------------------
+// Beyond causal / full and segment ids the functional API names three more things
+// (torchprime/utils/kernel_utils.py:259-294, torchprime/utils/parallelism_utils.py:87-152): a sliding window
+// (LocalMask), a soft cap on the logits, and a causal mask whose query rows are in another order than the keys
+// (LoadBalancedCausalMask: row i stands for position q_sequence[i]).  All three are a band per query row,
+//     allowed(i, j)  <=>  qp(i) - lo_off <= j <= qp(i) + hi_off,     qp(i) = qpos ? qpos[i] : i,
+// (causal: hi_off = offset, no window: the offsets are BAND_INF) plus s <- cap_out * tanh(s * cap_in) on the raw
+// scores.  Only the <non-causal, segment ids> instantiation of each kernel evaluates them (the host routes every
+// call that uses one there, with or without segment ids), so the other instantiations carry none of this.
+constexpr int BAND_INF = 1 << 29;
+struct MaskExt {
+  const int32_t* qpos;
+  int lo_off, hi_off;
+  float cap_in, cap_out;  // 0: no soft cap
+  int on;
+};
+// window_left / window_right < 0: unbounded on that side; soft_cap <= 0: none
+inline MaskExt make_mask_ext(const int32_t* q_positions, int causal, int causal_offset, int window_left, int window_right,
+                             float soft_cap, float sm_scale) {
+  MaskExt m;
+  m.qpos = q_positions;
+  const int hi_c = causal ? causal_offset : BAND_INF, hi_w = window_right >= 0 ? window_right : BAND_INF;
+  m.hi_off = hi_c < hi_w ? hi_c : hi_w;
+  m.lo_off = window_left >= 0 ? window_left : BAND_INF;
+  m.cap_in = soft_cap > 0.f ? sm_scale / soft_cap : 0.f;
+  m.cap_out = soft_cap > 0.f ? soft_cap / sm_scale : 0.f;
+  m.on = (q_positions != nullptr || window_left >= 0 || window_right >= 0 || soft_cap > 0.f || (causal && causal_offset != 0)) ? 1 : 0;
+  return m;
+}
+inline MaskExt no_mask_ext() {
+  MaskExt m;
+  m.qpos = nullptr; m.lo_off = BAND_INF; m.hi_off = BAND_INF; m.cap_in = 0.f; m.cap_out = 0.f; m.on = 0;
+  return m;
+}
+
 // ---- buffer loads ---------------------------------------------------------------------------------
 // K/V/Q/dO tiles are fetched with raw buffer loads: the per-thread byte offset inside a tile is computed
 // once, the tile's offset is a scalar, so the per-tile address arithmetic is free, and rows past the end

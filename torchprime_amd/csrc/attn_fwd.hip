@@ -31,10 +31,17 @@ struct FwdArgs {
   int B, Hq, Hkv, Sq, Skv, n_rep;
   int64_t qs[3], ks[3], vs[3], os[3];
   float scale_log2;  // sm_scale * log2(e)
+  MaskExt mx;
 };
 
+// Two workgroups per CU (256 registers per lane) where the kernel fits them; the 192-wide heads and the 128-wide
+// non-causal variants (run-time buffer index, mask extensions) need more and take one workgroup per CU instead of
+// spilling a hundred registers.
+template <int DQK, bool CAUSAL>
+constexpr int fwd_blocks_per_cu() { return (DQK > 128 || (DQK == 128 && !CAUSAL)) ? 1 : 2; }
+
 template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
-__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
+__global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_fwd_kernel(const FwdArgs a) {
   typedef typename MT<T>::v8 v8;
   constexpr int BN = 64;              // kv rows per LDS tile, processed as two halves of 32
   constexpr int BM = 128;             // q rows per workgroup, 32 per wave
@@ -74,7 +81,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
   const T* qb = (const T*)a.q + b * a.qs[0] + h * a.qs[1];
   const T* kb = (const T*)a.k + b * a.ks[0] + hk * a.ks[1];
   const T* vb = (const T*)a.v + b * a.vs[0] + hk * a.vs[1];
-  const int32_t* segb = SEG ? a.seg + (int64_t)b * Skv : nullptr;
+  // GEN: the instantiation that also evaluates the mask extensions (and then may run without segment ids)
+  constexpr bool GEN = !CAUSAL && SEG;
+  const bool has_seg = SEG && (!GEN || a.seg != nullptr);
+  const bool ext = GEN && a.mx.on;
+  const bool capped = GEN && a.mx.cap_in != 0.f;
+  const int32_t* segb = has_seg ? a.seg + (int64_t)b * Skv : nullptr;
 
   const int kv_end = CAUSAL ? min(Skv, q0 + BM) : Skv;
   const int ntiles = (kv_end + BN - 1) / BN;
@@ -87,13 +99,29 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) qf[ks] = *(const v8*)(qp + 16 * ks);
   }
-  const int segq = SEG ? segb[min(qrow, Sq - 1)] : 0;
+  const int segq = has_seg ? segb[min(qrow, Sq - 1)] : 0;
+  // band of allowed keys of this lane's query row, and its extent over the wave
+  int lo_q = -BAND_INF, hi_q = BAND_INF, wpmin = 0, wpmax = 0;
+  if (ext) {
+    const int qc = min(qrow, Sq - 1);
+    const int qp = a.mx.qpos ? a.mx.qpos[qc] : qc;
+    lo_q = qp - a.mx.lo_off;
+    hi_q = qp + a.mx.hi_off;
+    wpmin = qp; wpmax = qp;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) {
+      wpmin = min(wpmin, __shfl_xor(wpmin, o, 64));
+      wpmax = max(wpmax, __shfl_xor(wpmax, o, 64));
+    }
+    wpmin = __builtin_amdgcn_readfirstlane(wpmin);
+    wpmax = __builtin_amdgcn_readfirstlane(wpmax);
+  }
 
   // ---- segment bookkeeping: per-tile id ranges, list of tiles that can contain an allowed pair
   int* kvmin = (int*)(smem + 2 * BUF_BYTES);
   int* kvmax = kvmin + ntiles;
   int* active = kvmax + ntiles;
-  int* bq = active + ntiles;  // 8 ints: per-wave (min,max) of the query rows' ids
+  int* bq = active + ntiles;  // 16 ints: per-wave (min,max) of the query rows' ids, then of their positions
   int nact = ntiles;
   int wqmin = 0, wqmax = 0;
   if (SEG) {
@@ -105,17 +133,24 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
     }
     wqmin = __builtin_amdgcn_readfirstlane(wqmin);
     wqmax = __builtin_amdgcn_readfirstlane(wqmax);
-    if (lane == 0) { bq[2 * wave] = wqmin; bq[2 * wave + 1] = wqmax; }
+    if (lane == 0) { bq[2 * wave] = wqmin; bq[2 * wave + 1] = wqmax; bq[8 + 2 * wave] = wpmin; bq[9 + 2 * wave] = wpmax; }
     static_assert(BN == 64, "seg_tile_ranges works on 64-row tiles");
-    seg_tile_ranges(segb, Skv, 0, ntiles, kvmin, kvmax, tid, 256);
+    if (has_seg) {
+      seg_tile_ranges(segb, Skv, 0, ntiles, kvmin, kvmax, tid, 256);
+    } else {
+      for (int t = tid; t < ntiles; t += 256) { kvmin[t] = 0; kvmax[t] = 0; }
+    }
     __syncthreads();
     const int bqmin = min(min(bq[0], bq[2]), min(bq[4], bq[6]));
     const int bqmax = max(max(bq[1], bq[3]), max(bq[5], bq[7]));
+    // keys any row of the workgroup may see
+    const int b_lo = ext ? min(min(bq[8], bq[10]), min(bq[12], bq[14])) - a.mx.lo_off : -BAND_INF;
+    const int b_hi = ext ? max(max(bq[9], bq[11]), max(bq[13], bq[15])) + a.mx.hi_off : BAND_INF;
     // every wave builds the same list redundantly (no second barrier needed for the count)
     int cnt = 0;
     for (int base = 0; base < ntiles; base += 64) {
       const int t = base + lane;
-      const bool act = t < ntiles && !(kvmax[t] < bqmin || kvmin[t] > bqmax);
+      const bool act = t < ntiles && !(kvmax[t] < bqmin || kvmin[t] > bqmax) && t * BN <= b_hi && t * BN + BN - 1 >= b_lo;
       const unsigned long long m = __ballot(act);
       if (act && wave == 0) active[cnt + __popcll(m & ((1ull << lane) - 1ull))] = t;
       cnt += __popcll(m);
@@ -158,7 +193,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
         for (int ii = 0; ii < 4; ii++) vreg[i][ii] = buf_load16(vrs, vvo[i][ii], vso);
       }
     }
-    if (SEG && tid < BN) sreg = segb[min(t * BN + tid, Skv - 1)];
+    if (has_seg && tid < BN) sreg = segb[min(t * BN + tid, Skv - 1)];
   };
   // the same loads one at a time (piece P of K_ITEMS + 4 V_ITEMS), for issuing between MFMAs
   auto load_piece = [&](auto Pc, int t) {
@@ -272,7 +307,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
       for (int v = 0; v < 16; v++) {
         const int kvl = hf * 32 + 8 * (v / 4) + 4 * g + (v % 4);
         const int kv = kv0 + kvl;
-        const bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
+        bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
+        if (GEN) {
+          ok = ok && kv >= lo_q && kv <= hi_q;
+          // soft cap on the raw score, rescaled so that the common scale c still applies afterwards
+          if (capped) s[v] = a.mx.cap_out * fast_tanh(s[v] * a.mx.cap_in);
+        }
         s[v] = ok ? s[v] : -INFINITY;
       }
     };
@@ -339,7 +379,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
       // the next tile's loads, one per slot (past the last tile they re-read the last one: no branch here)
       if constexpr (i < K_ITEMS + 4 * V_ITEMS) load_piece(I, t_next);
       if constexpr (i == 0) {
-        if (SEG && tid < BN) sreg = segb[min(t_next * BN + tid, Skv - 1)];
+        if (has_seg && tid < BN) sreg = segb[min(t_next * BN + tid, Skv - 1)];
       }
       // one slot after the last MFMA of a half: mask, running max (the rare rescale of O is a wave-uniform
       // branch), then the exponentials under the following MFMAs
@@ -432,6 +472,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const FwdArgs a) {
         skip = skip || hi < wqmin || lo > wqmax;
         need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
       }
+      if (ext) {
+        // outside every row's band: nothing to do; not inside every row's band (or a soft cap): element-wise path
+        skip = skip || kv0 > wpmax + a.mx.hi_off || kv0 + BN - 1 < wpmin - a.mx.lo_off;
+        need_mask = need_mask || capped || !(kv0 >= wpmax - a.mx.lo_off && kv0 + BN - 1 <= wpmin + a.mx.hi_off);
+      }
       typedef std::integral_constant<int, -1> RT;
       if (skip) {
         if (has_next) {
@@ -476,7 +521,7 @@ static int launch_fwd(const FwdArgs& a, int B, hipStream_t st) {
   constexpr int BN = 64, BM = 128;
   constexpr int BUF = BN * RowTile<DQK>::STRIDE + DV * TrTile64::ROW_BYTES + (SEG ? BN * 4 : 0);
   const int ntiles_max = (a.Skv + BN - 1) / BN;
-  const size_t smem = 2 * (size_t)BUF + (SEG ? (size_t)(3 * ntiles_max + 8) * 4 : 0);
+  const size_t smem = 2 * (size_t)BUF + (SEG ? (size_t)(3 * ntiles_max + 16) * 4 : 0);
   TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_fwd: Skv=%d needs %zu bytes of LDS (max 163840)", a.Skv, smem);
   auto kern = attn_fwd_kernel<T, DQK, DV, CAUSAL, SEG>;
   static bool attr_set = false;  // benign race: every thread sets the same value
@@ -492,6 +537,11 @@ static int launch_fwd(const FwdArgs& a, int B, hipStream_t st) {
 
 template <typename T, int DQK, int DV>
 static int dispatch_fwd(const FwdArgs& a, int B, int causal, hipStream_t st) {
+  if (a.mx.on) {
+    // mask extensions: the general instantiation (causality is part of the band then)
+    if constexpr (DQK == DV && DQK <= 128) return launch_fwd<T, DQK, DV, false, true>(a, B, st);
+    else TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_attn_fwd_masked: windows, soft cap and query positions are built for head dims 64 and 128");
+  }
   if (causal) {
     if (a.seg) return launch_fwd<T, DQK, DV, true, true>(a, B, st);
     return launch_fwd<T, DQK, DV, true, false>(a, B, st);
@@ -509,16 +559,17 @@ int attn_fwd_f32(const void* q, const void* k, const void* v, const int32_t* seg
 
 using namespace tp;
 
-extern "C" int tp_attn_fwd(const void* q, const void* k, const void* v, const int32_t* seg, void* out, float* lse,
-                           int B, int Hq, int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t q_strides[3],
-                           const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
-                           float sm_scale, int causal, int dtype, void* stream) {
+static int attn_fwd_impl(const void* q, const void* k, const void* v, const int32_t* seg, void* out, float* lse,
+                         int B, int Hq, int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t q_strides[3],
+                         const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
+                         float sm_scale, int causal, int dtype, void* stream, const MaskExt& mx) {
   TP_REQUIRE(q && k && v && out && lse && q_strides && k_strides && v_strides && o_strides, TP_ERR_BAD_ARG,
              "tp_attn_fwd: null pointer");
   TP_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Sq > 0 && Skv > 0, TP_ERR_BAD_ARG, "tp_attn_fwd: non-positive size");
   TP_REQUIRE(Hq % Hkv == 0, TP_ERR_BAD_ARG, "tp_attn_fwd: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
   TP_REQUIRE(!seg || Sq == Skv, TP_ERR_BAD_ARG, "tp_attn_fwd: segment ids need Sq == Skv (got %d, %d)", Sq, Skv);
   TP_REQUIRE(sm_scale > 0.f, TP_ERR_BAD_ARG, "tp_attn_fwd: sm_scale must be positive");
+  TP_REQUIRE(!mx.on || dtype != TP_F32, TP_ERR_UNSUPPORTED, "tp_attn_fwd_masked: windows, soft cap and query positions need 16-bit tensors");
   if (dtype == TP_F32)
     return attn_fwd_f32(q, k, v, seg, out, lse, B, Hq, Hkv, Sq, Skv, Dqk, Dv, q_strides, k_strides, v_strides, o_strides, sm_scale,
                         causal, (hipStream_t)stream);
@@ -538,6 +589,7 @@ extern "C" int tp_attn_fwd(const void* q, const void* k, const void* v, const in
   TP_REQUIRE(((int64_t)Skv * k_strides[2] + Dqk) * 2 < (1ll << 31) && ((int64_t)Skv * v_strides[2] + Dv) * 2 < (1ll << 31),
              TP_ERR_UNSUPPORTED, "tp_attn_fwd: one (batch, head) slice of k or v spans 2 GiB or more");
   a.scale_log2 = sm_scale * LOG2E;
+  a.mx = mx;
   hipStream_t st = (hipStream_t)stream;
 #define TP_FWD(T, DQ, DVV) return dispatch_fwd<T, DQ, DVV>(a, B, causal, st)
   if (dtype == TP_BF16) {
@@ -551,4 +603,25 @@ extern "C" int tp_attn_fwd(const void* q, const void* k, const void* v, const in
   }
 #undef TP_FWD
   TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_attn_fwd: head dims (qk=%d, v=%d) not built", Dqk, Dv);
+}
+
+extern "C" int tp_attn_fwd(const void* q, const void* k, const void* v, const int32_t* seg, void* out, float* lse,
+                           int B, int Hq, int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t q_strides[3],
+                           const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
+                           float sm_scale, int causal, int dtype, void* stream) {
+  return attn_fwd_impl(q, k, v, seg, out, lse, B, Hq, Hkv, Sq, Skv, Dqk, Dv, q_strides, k_strides, v_strides, o_strides, sm_scale,
+                       causal, dtype, stream, no_mask_ext());
+}
+
+extern "C" int tp_attn_fwd_masked(const void* q, const void* k, const void* v, const int32_t* seg, const int32_t* q_positions,
+                                  void* out, float* lse, int B, int Hq, int Hkv, int Sq, int Skv, int Dqk, int Dv,
+                                  const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                                  const int64_t o_strides[3], float sm_scale, int causal, int causal_offset, int window_left,
+                                  int window_right, float logits_soft_cap, int dtype, void* stream) {
+  TP_REQUIRE(sm_scale > 0.f, TP_ERR_BAD_ARG, "tp_attn_fwd_masked: sm_scale must be positive");
+  TP_REQUIRE(window_left < BAND_INF && window_right < BAND_INF && causal_offset > -BAND_INF && causal_offset < BAND_INF, TP_ERR_BAD_ARG,
+             "tp_attn_fwd_masked: window or offset out of range");
+  return attn_fwd_impl(q, k, v, seg, out, lse, B, Hq, Hkv, Sq, Skv, Dqk, Dv, q_strides, k_strides, v_strides, o_strides, sm_scale,
+                       causal, dtype, stream,
+                       make_mask_ext(q_positions, causal, causal_offset, window_left, window_right, logits_soft_cap, sm_scale));
 }

@@ -12,6 +12,21 @@ from dataclasses import asdict, dataclass, field
 import torch
 
 from . import ops
+from .parallelism_utils import LoadBalancedCausalMask
+
+# q_sequence arrays as device tensors, one per (mask, device): the mask object is rebuilt every layer call
+# (attention.py:92-96) but equal masks hash equal
+_QSEQ_CACHE: dict = {}
+
+
+def _q_positions(mask: LoadBalancedCausalMask, device) -> torch.Tensor:
+  key = (mask, str(device))
+  t = _QSEQ_CACHE.get(key)
+  if t is None:
+    if len(_QSEQ_CACHE) > 16:
+      _QSEQ_CACHE.clear()
+    t = _QSEQ_CACHE[key] = torch.from_numpy(mask.q_sequence.astype("int32")).to(device)
+  return t
 
 
 @dataclass
@@ -55,16 +70,23 @@ def splash_attention_jax_wrapper(
   """Mask composition of kernel_utils.py:215-220, 238-241, 259-278: (causal | full) AND same-segment.
   ``query`` is expected pre-scaled like the reference's callers do (attention.py:107), so
   ``sm_scale=None`` means 1.0."""
+  q_positions, causal_offset = None, 0
   if mask is not None:
-    raise NotImplementedError("custom mask objects are not supported; use causal= and decoder_segment_ids=")
-  if attn_logits_soft_cap is not None:
-    raise NotImplementedError("attn_logits_soft_cap is not supported")
+    # the one custom mask the reference builds (attention.py:92-96); it replaces the causal / full choice
+    # (kernel_utils.py:259-263 only builds one when mask is None)
+    if not isinstance(mask, LoadBalancedCausalMask):
+      raise NotImplementedError(f"mask objects of type {type(mask).__name__} are not supported (LoadBalancedCausalMask is)")
+    if tuple(mask.shape) != (query.shape[2], key.shape[2]):
+      raise ValueError(f"mask shape {tuple(mask.shape)} does not match (q_len, kv_len) = {(query.shape[2], key.shape[2])}")
+    q_positions, causal_offset, causal = _q_positions(mask, query.device), int(mask.offset), True
   if isinstance(config, str):
     config = SplashAttentionConfig.from_json(config)
+  window = None
   if config is not None and getattr(config, "attentiontype_local_sliding", False):
     if getattr(config, "slide_window_size", None) is None:
       raise ValueError("Sliding_window_size must be set if Local Sliding attention type")
-    raise NotImplementedError("local sliding-window attention is not supported")
+    # LocalMask(window_size=(w, w), offset=0) ANDed into the mask (kernel_utils.py:266-275)
+    window = (int(config.slide_window_size), int(config.slide_window_size))
   if decoder_segment_ids is not None and not tuple(decoder_segment_ids.shape):
     decoder_segment_ids = None
   if decoder_segment_ids is not None:
@@ -72,7 +94,8 @@ def splash_attention_jax_wrapper(
       "Sharding along sequence dimension not allowed in tpu kernel attention"
     )
   return ops.attention(
-    query, key, value, decoder_segment_ids, 1.0 if sm_scale is None else float(sm_scale), bool(causal)
+    query, key, value, decoder_segment_ids, 1.0 if sm_scale is None else float(sm_scale), bool(causal),
+    window=window, soft_cap=attn_logits_soft_cap, q_positions=q_positions, causal_offset=causal_offset,
   )
 
 

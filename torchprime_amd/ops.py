@@ -384,17 +384,122 @@ def _attn_backward(ctx, dout, _dlse):
 attn_fwd.register_autograd(_attn_backward, setup_context=_attn_setup)
 
 
+# ---- mask extensions: sliding window, soft cap, query rows in another order than the keys -------------------
+def _prep_qpos(qpos: Tensor | None, Sq: int) -> Tensor | None:
+  if qpos is None:
+    return None
+  if qpos.shape != (Sq,):
+    raise ValueError(f"q_positions must have shape ({Sq},), got {tuple(qpos.shape)}")
+  return qpos.to(torch.int32).contiguous()
+
+
+@torch.library.custom_op("tprime::attn_fwd_masked", mutates_args=(), device_types="cuda")
+def attn_fwd_masked(
+  q: Tensor, k: Tensor, v: Tensor, seg: Tensor | None, qpos: Tensor | None, sm_scale: float, causal: bool,
+  causal_offset: int, window_left: int, window_right: int, soft_cap: float,
+) -> tuple[Tensor, Tensor]:  # fmt: skip
+  dev = _lib.require_gpu(q, k, v, seg, qpos)
+  B, Hq, Hkv, Sq, Skv, Dqk, Dv = _check_attn(q, k, v, seg)
+  q, k, v = _prep_heads(q), _prep_heads(k), _prep_heads(v)
+  if seg is not None:
+    seg = seg.to(torch.int32).contiguous()
+  qpos = _prep_qpos(qpos, Sq)
+  out = _empty_like_heads(q, Dv)
+  lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=dev)
+  if out.numel():
+    _lib.call(
+      "tp_attn_fwd_masked", q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.ptr(seg), _lib.ptr(qpos), out.data_ptr(),
+      lse.data_ptr(), B, Hq, Hkv, Sq, Skv, Dqk, Dv, _lib.strides3(q), _lib.strides3(k), _lib.strides3(v),
+      _lib.strides3(out), float(sm_scale), int(causal), int(causal_offset), int(window_left), int(window_right),
+      float(soft_cap), _lib.dtype_code(q.dtype), _lib.stream_ptr(dev),
+    )  # fmt: skip
+  return out, lse
+
+
+@attn_fwd_masked.register_fake
+def _(q, k, v, seg, qpos, sm_scale, causal, causal_offset, window_left, window_right, soft_cap):
+  B, Hq, Sq, _ = q.shape
+  return _empty_like_heads(q, v.shape[-1]), q.new_empty((B, Hq, Sq), dtype=torch.float32)
+
+
+@torch.library.custom_op("tprime::attn_bwd_masked", mutates_args=(), device_types="cuda")
+def attn_bwd_masked(
+  dout: Tensor, q: Tensor, k: Tensor, v: Tensor, out: Tensor, lse: Tensor, seg: Tensor | None, qpos: Tensor | None,
+  sm_scale: float, causal: bool, causal_offset: int, window_left: int, window_right: int, soft_cap: float,
+) -> tuple[Tensor, Tensor, Tensor]:  # fmt: skip
+  dev = _lib.require_gpu(dout, q, k, v, out, lse, seg, qpos)
+  if q.dtype == torch.float32:
+    raise NotImplementedError("fp32 attention is forward-only; run the backward in bfloat16 or float16")
+  B, Hq, Hkv, Sq, Skv, Dqk, Dv = _check_attn(q, k, v, seg)
+  q, k, v, out, dout = _prep_heads(q), _prep_heads(k), _prep_heads(v), _prep_heads(out), _prep_heads(dout)
+  lse = lse.contiguous()
+  if seg is not None:
+    seg = seg.to(torch.int32).contiguous()
+  qpos = _prep_qpos(qpos, Sq)
+  dq, dk, dv = _empty_like_heads(q), _empty_like_heads(k), _empty_like_heads(v)
+  if dq.numel() == 0 or dk.numel() == 0:
+    return dq.zero_(), dk.zero_(), dv.zero_()
+  lib = _lib.load()
+  ws = torch.empty((lib.tp_attn_bwd_workspace_bytes(B, Hq, Sq) // 4,), dtype=torch.float32, device=dev)
+  _lib.call(
+    "tp_attn_bwd_masked", dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+    _lib.ptr(seg), _lib.ptr(qpos), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), B, Hq, Hkv, Sq, Skv,
+    Dqk, Dv, _lib.strides3(dout), _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
+    _lib.strides3(dq), _lib.strides3(dk), _lib.strides3(dv), float(sm_scale), int(causal), int(causal_offset),
+    int(window_left), int(window_right), float(soft_cap), _lib.dtype_code(q.dtype), _lib.stream_ptr(dev),
+  )  # fmt: skip
+  return dq, dk, dv
+
+
+@attn_bwd_masked.register_fake
+def _(dout, q, k, v, out, lse, seg, qpos, sm_scale, causal, causal_offset, window_left, window_right, soft_cap):
+  return _empty_like_heads(q), _empty_like_heads(k), _empty_like_heads(v)
+
+
+def _attn_masked_setup(ctx, inputs, output):
+  q, k, v, seg, qpos, sm_scale, causal, causal_offset, window_left, window_right, soft_cap = inputs
+  out, lse = output
+  ctx.save_for_backward(*(t for t in (q, k, v, out, lse, seg, qpos) if t is not None))
+  ctx.has_seg, ctx.has_qpos = seg is not None, qpos is not None
+  ctx.scalars = (sm_scale, causal, causal_offset, window_left, window_right, soft_cap)
+
+
+def _attn_masked_backward(ctx, dout, _dlse):
+  saved = list(ctx.saved_tensors)
+  q, k, v, out, lse = saved[:5]
+  rest = saved[5:]
+  seg = rest.pop(0) if ctx.has_seg else None
+  qpos = rest.pop(0) if ctx.has_qpos else None
+  dq, dk, dv = attn_bwd_masked(dout, q, k, v, out, lse, seg, qpos, *ctx.scalars)
+  return (dq, dk, dv) + (None,) * 8
+
+
+attn_fwd_masked.register_autograd(_attn_masked_backward, setup_context=_attn_masked_setup)
+
+
 def attention(
-  q: Tensor, k: Tensor, v: Tensor, segment_ids: Tensor | None = None, sm_scale: float | None = None, causal: bool = True
-) -> Tensor:
+  q: Tensor, k: Tensor, v: Tensor, segment_ids: Tensor | None = None, sm_scale: float | None = None, causal: bool = True,
+  *, window: tuple[int | None, int | None] | None = None, soft_cap: float | None = None,
+  q_positions: Tensor | None = None, causal_offset: int = 0,
+) -> Tensor:  # fmt: skip
   """Causal / segment-masked GQA attention: q (B,Hq,S,Dqk), k (B,Hkv,S,Dqk), v (B,Hkv,S,Dv) -> (B,Hq,S,Dv).
 
   ``sm_scale=None`` means ``1/sqrt(v.shape[-1])``, the scale AttentionModule uses
-  (torchprime/torch_xla_models/attention.py:54-58, 107, 143, 154)."""
-  _lib.require_gpu(q, k, v, segment_ids)
+  (torchprime/torch_xla_models/attention.py:54-58, 107, 143, 154).
+
+  ``window=(left, right)``: key j only if ``pos - left <= j <= pos + right`` (None: unbounded; LocalMask,
+  kernel_utils.py:266-275).  ``soft_cap``: logits become ``cap * tanh(logits / cap)`` (kernel_utils.py:292).
+  ``q_positions`` (Sq) int: query row i stands for position ``q_positions[i]`` of the key order
+  (LoadBalancedCausalMask.q_sequence, parallelism_utils.py:109-132); ``causal_offset``: that mask's ``offset``."""
+  if soft_cap is not None and soft_cap <= 0:
+    raise ValueError(f"soft_cap must be positive, got {soft_cap}")
+  _lib.require_gpu(q, k, v, segment_ids, q_positions)
   if sm_scale is None:
     sm_scale = 1.0 / math.sqrt(v.shape[-1])
-  return attn_fwd(q, k, v, segment_ids, sm_scale, causal)[0]
+  wl, wr = (-1, -1) if window is None else tuple(-1 if w is None else int(w) for w in window)
+  if q_positions is None and wl < 0 and wr < 0 and soft_cap is None and (causal_offset == 0 or not causal):
+    return attn_fwd(q, k, v, segment_ids, sm_scale, causal)[0]
+  return attn_fwd_masked(q, k, v, segment_ids, q_positions, sm_scale, causal, causal_offset, wl, wr, float(soft_cap or 0.0))[0]
 
 
 # ------------------------------------------------------------------------------------------------
