@@ -814,18 +814,20 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       if (it + 1 < n_iter) iteration(std::integral_constant<int, 1>{}, it + 1);
     }
   } else {
-    // Wide heads: one buffer, and the register file does not hold the staggered schedule: the next tile is
-    // requested once this one has been used, both query blocks go through each step together.
-    int c_hl = 0, c_idx = 0;
-    auto stage = [&](int hl, int idx) {
-      issue_tile(hl, idx, 0, 0);
+    // Wide heads: one buffer of each kind, and the register file does not hold the staggered schedule: both query
+    // blocks go through each step together.  The row-major tiles are free once S and dP are done, so the next
+    // tile's loads are issued there and travel under the element-wise work and the dV / dK products, which read the
+    // transposed copies; the next tile is transposed once those are done.  Row vectors alternate two slots.
+    int c_hl = 0, c_idx = 0, n_hl = 0, n_idx = 0;
+    if (n_iter > 0) {
+      issue_tile(0, 0, 0, 0);
+      advance(n_hl, n_idx);
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
       transpose_tile<DQK>(smem + Q_AT, smem + QTR_AT, tid);
       transpose_tile<DV>(smem + DO_AT, smem + DOTR_AT, tid);
       __syncthreads();
-    };
-    if (n_iter > 0) stage(0, 0);
+    }
     for (int it = 0; it < n_iter; it++) {
       const int qi0 = qtile_of(c_idx) * BMQ;
       const int mode = tile_mode(c_idx, qi0);
@@ -834,12 +836,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       const unsigned char* dol = smem + DO_AT;
       const unsigned char* qtl = smem + QTR_AT;
       const unsigned char* dotl = smem + DOTR_AT;
-      const float* lsel = (const float*)rows_base;
+      const float* lsel = (const float*)(rows_base + (it & 1) * ROW_BYTES);
       const float* deltal = lsel + BMQ;
       const int* segl = (const int*)(deltal + BMQ);
       constexpr int QB = BMQ / 32;
+      f32x16 sacc[QB], dpacc[QB];
       if (mode != 0) {
-        f32x16 sacc[QB], dpacc[QB];
 #pragma unroll
         for (int qb = 0; qb < QB; qb++)
 #pragma unroll
@@ -860,6 +862,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
             const v8 dof = *(const v8*)(dol + fao[ks] + qb * 32 * OT::ROWB);
             dpacc[qb] = MT<T>::mfma32(dof, vf[ks], dpacc[qb]);
           }
+      }
+      __syncthreads();  // everyone is done with the row-major tiles
+      if (it + 1 < n_iter) {
+        issue_tile(n_hl, n_idx, 0, (it + 1) & 1);
+        advance(n_hl, n_idx);
+      }
+      if (mode != 0) {
         // P = exp2(S*c - lse), dS = P o (dP - delta); rows of the C tile are queries
         v8 pfr[BMQ / 16], dsf[BMQ / 16];
         const int kvcol = wkv0 + ln;
@@ -906,18 +915,23 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
 #pragma unroll
           for (int d = 0; d < DVB; d++) {
             const v8 f = *(const v8*)(dotl + ta[ks ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
-            dvacc[d] = MT<T>::mfma32(f, pfr[ks], dvacc[d]);
+            MT<T>::mfma32_acc_guarded(dvacc[d], f, pfr[ks]);  // accumulators pinned to the accumulation registers, as in the pipelined path
           }
 #pragma unroll
           for (int d = 0; d < DKB; d++) {
             const v8 f = *(const v8*)(qtl + ta[ks ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
-            dkacc[d] = MT<T>::mfma32(f, dsf[ks], dkacc[d]);
+            MT<T>::mfma32_acc_guarded(dkacc[d], f, dsf[ks]);
           }
         }
       }
-      __syncthreads();  // everyone is done with the tile
+      __builtin_amdgcn_s_waitcnt(0);
+      __syncthreads();  // the next tile has landed; everyone is done with the transposed tiles
       advance(c_hl, c_idx);
-      if (it + 1 < n_iter) stage(c_hl, c_idx);
+      if (it + 1 < n_iter) {
+        transpose_tile<DQK>(smem + Q_AT, smem + QTR_AT, tid);
+        transpose_tile<DV>(smem + DO_AT, smem + DOTR_AT, tid);
+      }
+      __syncthreads();
     }
   }
 

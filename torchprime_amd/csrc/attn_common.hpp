@@ -38,6 +38,9 @@ template <> struct MT<bf16_t> {
   static __device__ __forceinline__ void mfma32_acc(f32x16& c, v8 a, v8 b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
+  static __device__ __forceinline__ void mfma32_acc_guarded(f32x16& c, v8 a, v8 b) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
 };
 template <> struct MT<f16_t> {
   typedef f16x8 v8;
@@ -48,6 +51,9 @@ template <> struct MT<f16_t> {
   static __device__ __forceinline__ void mfma32_acc(f32x16& c, v8 a, v8 b) {
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
+  static __device__ __forceinline__ void mfma32_acc_guarded(f32x16& c, v8 a, v8 b) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
 };
 // mfma32_acc: long-lived accumulators that only MFMAs touch inside a loop (dK, dV) are kept in the
 // accumulation half of the register file by writing the instruction out with an "a" constraint.  With the
@@ -56,6 +62,10 @@ template <> struct MT<f16_t> {
 // What the compiler no longer sees, and the callers guarantee: the same accumulator is reused by a later
 // mfma32_acc only (exactly overlapping destination, for which the matrix unit forwards), and it is read
 // by ordinary instructions only after the loop and a barrier, hundreds of cycles after the last MFMA.
+// One more thing the compiler does for its own MFMAs and not for these: an A/B operand register written by a
+// vector-ALU instruction needs two wait states before a matrix instruction reads it (the packed P / dS operands
+// are such registers).  mfma32_acc leaves that distance to the caller's hand-placed schedule;
+// mfma32_acc_guarded carries the two wait states itself, for code whose order is left to the compiler.
 
 // eight floats -> one 16-byte MFMA operand (round to nearest even)
 template <typename T>
