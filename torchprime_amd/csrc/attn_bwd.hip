@@ -840,28 +840,30 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       const float* deltal = lsel + BMQ;
       const int* segl = (const int*)(deltal + BMQ);
       constexpr int QB = BMQ / 32;
+      constexpr int RING = 4;  // fragments in flight: four MFMAs (128 cycles) cover an LDS read
       f32x16 sacc[QB], dpacc[QB];
       if (mode != 0) {
 #pragma unroll
         for (int qb = 0; qb < QB; qb++)
 #pragma unroll
           for (int v = 0; v < 16; v++) { sacc[qb][v] = 0.f; dpacc[qb][v] = 0.f; }
-        // S = Q K^T  (rows = queries, columns = this wave's kv rows)
+        // S = Q K^T (rows = queries, columns = this wave's kv rows), then dP = dO V^T: one sequence of MFMAs whose
+        // A fragments are requested RING steps ahead, so that an LDS round trip is not paid in front of every one
+        constexpr int NS = KS_QK * QB, NA = NS + KS_DV * QB;
+        auto a_frag = [&](int i) {
+          if (i < NS) return *(const v8*)(ql + faq[i / QB] + (i % QB) * 32 * QT::ROWB);
+          return *(const v8*)(dol + fao[(i - NS) / QB] + ((i - NS) % QB) * 32 * OT::ROWB);
+        };
+        v8 ring[RING];
 #pragma unroll
-        for (int ks = 0; ks < KS_QK; ks++)
+        for (int r = 0; r < RING; r++) ring[r] = a_frag(r);
 #pragma unroll
-          for (int qb = 0; qb < QB; qb++) {
-            const v8 qf = *(const v8*)(ql + faq[ks] + qb * 32 * QT::ROWB);
-            sacc[qb] = MT<T>::mfma32(qf, kf[ks], sacc[qb]);
-          }
-        // dP = dO V^T
-#pragma unroll
-        for (int ks = 0; ks < KS_DV; ks++)
-#pragma unroll
-          for (int qb = 0; qb < QB; qb++) {
-            const v8 dof = *(const v8*)(dol + fao[ks] + qb * 32 * OT::ROWB);
-            dpacc[qb] = MT<T>::mfma32(dof, vf[ks], dpacc[qb]);
-          }
+        for (int i = 0; i < NA; i++) {
+          if (i < NS) sacc[i % QB] = MT<T>::mfma32(ring[i % RING], kf[i / QB], sacc[i % QB]);
+          else dpacc[(i - NS) % QB] = MT<T>::mfma32(ring[i % RING], vf[(i - NS) / QB], dpacc[(i - NS) % QB]);
+          if (i + RING < NA) ring[i % RING] = a_frag(i + RING);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
       __syncthreads();  // everyone is done with the row-major tiles
       if (it + 1 < n_iter) {
@@ -909,19 +911,25 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
                                         d[8 * hh + 5], d[8 * hh + 6], d[8 * hh + 7]);
           }
         }
-        // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 64 query rows)
+        // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 64 query rows), fragments requested ahead as
+        // above; the accumulators are pinned to the accumulation registers, as in the pipelined path
+        constexpr int PER_KS = DVB + DKB, NB = (BMQ / 16) * PER_KS;
+        auto t_frag = [&](int i) {
+          const int ks = i / PER_KS, d = i % PER_KS;
+          if (d < DVB) return *(const v8*)(dotl + ta[ks ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+          return *(const v8*)(qtl + ta[ks ^ ((d - DVB) & 3)] + (d - DVB) * 32 * TrTile64::ROW_BYTES);
+        };
+        v8 ring[RING];
 #pragma unroll
-        for (int ks = 0; ks < BMQ / 16; ks++) {
+        for (int r = 0; r < RING; r++) ring[r] = t_frag(r);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int d = 0; d < DVB; d++) {
-            const v8 f = *(const v8*)(dotl + ta[ks ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
-            MT<T>::mfma32_acc_guarded(dvacc[d], f, pfr[ks]);  // accumulators pinned to the accumulation registers, as in the pipelined path
-          }
-#pragma unroll
-          for (int d = 0; d < DKB; d++) {
-            const v8 f = *(const v8*)(qtl + ta[ks ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
-            MT<T>::mfma32_acc_guarded(dkacc[d], f, dsf[ks]);
-          }
+        for (int i = 0; i < NB; i++) {
+          const int ks = i / PER_KS, d = i % PER_KS;
+          if (d < DVB) MT<T>::mfma32_acc_guarded(dvacc[d], ring[i % RING], pfr[ks]);
+          else MT<T>::mfma32_acc_guarded(dkacc[d - DVB], ring[i % RING], dsf[ks]);
+          if (i + RING < NB) ring[i % RING] = t_frag(i + RING);
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
       __builtin_amdgcn_s_waitcnt(0);
