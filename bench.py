@@ -319,7 +319,7 @@ def packed_segment_ids(B, S, lo, hi, seed):
   return seg, lengths
 
 
-def bench_other_configs(dev, iters=5):
+def bench_other_configs(dev, iters=5, only=None):
   """The other benchmark configurations, forward + backward through the C ABI, inputs resident: packed documents
   (configuration 3), the Llama-3-70B layer (4) and the DeepSeek-V3 head dims (5).  FLOPs are counted like the
   headline: 3 x 2 * Hq * (dqk + dv) * (allowed query/key pairs)."""
@@ -334,7 +334,13 @@ def bench_other_configs(dev, iters=5):
     ("llama3_70b_layer", 1, 64, 8, 8192, 128, 128, False),
     ("deepseek_v3_heads", 1, 128, 128, 4096, 192, 128, False),
   ]
+  if only is not None:
+    unknown = [n for n in only if n not in [c[0] for c in cases]]
+    if unknown:
+      sys.exit(f"bench.py: unknown configuration(s) {unknown}")
   for name, B, Hq, Hkv, S, Dqk, Dv, packed in cases:
+    if only is not None and name not in only:
+      continue
     g = torch.Generator(device="cpu").manual_seed(1236)
 
     def mk(h, d):
@@ -447,6 +453,9 @@ def main():
   ap.add_argument("--no-extra", action="store_true", help="skip the RMSNorm / RoPE bandwidth leg")
   ap.add_argument("--calib-copy", action="store_true",
                   help="also run one 256 MiB device copy (the known-size kernel the HBM counters are scaled by)")
+  ap.add_argument("--other-configs", default=None, metavar="NAME[,NAME]",
+                  help="run only the named other configurations (llama3_8b_packed_segments, llama3_70b_layer, "
+                       "deepseek_v3_heads, or 'all') and print their line: the command the per-configuration kernel traces use")
   args = ap.parse_args()
   if args.gpus != 1:
     sys.exit("bench.py measures the one-GPU hot path only: run with --gpus 1 (no multi-GPU path is part of this build)")
@@ -464,6 +473,10 @@ def main():
     dst.copy_(src)  # reads 256 MiB, writes 256 MiB
     torch.cuda.synchronize()
     del src, dst
+  if args.other_configs:
+    names = None if args.other_configs == "all" else args.other_configs.split(",")
+    print(json.dumps({"other_configs": bench_other_configs(dev, iters=args.steps, only=names)}))
+    return
   ms_per_step, flops_step, roofline, kernels, shape = bench_attention(args, dev)
   extra = None if args.no_extra else bench_norm_rope(dev)
   if extra is not None:
