@@ -333,6 +333,43 @@ struct TransposeSteps {
   }
 };
 
+// TransposeSteps with its state cut to six registers (store offsets are formed per store from two of them) and
+// the block's data held by the caller, for kernels that run several of these side by side; any number of
+// blocks per tile (a caller with fewer threads than blocks makes more than one round: init(tid + round * threads)).
+template <int D>
+struct TransposeLean {
+  static constexpr int CPR = D / 8, TOT = CPR * 16;
+  unsigned rd, zs, wb, y, sel_even, sel_odd;
+  __device__ __forceinline__ void init(int idx) {
+    const int item = idx % TOT, c8 = item % CPR, rqi = item / CPR;
+    const int rq = (rqi & ~3) | ((rqi & 1) << 1) | ((rqi >> 1) & 1);
+    rd = (unsigned)(4 * rq * DmaTile<D>::ROWB);
+    zs = (unsigned)((c8 ^ DmaTile<D>::swz(4 * rq)) << 4);
+    const int flip = c8 & 1;
+    const int k = (((c8 & 1) << 2) ^ (c8 >> 1)) & 7, rqc = 2 * (rq >> 2) + (rq & 1);
+    wb = (unsigned)(c8 * 8 * TrTile64::ROW_BYTES + (((rq >> 1) & 1) << 3));
+    y = (unsigned)((flip << 7) | ((rqc ^ k) << 4));
+    sel_even = flip ? 0x07060302u : 0x05040100u;
+    sel_odd = flip ? 0x05040100u : 0x07060302u;
+  }
+  __device__ __forceinline__ void read(const unsigned char* src, u32x4 (&r)[4]) const {
+#pragma unroll
+    for (int ii = 0; ii < 4; ii++) {
+      const unsigned sw = (unsigned)((CPR % 16 == 0 ? ii : (ii >> 1)) << 4);
+      r[ii] = *(const u32x4*)(src + rd + (zs ^ sw) + ii * DmaTile<D>::ROWB);
+    }
+  }
+  template <int J>
+  __device__ __forceinline__ void write(unsigned char* dst, const u32x4 (&r)[4]) const {
+    constexpr int w = J >> 1;
+    const unsigned sel = (J & 1) ? sel_odd : sel_even;
+    u32x2 o;
+    o.x = __builtin_amdgcn_perm(r[1][w], r[0][w], sel);
+    o.y = __builtin_amdgcn_perm(r[3][w], r[2][w], sel);
+    *(u32x2*)(dst + wb + (y ^ (unsigned)(((J & 1) << 7) | ((J >> 1) << 4))) + (J >> 1) * 2 * TrTile64::ROW_BYTES) = o;
+  }
+};
+
 // ------------------------------------------------------------------------------------------------
 // dK / dV
 // ------------------------------------------------------------------------------------------------
@@ -814,24 +851,38 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       if (it + 1 < n_iter) iteration(std::integral_constant<int, 1>{}, it + 1);
     }
   } else {
-    // Wide heads: one buffer of each kind, and the register file does not hold the staggered schedule: both query
-    // blocks go through each step together.  The row-major tiles are free once S and dP are done, so the next
-    // tile's loads are issued there and travel under the element-wise work and the dV / dK products, which read the
-    // transposed copies; the next tile is transposed once those are done.  Row vectors alternate two slots.
+    // Wide heads: one buffer of each kind; both query blocks go through each step together.  Per tile:
+    //   part 1  S = Q K^T, dP = dO V^T from the row-major tiles; between the S MFMAs the same tile is copied into
+    //           its transposed form (that copy only reads the row-major tiles, and nobody reads the transposed
+    //           ones before the barrier); between the dP MFMAs P = exp2(S c - LSE) is computed and packed
+    //   barrier  row-major tiles free, transposed tiles complete; the next tile's loads are issued into the former
+    //   part 2  dV^T += dO^T P with dS = P o (dP - delta) computed between its MFMAs, then dK^T += Q^T dS
+    //   wait for the loads, barrier
+    // Every MFMA's LDS fragment is requested RING MFMAs ahead; row vectors alternate two slots.
+    constexpr int QB = BMQ / 32, RING = 4;
+    constexpr int NS = KS_QK * QB, NA = NS + KS_DV * QB;          // part 1: S steps, then dP steps
+    constexpr int NV = (BMQ / 16) * DVB, NB = NV + (BMQ / 16) * DKB;  // part 2: dV steps, then dK steps
+    constexpr int NCH = 16 * QB;                                  // values per lane of S (and of dP)
+    static_assert(NA - NS == NCH / 2 && NV >= NCH / 2 && NS >= 18, "two values per step under dP and under dV");
+    TransposeLean<DQK> trq0, trq1;
+    TransposeLean<DV> tro;
+    trq0.init(tid);
+    trq1.init(tid + 256);  // 384 blocks for 256 threads: the second round of threads 128..255 repeats blocks 0..127
+    tro.init(tid);
+    static_assert(TransposeLean<DQK>::TOT <= 512 && TransposeLean<DV>::TOT <= 256, "two rounds for Q, one for dO");
+    unsigned char* const qtw = smem + QTR_AT;
+    unsigned char* const dotw = smem + DOTR_AT;
+    const int kvcol = wkv0 + ln;
     int c_hl = 0, c_idx = 0, n_hl = 0, n_idx = 0;
     if (n_iter > 0) {
       issue_tile(0, 0, 0, 0);
       advance(n_hl, n_idx);
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();
-      transpose_tile<DQK>(smem + Q_AT, smem + QTR_AT, tid);
-      transpose_tile<DV>(smem + DO_AT, smem + DOTR_AT, tid);
-      __syncthreads();
     }
     for (int it = 0; it < n_iter; it++) {
       const int qi0 = qtile_of(c_idx) * BMQ;
       const int mode = tile_mode(c_idx, qi0);
-      const bool need_mask = mode == 2;
       const unsigned char* ql = smem + Q_AT;
       const unsigned char* dol = smem + DO_AT;
       const unsigned char* qtl = smem + QTR_AT;
@@ -839,107 +890,138 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       const float* lsel = (const float*)(rows_base + (it & 1) * ROW_BYTES);
       const float* deltal = lsel + BMQ;
       const int* segl = (const int*)(deltal + BMQ);
-      constexpr int QB = BMQ / 32;
-      constexpr int RING = 4;  // fragments in flight: four MFMAs (128 cycles) cover an LDS read
       f32x16 sacc[QB], dpacc[QB];
-      if (mode != 0) {
-#pragma unroll
-        for (int qb = 0; qb < QB; qb++)
-#pragma unroll
-          for (int v = 0; v < 16; v++) { sacc[qb][v] = 0.f; dpacc[qb][v] = 0.f; }
-        // S = Q K^T (rows = queries, columns = this wave's kv rows), then dP = dO V^T: one sequence of MFMAs whose
-        // A fragments are requested RING steps ahead, so that an LDS round trip is not paid in front of every one
-        constexpr int NS = KS_QK * QB, NA = NS + KS_DV * QB;
-        auto a_frag = [&](int i) {
-          if (i < NS) return *(const v8*)(ql + faq[i / QB] + (i % QB) * 32 * QT::ROWB);
-          return *(const v8*)(dol + fao[(i - NS) / QB] + ((i - NS) % QB) * 32 * OT::ROWB);
+      v8 pfr[BMQ / 16];
+      u32x4 trd[4];
+      // transposition of this tile in 3 reads and 12 double stores, placed at steps T0.. of part 1
+      auto tr_piece = [&](auto K) {
+        constexpr int k = decltype(K)::value;  // 0..17: per block one read step, one idle step, four store steps
+        constexpr int blk = k / 6, w = k % 6;
+        if constexpr (w == 0) {
+          if constexpr (blk == 0) trq0.read(ql, trd);
+          else if constexpr (blk == 1) trq1.read(ql, trd);
+          else tro.read(dol, trd);
+        } else if constexpr (w >= 2) {
+          constexpr int j = 2 * (w - 2);
+          if constexpr (blk == 0) { trq0.template write<j>(qtw, trd); trq0.template write<j + 1>(qtw, trd); }
+          else if constexpr (blk == 1) { trq1.template write<j>(qtw, trd); trq1.template write<j + 1>(qtw, trd); }
+          else { tro.template write<j>(dotw, trd); tro.template write<j + 1>(dotw, trd); }
+        }
+      };
+      auto part1 = [&](auto masked_c) {
+        constexpr bool MASKED = decltype(masked_c)::value;
+        const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        auto a_frag = [&](auto I) {
+          constexpr int i = decltype(I)::value;
+          if constexpr (i < NS) return *(const v8*)(ql + faq[i / QB] + (i % QB) * 32 * QT::ROWB);
+          else return *(const v8*)(dol + fao[(i - NS) / QB] + ((i - NS) % QB) * 32 * OT::ROWB);
         };
         v8 ring[RING];
+        f32x4 l4[NCH / 4];
+        i32x4 sg[NCH / 4];
+        static_for<0, RING>([&](auto R) { ring[decltype(R)::value] = a_frag(R); });
+        static_for<0, NA>([&](auto I) {
+          constexpr int i = decltype(I)::value;
+          if constexpr (i < 18) tr_piece(I);
+          if constexpr (i < NS) sacc[i % QB] = MT<T>::mfma32(ring[i % RING], kf[i / QB], i < QB ? zero16 : sacc[i % QB]);
+          else dpacc[(i - NS) % QB] = MT<T>::mfma32(ring[i % RING], vf[(i - NS) / QB], i - NS < QB ? zero16 : dpacc[(i - NS) % QB]);
+          if constexpr (i + RING < NA) ring[i % RING] = a_frag(std::integral_constant<int, i + RING>{});
+          // row vector quad m is used at steps NS + 2m, NS + 2m + 1 and requested four steps before
+          if constexpr (i + 4 >= NS && (i + 4 - NS) % 2 == 0 && (i + 4 - NS) / 2 < NCH / 4) {
+            constexpr int m = (i + 4 - NS) / 2, qb = m / 4, vq = m % 4;
+            l4[m] = *(const f32x4*)(lsel + qb * 32 + 8 * vq + 4 * g);
+            if constexpr (MASKED && SEG) sg[m] = *(const i32x4*)(segl + qb * 32 + 8 * vq + 4 * g);
+          }
+          if constexpr (i >= NS) {
+            // P = exp2(S c - LSE) for two values (l4 holds -LSE in log2 units); rows of the C tile are queries
+            constexpr int k = i - NS;
 #pragma unroll
-        for (int r = 0; r < RING; r++) ring[r] = a_frag(r);
-#pragma unroll
-        for (int i = 0; i < NA; i++) {
-          if (i < NS) sacc[i % QB] = MT<T>::mfma32(ring[i % RING], kf[i / QB], sacc[i % QB]);
-          else dpacc[(i - NS) % QB] = MT<T>::mfma32(ring[i % RING], vf[(i - NS) / QB], dpacc[(i - NS) % QB]);
-          if (i + RING < NA) ring[i % RING] = a_frag(i + RING);
+            for (int idx = 2 * k; idx < 2 * k + 2; idx++) {
+              const int qb = idx / 16, v = idx % 16, m = idx / 4, e = idx % 4;
+              float pv = fast_exp2(__builtin_fmaf(sacc[qb][v], c, l4[m][e]));
+              if constexpr (MASKED) {
+                const int qrow = qi0 + qb * 32 + 8 * (v / 4) + 4 * g + e;
+                bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow);
+                if constexpr (SEG) ok = ok && sg[m][e] == segk;
+                pv = ok ? pv : 0.f;
+              }
+              asm volatile("" : "+v"(pv));  // keeps the computation in this step
+              sacc[qb][v] = pv;
+            }
+            if constexpr (k % 4 == 3) {
+              constexpr int h = k / 4, qb = h / 2, hh = h % 2;
+              const f32x16& x = sacc[qb];
+              pfr[h] = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4], x[8 * hh + 5],
+                                x[8 * hh + 6], x[8 * hh + 7]);
+            }
+          }
           __builtin_amdgcn_sched_barrier(0);
-        }
+        });
+      };
+      if (mode == 0) {
+        static_for<0, 18>([&](auto K) { tr_piece(K); });  // this wave's share of the copy, nothing to multiply
+      } else if (mode == 2) {
+        part1(std::true_type{});
+      } else {
+        part1(std::false_type{});
       }
-      __syncthreads();  // everyone is done with the row-major tiles
+      __syncthreads();  // everyone is done with the row-major tiles; the transposed ones are complete
       if (it + 1 < n_iter) {
         issue_tile(n_hl, n_idx, 0, (it + 1) & 1);
         advance(n_hl, n_idx);
       }
       if (mode != 0) {
-        // P = exp2(S*c - lse), dS = P o (dP - delta); rows of the C tile are queries
-        v8 pfr[BMQ / 16], dsf[BMQ / 16];
-        const int kvcol = wkv0 + ln;
-#pragma unroll
-        for (int qb = 0; qb < QB; qb++)
-#pragma unroll
-          for (int vq = 0; vq < 4; vq++) {
-            const f32x4 l4 = *(const f32x4*)(lsel + qb * 32 + 8 * vq + 4 * g);
-#pragma unroll
-            for (int e = 0; e < 4; e++) sacc[qb][4 * vq + e] = fast_exp2(__builtin_fmaf(sacc[qb][4 * vq + e], c, l4[e]));  // l4 = -LSE
+        // dV^T += dO^T P,  dK^T += Q^T dS  (contraction over the 64 query rows); the accumulators are pinned to the
+        // accumulation registers, as in the pipelined path
+        auto t_frag = [&](auto I) {
+          constexpr int i = decltype(I)::value;
+          if constexpr (i < NV) {
+            constexpr int ks = i / DVB, d = i % DVB;
+            return *(const v8*)(dotl + ta[ks ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+          } else {
+            constexpr int ks = (i - NV) / DKB, d = (i - NV) % DKB;
+            return *(const v8*)(qtl + ta[ks ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
           }
-        if (need_mask) {  // separate pass: the common unmasked tile carries no per-element branches
-#pragma unroll
-          for (int qb = 0; qb < QB; qb++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-              const int r = qb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
-              const int qrow = qi0 + r;
-              const bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || segl[r] == segk);
-              sacc[qb][v] = ok ? sacc[qb][v] : 0.f;
-            }
-        }
-#pragma unroll
-        for (int qb = 0; qb < QB; qb++) {
-#pragma unroll
-          for (int vq = 0; vq < 4; vq++) {
-            const f32x4 d4 = *(const f32x4*)(deltal + qb * 32 + 8 * vq + 4 * g);
-#pragma unroll
-            for (int e = 0; e < 4; e++) dpacc[qb][4 * vq + e] = sacc[qb][4 * vq + e] * (dpacc[qb][4 * vq + e] + d4[e]);
-          }
-#pragma unroll
-          for (int hh = 0; hh < 2; hh++) {
-            const f32x16& s = sacc[qb];
-            const f32x16& d = dpacc[qb];
-            pfr[qb * 2 + hh] = pack8<T>(s[8 * hh + 0], s[8 * hh + 1], s[8 * hh + 2], s[8 * hh + 3], s[8 * hh + 4],
-                                        s[8 * hh + 5], s[8 * hh + 6], s[8 * hh + 7]);
-            dsf[qb * 2 + hh] = pack8<T>(d[8 * hh + 0], d[8 * hh + 1], d[8 * hh + 2], d[8 * hh + 3], d[8 * hh + 4],
-                                        d[8 * hh + 5], d[8 * hh + 6], d[8 * hh + 7]);
-          }
-        }
-        // dV^T += dO^T P,  dK^T += Q^T dS   (contraction over the 64 query rows), fragments requested ahead as
-        // above; the accumulators are pinned to the accumulation registers, as in the pipelined path
-        constexpr int PER_KS = DVB + DKB, NB = (BMQ / 16) * PER_KS;
-        auto t_frag = [&](int i) {
-          const int ks = i / PER_KS, d = i % PER_KS;
-          if (d < DVB) return *(const v8*)(dotl + ta[ks ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
-          return *(const v8*)(qtl + ta[ks ^ ((d - DVB) & 3)] + (d - DVB) * 32 * TrTile64::ROW_BYTES);
         };
-        v8 ring[RING];
-#pragma unroll
-        for (int r = 0; r < RING; r++) ring[r] = t_frag(r);
+        v8 ring[RING], dsf[BMQ / 16];
+        f32x4 d4[NCH / 4];
+        static_for<0, RING>([&](auto R) { ring[decltype(R)::value] = t_frag(R); });
+        static_for<0, 2>([&](auto M) {
+          constexpr int m = decltype(M)::value;
+          d4[m] = *(const f32x4*)(deltal + (m / 4) * 32 + 8 * (m % 4) + 4 * g);
+        });
         __builtin_amdgcn_sched_barrier(0);
+        static_for<0, NB>([&](auto I) {
+          constexpr int i = decltype(I)::value;
+          if constexpr (i < NV) MT<T>::mfma32_acc_guarded(dvacc[i % DVB], ring[i % RING], pfr[i / DVB]);
+          else MT<T>::mfma32_acc_guarded(dkacc[(i - NV) % DKB], ring[i % RING], dsf[(i - NV) / DKB]);
+          if constexpr (i + RING < NB) ring[i % RING] = t_frag(std::integral_constant<int, i + RING>{});
+          if constexpr (i % 2 == 0 && i / 2 + 2 < NCH / 4) {
+            constexpr int m = i / 2 + 2;
+            d4[m] = *(const f32x4*)(deltal + (m / 4) * 32 + 8 * (m % 4) + 4 * g);
+          }
+          if constexpr (i < NCH / 2) {
+            // dS = P o (dP - delta) for two values (d4 holds -delta)
 #pragma unroll
-        for (int i = 0; i < NB; i++) {
-          const int ks = i / PER_KS, d = i % PER_KS;
-          if (d < DVB) MT<T>::mfma32_acc_guarded(dvacc[d], ring[i % RING], pfr[ks]);
-          else MT<T>::mfma32_acc_guarded(dkacc[d - DVB], ring[i % RING], dsf[ks]);
-          if (i + RING < NB) ring[i % RING] = t_frag(i + RING);
+            for (int idx = 2 * i; idx < 2 * i + 2; idx++) {
+              const int qb = idx / 16, v = idx % 16, m = idx / 4, e = idx % 4;
+              float dsv = sacc[qb][v] * (dpacc[qb][v] + d4[m][e]);
+              asm volatile("" : "+v"(dsv));
+              dpacc[qb][v] = dsv;
+            }
+            if constexpr (i % 4 == 3) {
+              constexpr int h = i / 4, qb = h / 2, hh = h % 2;
+              const f32x16& x = dpacc[qb];
+              dsf[h] = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4], x[8 * hh + 5],
+                                x[8 * hh + 6], x[8 * hh + 7]);
+            }
+          }
           __builtin_amdgcn_sched_barrier(0);
-        }
+        });
       }
       __builtin_amdgcn_s_waitcnt(0);
       __syncthreads();  // the next tile has landed; everyone is done with the transposed tiles
       advance(c_hl, c_idx);
-      if (it + 1 < n_iter) {
-        transpose_tile<DQK>(smem + Q_AT, smem + QTR_AT, tid);
-        transpose_tile<DV>(smem + DO_AT, smem + DOTR_AT, tid);
-      }
-      __syncthreads();
     }
   }
 
