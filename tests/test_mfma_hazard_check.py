@@ -71,3 +71,33 @@ def test_main_exit_status(tmp_path, capsys):
   assert chk.main([str(good)]) == 0
   assert chk.main([str(good), str(bad)]) == 1
   assert "less than 2 wait states" in capsys.readouterr().out
+
+
+def test_flags_accumulator_copied_right_behind_the_mfma_that_writes_it():
+  body = """
+	;;#ASMSTART
+	s_nop 1
+	v_mfma_f32_32x32x16_bf16 a[48:63], v[2:5], v[14:17], a[48:63]
+	;;#ASMEND
+	v_accvgpr_mov_b32 a127, a63
+"""
+  found = chk.scan(_asm(body))
+  assert len(found) == 1 and found[0][2].startswith("v_mfma") and "a127, a63" in found[0][3]
+  # unrelated accumulation registers, and the same read behind enough wait states, are fine
+  assert chk.scan(_asm(body.replace("a127, a63", "a127, a15"))) == []
+  waited = body.replace("\tv_accvgpr_mov_b32", "\t;;#ASMSTART\n\ts_nop 15\n\ts_nop 3\n\t;;#ASMEND\n\tv_accvgpr_mov_b32")
+  assert chk.scan(_asm(waited)) == []
+
+
+def test_accumulating_into_the_same_registers_is_not_a_read_hazard():
+  found = chk.scan(_asm("""
+	;;#ASMSTART
+	v_mfma_f32_32x32x16_bf16 a[0:15], v[2:5], v[14:17], a[0:15]
+	;;#ASMEND
+	ds_read_b128 v[2:5], v40
+	s_waitcnt lgkmcnt(0)
+	;;#ASMSTART
+	v_mfma_f32_32x32x16_bf16 a[0:15], v[2:5], v[14:17], a[0:15]
+	;;#ASMEND
+"""))
+  assert found == []

@@ -1221,11 +1221,21 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
 #pragma unroll
   for (int m = 0; m < 4; m++) ta[m] = (unsigned)TrTile64::chunk_off(ln, m, g);
 
+  // Wide heads, causal (four waves, one per SIMD, 512 registers each): the dQ accumulators are pinned to the
+  // accumulation registers like dK / dV in the other kernel.  Not the other four-wave variants: there the branches
+  // of the tile loop end with the accumulators in different registers and the compiler copies them right behind the
+  // MFMAs, which it does not know to be MFMAs (the build's assembly scan rejects that).  Eight waves have 256
+  // registers in all and keep the compiler's MFMA form.
+  constexpr bool ACC_PINNED = NW == 4 && CAUSAL && DQK > 128;
   f32x16 dqacc[DKB];
+  {
+    f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int d = 0; d < DKB; d++)
-#pragma unroll
-    for (int v = 0; v < 16; v++) dqacc[d][v] = 0.f;
+    for (int d = 0; d < DKB; d++) {
+      if constexpr (ACC_PINNED) asm volatile("" : "+a"(zero16));
+      dqacc[d] = zero16;
+    }
+  }
   const float c = a.scale_log2;
   const int wq_last = wq0 + 31;
   const int qrow = wq0 + ln;
@@ -1482,7 +1492,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
             else dp[nb] = MT<T>::mfma32(f, dof[sl.k], sl.k == 0 ? zero : dp[nb]);
           } else {
             constexpr int nb = i >= ACC1 ? 1 : 0, j = nb ? i - ACC1 : i - ACC0, hh = j / DKB, d = j % DKB;
-            dqacc[d] = MT<T>::mfma32(f, df[nb][hh], dqacc[d]);
+            if constexpr (ACC_PINNED) MT<T>::mfma32_acc_guarded(dqacc[d], f, df[nb][hh]);
+            else dqacc[d] = MT<T>::mfma32(f, df[nb][hh], dqacc[d]);
           }
         };
         // elements [E0, E0 + N) of block NB spread evenly over the LEN slots starting at START
@@ -1572,6 +1583,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   
   }
 
+  // (pinned accumulators come out of asm MFMAs: the compiler inserts no wait states before reading them)
+  if constexpr (ACC_PINNED) asm volatile("s_nop 15\n\ts_nop 3" ::: "memory");
   if (qrow < Sq) {
     T* dqp = (T*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qrow * a.dqs[2];
     const float sc = a.sm_scale;
