@@ -313,3 +313,8 @@ def test_llama3_70b_shape_slice():  # benchmark configuration 3: B=1, S=8192, 64
 
 def test_deepseek_v3_shape_slice():  # benchmark configuration 4: B=1, S=4096, 128 heads, qk 192 / v 128, scale 1/sqrt(128)
   _slice_check(1, 128, 128, 4096, 192, 128, None, 1234 + 4, b_sel=0, g_sel=77)
+
+
+def test_deepseek_v3_shape_slice_qk_scale():
+  # the same configuration with the scale a 192-wide q.k product would usually take (the reference uses the v head dim)
+  _slice_check(1, 128, 128, 4096, 192, 128, None, 1234 + 4, b_sel=0, g_sel=3, sm_scale=192 ** -0.5)

@@ -258,6 +258,54 @@ def test_rope_full_size_llama3_8b_bitwise():
   assert torch.equal(gq, gqr) and torch.equal(gk, gkr)
 
 
+@pytest.mark.parametrize("hidden", [1536, 512])
+def test_rmsnorm_full_size_deepseek_latents(hidden):
+  """The DeepSeek-V3 configuration's norms: x (1, 4096, hidden) bf16 with hidden = the q / kv latent widths, eps 1e-6
+  (narrow rows: one wave per row for 512).  y bit-compared with the eager-order oracle, dx and dw against fp64."""
+  S, eps = 4096, 1e-6
+  g = torch.Generator(device="cpu").manual_seed(1234 + 4)
+  x = torch.randn((1, S, hidden), generator=g).to(torch.bfloat16)
+  dy = torch.randn((1, S, hidden), generator=g).to(torch.bfloat16)
+  w = (1 + 0.1 * torch.randn((hidden,), generator=g)).to(torch.bfloat16)
+  xg, wg = x.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+  y = tpa.ops.rmsnorm(xg, wg, eps)
+  y.backward(dy.to(DEV))
+  y_ref = orc.rms_norm(x, w, eps)
+  assert (y.detach().cpu() != y_ref).float().mean().item() < 2e-3
+  assert_close(y, y_ref, "y", rel_l2=1e-3, scale_abs=True)
+  x64 = x.double().requires_grad_(True)
+  orc.rms_norm_exact(x64, w.double(), eps).backward(dy.double())
+  assert_close(xg.grad, x64.grad, "dx", scale_abs=True)
+  _, dw = orc.rms_norm_grads_eager_order(x, w, dy, eps)
+  assert_close(wg.grad, dw, "dw", scale_abs=True)
+
+
+def test_rope_full_size_deepseek_interleaved_bitwise():
+  """The DeepSeek-V3 configuration's rotary step: the 64 rotated dims of q (1, 128, 4096, 64) and of the shared key
+  (1, 1, 4096, 64), interleaved pairs, theta 1e4: identical bits to the eager expression, forward and backward."""
+  Hq, S, D = 128, 4096, 64
+  g = torch.Generator(device="cpu").manual_seed(1234 + 4)
+  q = torch.randn((1, S, Hq, D), generator=g).to(torch.bfloat16).transpose(1, 2)
+  k = torch.randn((1, S, 1, D), generator=g).to(torch.bfloat16).transpose(1, 2)
+  pos = torch.arange(S)[None].float()
+  cos, sin = orc.rotary_cos_sin(orc.default_rope_frequencies(D, 10000.0), pos, torch.bfloat16)
+  qd, kd, cd, sd = q.to(DEV), k.to(DEV), cos.to(DEV), sin.to(DEV)
+  qo, ko = tpa.apply_rotary_pos_emb_interleave(qd, kd, cd, sd)
+  qr, kr = orc.apply_rotary_pos_emb_interleave(q, k, cos, sin)
+  assert torch.equal(qo.cpu(), qr) and torch.equal(ko.cpu(), kr)
+  # gradient of sum(out * w) with respect to the inputs, against autograd through the eager expression in fp64
+  wq = torch.randn((1, S, Hq, D), generator=g).to(torch.bfloat16).transpose(1, 2)
+  qg = qd.clone().requires_grad_(True)
+  kg = kd.clone().requires_grad_(True)
+  qo2, ko2 = tpa.apply_rotary_pos_emb_interleave(qg, kg, cd, sd)
+  (qo2.float() * wq.to(DEV).float()).sum().backward()
+  q64 = q.double().requires_grad_(True)
+  qr64, _ = orc.apply_rotary_pos_emb_interleave(q64, k.double(), cos.double(), sin.double())
+  (qr64 * wq.double()).sum().backward()
+  assert_close(qg.grad, q64.grad, "dq rot", scale_abs=True)
+  assert kg.grad is None or float(kg.grad.abs().max()) == 0.0
+
+
 def test_rope_offsets_beyond_32_bits():
   """A q view whose rows lie 2^18 elements apart: offsets inside one batch element pass 2^31 elements, which
   takes the kernel instantiation with 64-bit per-lane offsets."""
