@@ -270,14 +270,16 @@ __global__ __launch_bounds__(256) void xent_mean_kernel(const float* __restrict_
 }
 
 // dlogits[b, s, c] = dloss / count * (softmax(logits[b, s])[c] - [c == label]) for rows with a target, else 0
+constexpr int XENT_BWD_U = 1;
 template <typename T>
 __global__ __launch_bounds__(256) void xent_bwd_kernel(const T* __restrict__ logits, const int64_t* __restrict__ labels,
                                                        const float* __restrict__ lse, const float* __restrict__ loss_and_count,
                                                        const float* __restrict__ dloss, T* __restrict__ dlogits, int S, int V,
                                                        int64_t ls_b, int64_t ls_s, int64_t lab_b, int64_t ds_b, int64_t ds_s,
-                                                       int ignore_index) {
+                                                       int ignore_index, int chunks) {
   constexpr int E = 16 / sizeof(T);
-  const int row = blockIdx.x;
+  // consecutive blocks walk one row before the next: the card streams through the tensor like a flat copy
+  const int row = blockIdx.x / chunks, chunk = blockIdx.x - row * chunks;
   const int b = row / S, s = row - b * S;
   const T* lr = logits + b * ls_b + s * ls_s;
   T* dr = dlogits + b * ds_b + s * ds_s;
@@ -288,12 +290,17 @@ __global__ __launch_bounds__(256) void xent_bwd_kernel(const T* __restrict__ log
   }
   const float scale = lab < 0 ? 0.f : dloss[0] / loss_and_count[1];
   const float l = lse[row];
+  const int lab32 = (int)lab;  // labels are below V, which is an int
+  constexpr float LOG2E_F = 1.4426950408889634f;
+  const float nl2 = -l * LOG2E_F;
   const int nvec = V / E;
   const bool vec = ((((size_t)lr) | ((size_t)dr)) & 15) == 0;
   if (vec) {
-    // four vectors per thread and step, all loads first: one load in flight per thread does not keep HBM busy
-    constexpr int U = 4;
-    for (int v0 = threadIdx.x; v0 < nvec; v0 += 256 * U) {
+    // XENT_BWD_U vectors per thread, all loads first, and one such step per block (`chunks` blocks per row): the card
+    // sees many short blocks instead of a loop per row.  Measured at 8192 rows x 128256 fp32: a loop per row 5.1 TB/s,
+    // 4 vectors per thread in short blocks 5.7 TB/s, 1 vector per thread 5.9 TB/s
+    constexpr int U = XENT_BWD_U;
+    for (int v0 = chunk * (256 * U) + threadIdx.x; v0 < nvec; v0 += chunks * 256 * U) {
       float x[U][E];
 #pragma unroll
       for (int u = 0; u < U; u++) {
@@ -304,17 +311,22 @@ __global__ __launch_bounds__(256) void xent_bwd_kernel(const T* __restrict__ log
       for (int u = 0; u < U; u++) {
         const int v = v0 + 256 * u;
         if (v < nvec) {
+          // two instructions per element (an fma into log2 units and the exponential); the label's one-hot term is
+          // taken off in the one vector that holds it (per-element 64-bit compares cost more than the stream)
           float o[E];
 #pragma unroll
-          for (int e = 0; e < E; e++) {
-            const int c = v * E + e;
-            o[e] = lab < 0 ? 0.f : scale * (__expf(x[u][e] - l) - (c == lab ? 1.f : 0.f));
+          for (int e = 0; e < E; e++) o[e] = lab32 < 0 ? 0.f : scale * __builtin_amdgcn_exp2f(__builtin_fmaf(x[u][e], LOG2E_F, nl2));
+          if ((unsigned)(lab32 - v * E) < (unsigned)E) {
+#pragma unroll
+            for (int e = 0; e < E; e++)
+              if (v * E + e == lab32) o[e] -= scale;
           }
           store_f_nt<T, E>(dr + (int64_t)v * E, o);
         }
       }
     }
   }
+  if (chunk != 0) return;
   for (int c = (vec ? nvec * E : 0) + threadIdx.x; c < V; c += 256) {
     const float x = lab < 0 ? 0.f : Elem<T>::to_f(lr[c]);
     dr[c] = Elem<T>::from_f(lab < 0 ? 0.f : scale * (__expf(x - l) - (c == lab ? 1.f : 0.f)));
@@ -448,11 +460,15 @@ extern "C" int tp_cross_entropy_bwd(const void* logits, const int64_t* labels, c
   TP_REQUIRE(logits && labels && lse && loss_and_count && dloss && dlogits, TP_ERR_BAD_ARG, "tp_cross_entropy_bwd: null pointer");
   TP_REQUIRE(B > 0 && S > 0 && V > 0 && (int64_t)B * S < (1ll << 31), TP_ERR_BAD_ARG, "tp_cross_entropy_bwd: bad shape");
   hipStream_t st = (hipStream_t)stream;
-  const dim3 grid((unsigned)(B * S)), block(256);
+  // (vectors per row / vectors per block, for the narrower element type's vector count at most 65535 blocks along y)
+  const int64_t vec_per_row = (int64_t)V / (dtype == TP_F32 ? 4 : 8);
+  int64_t chunks = std::max<int64_t>((vec_per_row + 256 * XENT_BWD_U - 1) / (256 * XENT_BWD_U), 1);
+  chunks = std::min<int64_t>(chunks, ((1ll << 31) - 1) / ((int64_t)B * S));  // (rows x chunks blocks in a 1-D grid)
+  const dim3 grid((unsigned)((int64_t)B * S * chunks)), block(256);
   if (dtype == TP_F32)
-    xent_bwd_kernel<float><<<grid, block, 0, st>>>((const float*)logits, labels, lse, loss_and_count, dloss, (float*)dlogits, S, V, logits_b_stride, logits_s_stride, labels_b_stride, dlogits_b_stride, dlogits_s_stride, ignore_index);
+    xent_bwd_kernel<float><<<grid, block, 0, st>>>((const float*)logits, labels, lse, loss_and_count, dloss, (float*)dlogits, S, V, logits_b_stride, logits_s_stride, labels_b_stride, dlogits_b_stride, dlogits_s_stride, ignore_index, (int)chunks);
   else if (dtype == TP_BF16)
-    xent_bwd_kernel<bf16_t><<<grid, block, 0, st>>>((const bf16_t*)logits, labels, lse, loss_and_count, dloss, (bf16_t*)dlogits, S, V, logits_b_stride, logits_s_stride, labels_b_stride, dlogits_b_stride, dlogits_s_stride, ignore_index);
+    xent_bwd_kernel<bf16_t><<<grid, block, 0, st>>>((const bf16_t*)logits, labels, lse, loss_and_count, dloss, (bf16_t*)dlogits, S, V, logits_b_stride, logits_s_stride, labels_b_stride, dlogits_b_stride, dlogits_s_stride, ignore_index, (int)chunks);
   else
     TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_cross_entropy_bwd: dtype %d (fp32 and bf16 logits only)", dtype);
   return check_launch("tp_cross_entropy_bwd");
