@@ -432,6 +432,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   int* bk = active + nqt;  // 8 ints: per-wave (min,max) of kv ids
   int* pmin = bk + 8;      // per query tile: (min,max) of the rows' positions in the key order (mask extensions)
   int* pmax = pmin + nqt;
+  // per visited tile, in visiting order: (query tile, min id, max id, index into the range arrays), 16 bytes that one
+  // LDS read fetches a whole tile ahead of their use (the tile loop would otherwise start every tile by waiting out
+  // a chain of dependent LDS reads: list entry -> its ranges -> which body to run)
+  int* ctl = (int*)(((size_t)(pmax + nqt) + 15) & ~(size_t)15);
   int nact = nqt;
   int wkmin = 0, wkmax = 0;
   if (SEG) {
@@ -470,6 +474,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       cnt += __popcll(m);
     }
     nact = cnt;
+    __syncthreads();
+    for (int i = tid; i < nact; i += 256) {
+      const int t = active[i];
+      *(i32x4*)(ctl + 4 * i) = i32x4{qt_first + t, qmin[t], qmax[t], t};
+    }
     __syncthreads();
   }
   const int n_iter = nact * a.n_rep;
@@ -528,20 +537,24 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   const float c = a.scale_log2;
 
   // wave-level decisions for a query tile (uniform): skip if every query row precedes every kv row
-  auto tile_mode = [&](int idx, int qi0) {  // 0 = nothing to compute, 1 = no masking needed, 2 = masked
+  // (lo, hi: id range of the query tile; t: its index into the position ranges)
+  auto tile_mode_of = [&](int lo, int hi, int t, int qi0) {  // 0 = nothing to compute, 1 = no masking needed, 2 = masked
     bool skip = (CAUSAL && qi0 + BMQ - 1 < wkv0) || wkv0 >= Skv;
     bool need_mask = (qi0 + BMQ > Sq) || (wkv0 + 32 > Skv) || (CAUSAL && qi0 < wkv0 + 31);
     if (SEG) {
-      const int lo = qmin[active[idx]], hi = qmax[active[idx]];
       skip = skip || hi < wkmin || lo > wkmax;
       need_mask = need_mask || !(lo == hi && wkmin == wkmax && lo == wkmin);
     }
     if (ext) {
-      const int plo = pmin[active[idx]], phi = pmax[active[idx]];
+      const int plo = pmin[t], phi = pmax[t];
       skip = skip || wkv0 > phi + a.mx.hi_off || wkv0 + 31 < plo - a.mx.lo_off;
       need_mask = need_mask || capped || !(wkv0 >= phi - a.mx.lo_off && wkv0 + 31 <= plo + a.mx.hi_off);
     }
     return skip ? 0 : (need_mask ? 2 : 1);
+  };
+  auto tile_mode = [&](int idx, int qi0) {
+    const int t = SEG ? active[idx] : 0;
+    return tile_mode_of(SEG ? qmin[t] : 0, SEG ? qmax[t] : 0, t, qi0);
   };
   // iteration -> (query head of the group, query tile): heads outer, tiles inner, no division in the loop
   auto advance = [&](int& hl, int& idx) {
@@ -572,6 +585,18 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     for (int m = 0; m < 4; m++) tb[m] = ta[m] + tr_bias;
     if (n_iter > 0) { issue_tile(n_hl, n_idx, 0, 0); advance(n_hl, n_idx); }
     if (n_iter > 1) { issue_tile(n_hl, n_idx, 1, 1); advance(n_hl, n_idx); }
+    // the control entry of the tile being computed and the query tile whose loads are issued next, as scalars; their
+    // successors are read at the top of a tile and taken over at its end
+    auto entry = [&](int idx) {
+      if constexpr (SEG) return *(const i32x4*)(ctl + 4 * min(idx, max(nact - 1, 0)));
+      else return i32x4{qt_first + idx, 0, 0, 0};
+    };
+    auto scalar4 = [&](i32x4 v) {
+      return i32x4{__builtin_amdgcn_readfirstlane(v[0]), __builtin_amdgcn_readfirstlane(v[1]),
+                   __builtin_amdgcn_readfirstlane(v[2]), __builtin_amdgcn_readfirstlane(v[3])};
+    };
+    i32x4 cur = scalar4(entry(0));
+    int nq_cur = __builtin_amdgcn_readfirstlane(entry(n_idx)[0]);
     // all earlier loads (the K/V fragments, the first tiles) have landed
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
@@ -605,9 +630,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     // one query tile; the buffer index is a constant (the loop below alternates two copies of this)
     auto iteration = [&](auto BUFc, const int it) {
       constexpr int buf = decltype(BUFc)::value;
-      const int qi0 = qtile_of(c_idx) * BMQ;
-      const int mode = tile_mode(c_idx, qi0);
+      const int qi0 = cur[0] * BMQ;
+      const int mode = tile_mode_of(cur[1], cur[2], cur[3], qi0);
       const bool issue_next = it + 2 < n_iter;
+      // successors of the two cursors (read now, used when this tile is done)
+      int c_hl2 = c_hl, c_idx2 = c_idx, n_hl2 = n_hl, n_idx2 = n_idx;
+      advance(c_hl2, c_idx2);
+      if (issue_next) advance(n_hl2, n_idx2);
+      const i32x4 cur_next = entry(c_idx2);
+      const int nq_next = entry(n_idx2)[0];
       const unsigned char* ql = smem + Q_AT + buf * Q_BYTES;
       const unsigned char* dol = smem + DO_AT + buf * DO_BYTES;
       const unsigned char* qtl = smem + (QTR_AT + buf * QTR_BYTES - TR_BIAS);     // + tb[]
@@ -639,7 +670,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         nx.rr = make_rsrc_words(src, (issue_next && (wave < 2 || (wave == 2 && has_seg) || (wave == 3 && has_pos))) ? (unsigned)Sq * 4u : 0u);
       }
       {
-        const int qt = issue_next ? qtile_of(n_idx) : 0;
+        const int qt = issue_next ? nq_cur : 0;
         nx.offq = __builtin_amdgcn_readfirstlane((unsigned)qt * q_tile_bytes);
         nx.offo = __builtin_amdgcn_readfirstlane((unsigned)qt * do_tile_bytes);
         nx.offr = __builtin_amdgcn_readfirstlane((unsigned)(qt * BMQ) * 4u);
@@ -842,8 +873,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       else if (mode == 2) body(std::integral_constant<int, 2>{});
       else body(std::integral_constant<int, 0>{});
       __syncthreads();
-      if (issue_next) advance(n_hl, n_idx);
-      advance(c_hl, c_idx);
+      n_hl = n_hl2; n_idx = n_idx2;
+      c_hl = c_hl2; c_idx = c_idx2;
+      cur = scalar4(cur_next);
+      nq_cur = __builtin_amdgcn_readfirstlane(nq_next);
       rslot = rslot == 2 ? 0 : rslot + 1;
     };
     for (int it = 0; it < n_iter; it += 2) {
@@ -1169,7 +1202,24 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
     }
     nact = cnt;
     __syncthreads();
+    // One word per visited tile, in visiting order: the kv tile in the low half, above it two bits per wave (its rows'
+    // ids miss the tile's range / the ranges are not one shared id).  The tile loop reads the word a tile ahead of
+    // its use; it would otherwise start every tile by waiting out a chain of dependent LDS reads (list entry ->
+    // ranges -> which body to run).
+    for (int i = tid; i < nact; i += 64 * NW) {
+      const int t = active[i], lo = kvmin[t], hi = kvmax[t];
+      unsigned bits = 0;
+#pragma unroll
+      for (int w = 0; w < NW; w++) {
+        const int wmin = bq[2 * w], wmax = bq[2 * w + 1];
+        const unsigned sk = (hi < wmin || lo > wmax) ? 1u : 0u, nm = (lo == hi && wmin == wmax && lo == wmin) ? 0u : 2u;
+        bits |= (sk | nm) << (2 * w);
+      }
+      active[i] = (int)((unsigned)t | (bits << 16));  // (thread i owns entry i: read above, replaced here)
+    }
+    __syncthreads();
   }
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
 
   // ---- staging of one K/V tile through registers.  Every thread owns one 4-row x 8-column block of K and
   // (4 waves) one of V; with 8 waves the first four stage K, the last four V.
@@ -1242,9 +1292,11 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
 
   // i-th kv tile to visit, as a scalar (a tile offset in vector registers would put every staging load into a
   // loop over its distinct values)
-  auto tile_at = [&](int i) { return SEG ? __builtin_amdgcn_readfirstlane(active[i]) : i; };
+  auto entry = [&](int i) { return SEG ? active[min(i, max(nact - 1, 0))] : i; };
+  // entries of the tile being computed and of the one after it (whose loads are issued at the top of this one)
+  int cur = __builtin_amdgcn_readfirstlane(entry(0)), nxt = __builtin_amdgcn_readfirstlane(entry(1));
   if (nact > 0) {
-    load_tile(tile_at(0), 0);
+    load_tile(cur & 0xffff, 0);
     store_tile(0, 0, 0);
   }
   __builtin_amdgcn_s_waitcnt(0);  // Q / dO fragments, LSE and delta have landed (see the dK/dV kernel)
@@ -1304,10 +1356,11 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
     bool pending = false;
     int kslot = 0;
     for (int it = 0; it < nact; it++) {
-      const int t = tile_at(it);
+      const int t = cur & 0xffff;
       const int kv0 = t * BN;
       const int buf = it & 1;
-      if (it + 1 < nact) load_tile(tile_at(it + 1), it);
+      if (it + 1 < nact) load_tile(nxt & 0xffff, it);
+      const int after = entry(it + 2);  // read now, taken over at the end of the tile
       const int kprev = kslot == 0 ? 2 : kslot - 1, knext = kslot == 2 ? 0 : kslot + 1;
       const unsigned char* kl = smem + buf * KV_BYTES;
       const unsigned char* vl = kl + K_BYTES;
@@ -1318,9 +1371,9 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
       bool skip = CAUSAL && kv0 > wq_last;
       bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0);
       if (SEG) {
-        const int lo = kvmin[t], hi = kvmax[t];
-        skip = skip || hi < wqmin || lo > wqmax;
-        need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
+        const unsigned my = ((unsigned)cur >> (16 + 2 * wave_s)) & 3u;
+        skip = skip || (my & 1u);
+        need_mask = need_mask || (my & 2u);
       }
       if (ext) {
         skip = skip || kv0 > wpmax + a.mx.hi_off || kv0 + BN - 1 < wpmin - a.mx.lo_off;
@@ -1423,14 +1476,17 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
       }
       __syncthreads();
       kslot = knext;
+      cur = nxt;
+      nxt = __builtin_amdgcn_readfirstlane(after);
     }
     if (pending) drain(smem + KTR_AT + (kslot == 0 ? 2 : kslot - 1) * KTR_BYTES);
   } else {
   for (int it = 0; it < nact; it++) {
-      const int t = tile_at(it);
+      const int t = cur & 0xffff;
       const int kv0 = t * BN;
       const int buf = it & 1;
-      if (it + 1 < nact) load_tile(tile_at(it + 1), it);
+      if (it + 1 < nact) load_tile(nxt & 0xffff, it);
+      const int after = entry(it + 2);  // read now, taken over at the end of the tile
   
       const unsigned char* kl = smem + buf * KV_BYTES;
       const unsigned char* vl = kl + K_BYTES;
@@ -1440,9 +1496,9 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
       bool skip = CAUSAL && kv0 > wq_last;
       bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0);
       if (SEG) {
-        const int lo = kvmin[t], hi = kvmax[t];
-        skip = skip || hi < wqmin || lo > wqmax;
-        need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
+        const unsigned my = ((unsigned)cur >> (16 + 2 * wave_s)) & 3u;
+        skip = skip || (my & 1u);
+        need_mask = need_mask || (my & 2u);
       }
       if (ext) {
         skip = skip || kv0 > wpmax + a.mx.hi_off || kv0 + BN - 1 < wpmin - a.mx.lo_off;
@@ -1579,6 +1635,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
         ((int*)(smem + SEG_AT + (buf ^ 1) * BN * 4))[tid] = sreg;
       }
       __syncthreads();
+      cur = nxt;
+      nxt = __builtin_amdgcn_readfirstlane(after);
     }
   
   }
@@ -1631,7 +1689,7 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
     constexpr int ROWS = 3 * BMQ * 16;
     constexpr int NBUF = (2 * BUF + ROWS + 4096 <= 160 * 1024) ? 2 : 1;
     const int nqt = (a.Sq + BMQ - 1) / BMQ;
-    const size_t smem = (size_t)NBUF * BUF + ROWS + (SEG ? (size_t)(5 * nqt + 8) * 4 : 0);
+    const size_t smem = (size_t)NBUF * BUF + ROWS + (SEG ? (size_t)(9 * nqt + 8 + 4) * 4 : 0);
     TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_bwd: Sq=%d needs %zu bytes of LDS (max 163840)", a.Sq, smem);
     auto kern = attn_bwd_dkdv_kernel<T, DQK, DV, NBUF, CAUSAL, SEG>;
     static bool attr_set = false;
