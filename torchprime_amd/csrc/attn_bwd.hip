@@ -713,6 +713,33 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         // for no fragment that is not due anyway
         f32x4 nl0[4], nl1[4], nd0[4], nd1[4];
         float fc[2][16];  // soft cap: 1 - tanh^2 of every score, kept from P to dS
+        // Masked tiles without the mask extensions: which of the tile's 64 query rows this lane's kv column may see,
+        // as one bit per row, built once per tile (bounds and causality are a bit range; the rows of each id present
+        // among the wave's columns come from a ballot over the tile's id vector).  An element then costs a bit-field
+        // extract and an AND instead of four compares.  rowbits[qb] is shifted so that value v of the lane's 16 is
+        // bit 8 (v / 4) + v % 4.
+        unsigned rowbits[2] = {0u, 0u};
+        const bool by_bits = MASKED && !(GEN && ext);
+        if (MASKED && by_bits) {
+          const int lo_r = CAUSAL ? max(kvcol - qi0, 0) : 0;
+          const int hi_r = kvcol < Skv ? min(Sq - qi0, BMQ) : 0;
+          unsigned long long m = 0ull;
+          if (hi_r > lo_r) m = (~0ull << lo_r) & (~0ull >> (64 - hi_r));
+          if (SEG && has_seg) {
+            const int rowseg = segl[lane];  // lane l: id of the tile's query row l
+            unsigned long long ms = 0ull, todo = ~0ull;
+            while (todo) {
+              const int x = __builtin_amdgcn_readlane(segk, (int)__builtin_ctzll(todo));
+              const unsigned long long rows = __ballot(rowseg == x);
+              const bool mine = segk == x;
+              ms = mine ? rows : ms;
+              todo &= ~__ballot(mine);
+            }
+            m &= ms;
+          }
+          rowbits[0] = (unsigned)m >> (4 * g);
+          rowbits[1] = (unsigned)(m >> 32) >> (4 * g);
+        }
 
         auto frag = [&](auto I) -> v8 {
           constexpr int i = decltype(I)::value;
@@ -773,16 +800,20 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
                 }
                 float pv = fast_exp2(__builtin_fmaf(sval, c, nl[vq][e]));
                 if (MASKED) {
-                  const int r = qb * 32 + 8 * vq + 4 * g + e;
-                  const int qrow = qi0 + r;
-                  bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || !has_seg || segl[r] == segk);
-                  if (GEN) {
-                    if (ext) {
-                      const int qp = has_pos ? posl[r] : qrow;
-                      ok = ok && kvcol >= qp - a.mx.lo_off && kvcol <= qp + a.mx.hi_off;
+                  if (by_bits) {
+                    pv = __builtin_bit_cast(float, __builtin_bit_cast(int, pv) & __builtin_amdgcn_sbfe((int)rowbits[qb], 8 * vq + e, 1));
+                  } else {
+                    const int r = qb * 32 + 8 * vq + 4 * g + e;
+                    const int qrow = qi0 + r;
+                    bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || !has_seg || segl[r] == segk);
+                    if (GEN) {
+                      if (ext) {
+                        const int qp = has_pos ? posl[r] : qrow;
+                        ok = ok && kvcol >= qp - a.mx.lo_off && kvcol <= qp + a.mx.hi_off;
+                      }
                     }
+                    pv = ok ? pv : 0.f;
                   }
-                  pv = ok ? pv : 0.f;
                 }
                 asm volatile("" : "+v"(pv));  // anchors the computation in this slot (it would sink past the barrier)
                 s[qb][v] = pv;
