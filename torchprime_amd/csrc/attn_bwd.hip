@@ -1326,6 +1326,35 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   auto entry = [&](int i) { return SEG ? active[min(i, max(nact - 1, 0))] : i; };
   // entries of the tile being computed and of the one after it (whose loads are issued at the top of this one)
   int cur = __builtin_amdgcn_readfirstlane(entry(0)), nxt = __builtin_amdgcn_readfirstlane(entry(1));
+  // Masked tiles: which of the tile's 64 kv rows this lane's query row may see, one bit per row, built once per tile
+  // (bounds, causality and the band of the mask extensions are a bit range; the rows of each id present among the
+  // wave's query rows come from a ballot over the tile's id vector).  An element then costs a bit-field extract and
+  // an AND instead of its compares.  kbits[nb] is shifted so that value v of the lane's 16 is bit 8 (v / 4) + v % 4.
+  unsigned kbits[2] = {0u, 0u};
+  auto make_key_bits = [&](int kv0, const int* sl) {
+    int lo = 0, hi = min(Skv - kv0, BN);
+    if (CAUSAL) hi = min(hi, wq0 + ln - kv0 + 1);
+    if (GEN) {
+      lo = max(lo_q - kv0, 0);
+      hi = min(hi, hi_q - kv0 + 1);
+    }
+    unsigned long long m = 0ull;
+    if (hi > lo) m = (~0ull << lo) & (~0ull >> (64 - hi));
+    if (SEG && has_seg) {
+      const int rowseg = sl[lane];  // lane l: id of the tile's kv row l
+      unsigned long long ms = 0ull, todo = ~0ull;
+      while (todo) {
+        const int x = __builtin_amdgcn_readlane(segq, (int)__builtin_ctzll(todo));
+        const unsigned long long rows = __ballot(rowseg == x);
+        const bool mine = segq == x;
+        ms = mine ? rows : ms;
+        todo &= ~__ballot(mine);
+      }
+      m &= ms;
+    }
+    kbits[0] = (unsigned)m >> (4 * g);
+    kbits[1] = (unsigned)(m >> 32) >> (4 * g);
+  };
   if (nact > 0) {
     load_tile(cur & 0xffff, 0);
     store_tile(0, 0, 0);
@@ -1410,6 +1439,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
         skip = skip || kv0 > wpmax + a.mx.hi_off || kv0 + BN - 1 < wpmin - a.mx.lo_off;
         need_mask = need_mask || capped || !(kv0 >= wpmax - a.mx.lo_off && kv0 + BN - 1 <= wpmin + a.mx.hi_off);
       }
+      if (need_mask && !skip) make_key_bits(kv0, sl);
       auto body = [&](auto masked_c) {
         constexpr bool MASKED = decltype(masked_c)::value;
         v8 fr[NF];
@@ -1461,14 +1491,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
               }
               float pv = fast_exp2(__builtin_fmaf(sval, c, -lse_s));
               if (MASKED) {
-                const int kvl = nb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
-                const int kv = kv0 + kvl;
-                bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
-                if (GEN) {
-                  ok = ok && kv >= lo_q && kv <= hi_q;
-                  pv *= dcap;
-                }
-                pv = ok ? pv : 0.f;
+                if (GEN) pv *= dcap;
+                pv = __builtin_bit_cast(float, __builtin_bit_cast(int, pv) & __builtin_amdgcn_sbfe((int)kbits[nb], 8 * (v / 4) + (v % 4), 1));
               }
               asm volatile("" : "+v"(pv));
               sv[v] = pv;
@@ -1541,6 +1565,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
       //   slots   S0^T = K0 Q^T alternating with dP0^T = V0 dO^T;  S1^T with dP1^T;
       //           dQ^T += K0^T dS0^T;  dQ^T += K1^T dS1^T (first the half whose operand is ready first)
       //   VALU    dS0^T under S1^T/dP1^T; dS1^T under the dQ^T slots that do not need it yet
+      if (need_mask && !skip) make_key_bits(kv0, sl);
       auto body = [&](auto masked_c) {
         constexpr bool MASKED = decltype(masked_c)::value;
         // 4 waves: S/dP of both kv blocks first, so that dS of block 0 has the MFMAs of block 1 next to it.
@@ -1601,14 +1626,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
               }
               float pv = fast_exp2(__builtin_fmaf(sval, c, -lse_s));
               if (MASKED) {
-                const int kvl = nb * 32 + 8 * (v / 4) + 4 * g + (v % 4);
-                const int kv = kv0 + kvl;
-                bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
-                if (GEN) {
-                  ok = ok && kv >= lo_q && kv <= hi_q;
-                  pv *= dcap;
-                }
-                pv = ok ? pv : 0.f;
+                if (GEN) pv *= dcap;
+                pv = __builtin_bit_cast(float, __builtin_bit_cast(int, pv) & __builtin_amdgcn_sbfe((int)kbits[nb], 8 * (v / 4) + (v % 4), 1));
               }
               float dsv = pv * (dp[nb][v] + ndelta_s);
               asm volatile("" : "+v"(dsv));  // keeps the computation in this slot
