@@ -302,18 +302,46 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
     const unsigned char* kl = smem + K_AT + buf * K_STEP;
     const unsigned char* vl = smem + buf * V_BYTES;  // + tb[]
     const int* sl = (const int*)(kl + (SEG_AT - K_AT) + buf * (SEG_STEP - K_STEP));
+    // Masked tiles: which of the tile's 64 kv rows this lane's query row may see, one bit per row, built once per
+    // tile (bounds, causality and the band of the mask extensions are a bit range; the rows of each id present among
+    // the wave's query rows come from a ballot over the tile's id vector).  An element then costs a bit-field
+    // extract and a bit-field insert of -inf instead of its compares.  kbits[hf] is shifted so that value v of the
+    // lane's 16 is bit 8 (v / 4) + v % 4.
+    unsigned kbits[2] = {0u, 0u};
+    if (MASKED) {
+      int lo = 0, hi = min(Skv - kv0, BN);
+      if (CAUSAL) hi = min(hi, qrow - kv0 + 1);
+      if (GEN) {
+        lo = max(lo_q - kv0, 0);
+        hi = min(hi, hi_q - kv0 + 1);
+      }
+      unsigned long long m = 0ull;
+      if (hi > lo) m = (~0ull << lo) & (~0ull >> (64 - hi));
+      if (SEG && has_seg) {
+        const int rowseg = sl[lane];  // lane l: id of the tile's kv row l
+        unsigned long long ms = 0ull, todo = ~0ull;
+        while (todo) {
+          const int x = __builtin_amdgcn_readlane(segq, (int)__builtin_ctzll(todo));
+          const unsigned long long rows = __ballot(rowseg == x);
+          const bool mine = segq == x;
+          ms = mine ? rows : ms;
+          todo &= ~__ballot(mine);
+        }
+        m &= ms;
+      }
+      kbits[0] = (unsigned)m >> (4 * g);
+      kbits[1] = (unsigned)(m >> 32) >> (4 * g);
+    }
     auto mask_half = [&](f32x16& s, int hf) {
 #pragma unroll
       for (int v = 0; v < 16; v++) {
-        const int kvl = hf * 32 + 8 * (v / 4) + 4 * g + (v % 4);
-        const int kv = kv0 + kvl;
-        bool ok = kv < Skv && (!CAUSAL || kv <= qrow) && (!SEG || sl[kvl] == segq);
+        // soft cap on the raw score, rescaled so that the common scale c still applies afterwards
         if (GEN) {
-          ok = ok && kv >= lo_q && kv <= hi_q;
-          // soft cap on the raw score, rescaled so that the common scale c still applies afterwards
           if (capped) s[v] = a.mx.cap_out * fast_tanh(s[v] * a.mx.cap_in);
         }
-        s[v] = ok ? s[v] : -INFINITY;
+        const unsigned keep = (unsigned)__builtin_amdgcn_sbfe((int)kbits[hf], 8 * (v / 4) + (v % 4), 1);  // all ones or zero
+        const float x = s[v];
+        s[v] = __uint_as_float((__float_as_uint(x) & keep) | (0xff800000u & ~keep));
       }
     };
     constexpr int S1 = KSTEPS, PV0 = 2 * KSTEPS, PV1 = PV0 + 2 * DVB, NS = PV1 + 2 * DVB;
