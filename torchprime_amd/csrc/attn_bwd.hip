@@ -982,7 +982,28 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         };
         v8 ring[RING];
         f32x4 l4[NCH / 4];
-        i32x4 sg[NCH / 4];
+        // masked tiles: one bit per query row of the tile for this lane's kv column (see the pipelined path)
+        unsigned rowbits[2] = {0u, 0u};
+        if constexpr (MASKED) {
+          const int lo_r = CAUSAL ? max(kvcol - qi0, 0) : 0;
+          const int hi_r = kvcol < Skv ? min(Sq - qi0, BMQ) : 0;
+          unsigned long long m = 0ull;
+          if (hi_r > lo_r) m = (~0ull << lo_r) & (~0ull >> (64 - hi_r));
+          if (SEG && has_seg) {
+            const int rowseg = segl[lane];
+            unsigned long long ms = 0ull, todo = ~0ull;
+            while (todo) {
+              const int x = __builtin_amdgcn_readlane(segk, (int)__builtin_ctzll(todo));
+              const unsigned long long rows = __ballot(rowseg == x);
+              const bool mine = segk == x;
+              ms = mine ? rows : ms;
+              todo &= ~__ballot(mine);
+            }
+            m &= ms;
+          }
+          rowbits[0] = (unsigned)m >> (4 * g);
+          rowbits[1] = (unsigned)(m >> 32) >> (4 * g);
+        }
         static_for<0, RING>([&](auto R) { ring[decltype(R)::value] = a_frag(R); });
         static_for<0, NA>([&](auto I) {
           constexpr int i = decltype(I)::value;
@@ -994,7 +1015,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
           if constexpr (i + 4 >= NS && (i + 4 - NS) % 2 == 0 && (i + 4 - NS) / 2 < NCH / 4) {
             constexpr int m = (i + 4 - NS) / 2, qb = m / 4, vq = m % 4;
             l4[m] = *(const f32x4*)(lsel + qb * 32 + 8 * vq + 4 * g);
-            if constexpr (MASKED && SEG) sg[m] = *(const i32x4*)(segl + qb * 32 + 8 * vq + 4 * g);
           }
           if constexpr (i >= NS) {
             // P = exp2(S c - LSE) for two values (l4 holds -LSE in log2 units); rows of the C tile are queries
@@ -1003,12 +1023,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
             for (int idx = 2 * k; idx < 2 * k + 2; idx++) {
               const int qb = idx / 16, v = idx % 16, m = idx / 4, e = idx % 4;
               float pv = fast_exp2(__builtin_fmaf(sacc[qb][v], c, l4[m][e]));
-              if constexpr (MASKED) {
-                const int qrow = qi0 + qb * 32 + 8 * (v / 4) + 4 * g + e;
-                bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow);
-                if constexpr (SEG) ok = ok && sg[m][e] == segk;
-                pv = ok ? pv : 0.f;
-              }
+              if constexpr (MASKED)
+                pv = __uint_as_float(__float_as_uint(pv) & (unsigned)__builtin_amdgcn_sbfe((int)rowbits[qb], 8 * (v / 4) + e, 1));
               asm volatile("" : "+v"(pv));  // keeps the computation in this step
               sacc[qb][v] = pv;
             }
