@@ -28,6 +28,8 @@ reference, which needs torch_xla / jax / omegaconf):
                             k_rot expanded by hand; gradient of k_rot = sum over heads       pinned
   add_rms_norm, l2_norm     F.rms_norm without a weight, explicit fp64 loops                pinned
   apply_rotary_emb_llama4   complex rotation of adjacent pairs (torch.polar), norm preservation      pinned
+  llama4_attention          explicit loops (pair rotation, unit-RMS q/k, per-position scale, softmax);
+                            = llama_attention with de-interleaved projection rows on rotary layers     pinned
   attn temperature          closed form log(floor((p+1)/f)+1) a + 1 at hand-computed positions       pinned
   swiglu                    x * sigmoid(x) * u in fp64 loops                                          pinned
   cross_entropy_loss        explicit per-token -log softmax loops incl. ignored labels; F.cross_entropy   pinned
@@ -404,6 +406,27 @@ def apply_attn_temperature(q, floor_scale, attn_scale):
   """model/llama4/model.py:522-525: q (B, S, N, D) times the per-position scale, cast back to q's dtype."""
   sc = attn_temperature_scales(q.shape[1], floor_scale, attn_scale).view(1, -1, 1, 1)
   return (q * (sc.double() if q.dtype == torch.float64 else sc)).to(q.dtype)
+
+
+def llama4_attention(x, wq, wk, wv, wo, n_heads, n_kv_heads, cos, sin, use_rope, use_qk_norm, eps,
+                     attn_temperature_tuning, floor_scale, attn_scale, attention_mask="causal"):
+  """``Llama4TextAttention.forward`` (model/llama4/model.py:489-533): projections viewed (B, S, N, D); on rotary layers
+  the adjacent-pair rotation and, with ``use_qk_norm``, the weightless L2 norm of q and k; on the others the attention
+  temperature on q; then eager attention, head merge, output projection."""
+  B, S, hidden = x.shape
+  hd = hidden // n_heads
+  q = (x @ wq.T).view(B, S, n_heads, hd)
+  k = (x @ wk.T).view(B, S, n_kv_heads, hd)
+  v = (x @ wv.T).view(B, S, n_kv_heads, hd).transpose(1, 2)
+  if use_rope:
+    q, k = apply_rotary_emb_llama4(q, k, cos, sin)
+    if use_qk_norm:
+      q, k = l2_norm(q, eps), l2_norm(k, eps)
+  if attn_temperature_tuning and not use_rope:
+    q = apply_attn_temperature(q, floor_scale, attn_scale)
+  mask = causal_additive_mask(S, x.dtype) if isinstance(attention_mask, str) else attention_mask
+  o = eager_attention(q.transpose(1, 2), k.transpose(1, 2), v, mask)
+  return o.transpose(1, 2).contiguous().reshape(B, S, hidden) @ wo.T
 
 
 def swiglu(gate, up):

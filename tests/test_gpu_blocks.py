@@ -138,3 +138,33 @@ def test_deepseek_v3_attention_module(q_lora, interleave):
   y_ref = orc.deepseek_v3_attention(x64, {k.replace(".weight", ""): v for k, v in r.items()}, H, nope, rope, vd, kvl,
                                     cos.cpu().double(), sin.cpu().double(), rope_interleave=interleave)
   _compare(y, y_ref, xg, x64, dict(m.named_parameters()), r, do)
+
+
+@pytest.mark.parametrize("layer,qk_norm,temperature", [(0, True, True), (0, False, True), (1, True, True), (1, True, False)])
+def test_llama4_attention_module(layer, qk_norm, temperature):
+  """``Llama4TextAttention``: layer 0 is a rotary layer (adjacent-pair rotation, optional L2 norm of q and k), layer 1
+  a NoPE layer (attention temperature on q), GQA 8:2, head dim 128 as in the Llama-4 configurations."""
+  B, S, H, Hkv, hd = 2, 192, 8, 2, 128
+  hidden = H * hd
+  cfg = _cfg(attention_kernel="splash_attention", hidden_size=hidden, num_attention_heads=H, num_key_value_heads=Hkv,
+             head_dim=hd, no_rope_layers=[1, 0], use_qk_norm=qk_norm, rms_norm_eps=1e-5, attn_temperature_tuning=temperature,
+             floor_scale=64.0, attn_scale=0.1, max_position_embeddings=4096)
+  m = tpa.Llama4TextAttention(cfg, layer_idx=layer).to(DEV).to(DT)
+  assert m.use_rope == (layer == 0) and hasattr(m, "qk_norm") == (qk_norm and layer == 0)
+  w = {
+    "q_proj.weight": randn((hidden, hidden), 41, DT, 0.02), "k_proj.weight": randn((Hkv * hd, hidden), 42, DT, 0.02),
+    "v_proj.weight": randn((Hkv * hd, hidden), 43, DT, 0.02), "o_proj.weight": randn((hidden, hidden), 44, DT, 0.02),
+  }
+  _load(m, w)
+  x, do = randn((B, S, hidden), 45, DT), randn((B, S, hidden), 46, DT)
+  pos = torch.arange(S)[None].float()
+  rot = tpa.Llama4TextRotaryEmbedding(hd, 500000.0).to(DEV)
+  xg = x.to(DEV).requires_grad_(True)
+  cos, sin = rot(xg, pos.to(DEV))
+  y = m(xg, (cos, sin))
+  assert y.shape == (B, S, hidden) and y.dtype == DT
+  x64 = x.double().requires_grad_(True)
+  r = {k: v.double().requires_grad_(True) for k, v in w.items()}
+  y_ref = orc.llama4_attention(x64, r["q_proj.weight"], r["k_proj.weight"], r["v_proj.weight"], r["o_proj.weight"], H, Hkv,
+                               cos.cpu().double(), sin.cpu().double(), layer == 0, qk_norm, 1e-5, temperature, 64.0, 0.1)
+  _compare(y, y_ref, xg, x64, dict(m.named_parameters()), r, do)

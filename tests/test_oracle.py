@@ -492,6 +492,52 @@ def test_attn_temperature_closed_form():
   assert torch.equal(out, (q.float() * s6.view(1, 6, 1, 1)).bfloat16())
 
 
+@pytest.mark.parametrize("use_rope,qk_norm,temperature", [(True, True, False), (True, False, False), (False, False, True), (False, False, False)])
+def test_llama4_attention_against_explicit_loops(use_rope, qk_norm, temperature):
+  B, S, H, Hkv, hd = 1, 7, 4, 2, 8
+  hidden = H * hd
+  x = randn((B, S, hidden), 90).double()
+  wq, wk, wv, wo = (randn(shape, 91 + i, std=0.2).double() for i, shape in
+                    enumerate(((hidden, hidden), (Hkv * hd, hidden), (Hkv * hd, hidden), (hidden, hidden))))
+  inv = orc.default_rope_frequencies(hd, 10000.0).double()
+  pos = torch.arange(S).double() * 3
+  ang = pos[:, None] * inv[None]  # (S, hd/2)
+  cos = torch.cat([ang.cos(), ang.cos()], -1)[None]
+  sin = torch.cat([ang.sin(), ang.sin()], -1)[None]
+  eps, floor_scale, attn_scale = 1e-6, 2.0, 0.3
+  out = orc.llama4_attention(x, wq, wk, wv, wo, H, Hkv, cos, sin, use_rope, qk_norm, eps, temperature, floor_scale, attn_scale)
+  # explicit form
+  q = (x[0] @ wq.T).view(S, H, hd)
+  k = (x[0] @ wk.T).view(S, Hkv, hd)
+  v = (x[0] @ wv.T).view(S, Hkv, hd)
+  def prep(t, i, n):
+    vec = t[i, n].clone()
+    if use_rope:
+      z = torch.complex(vec[0::2], vec[1::2]) * torch.polar(torch.ones(hd // 2, dtype=torch.float64), ang[i])
+      vec = torch.stack([z.real, z.imag], -1).reshape(hd)
+      if qk_norm:
+        vec = vec / math.sqrt((vec * vec).mean().item() + eps)
+    return vec
+  merged = torch.zeros(S, hidden, dtype=torch.float64)
+  for h in range(H):
+    for i in range(S):
+      qi = prep(q, i, h)
+      if temperature and not use_rope:
+        qi = qi * (math.log(math.floor((i + 1.0) / floor_scale) + 1.0) * attn_scale + 1.0)
+      sc = torch.tensor([float(qi @ prep(k, j, h // (H // Hkv))) / math.sqrt(hd) for j in range(i + 1)], dtype=torch.float64)
+      p_ = torch.softmax(sc, 0)
+      merged[i, h * hd : (h + 1) * hd] = sum(p_[j] * v[j, h // (H // Hkv)] for j in range(i + 1))
+  # (the eager softmax is evaluated in fp32, attention.py:163-165: 1e-7-sized differences from the fp64 loops)
+  torch.testing.assert_close(out[0], merged @ wo.T, rtol=2e-5, atol=2e-6)
+  if use_rope and not qk_norm:
+    # the adjacent-pair rotation is the rotate-half rotation on de-interleaved head dims, and q.k does not care
+    perm = torch.cat([torch.arange(0, hd, 2), torch.arange(1, hd, 2)])
+    pq = torch.cat([h * hd + perm for h in range(H)])
+    pk = torch.cat([h * hd + perm for h in range(Hkv)])
+    ref = orc.llama_attention(x, wq[pq], wk[pk], wv, wo, H, Hkv, cos, sin)
+    torch.testing.assert_close(out, ref, rtol=2e-5, atol=2e-6)
+
+
 def test_swiglu_and_cross_entropy_explicit_forms():
   g, u = randn((5, 24), 68).double(), randn((5, 24), 69).double()
   ref = torch.empty_like(g)

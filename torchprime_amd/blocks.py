@@ -143,3 +143,57 @@ class DeepseekV3Attention(nn.Module):
     out = self.attention_block(q, k, v, attention_mask)
     out = out.transpose(1, 2).contiguous().reshape(bsz, q_len, -1)
     return self.o_proj(out)
+
+
+class Llama4TextAttention(nn.Module):
+  """model/llama4/model.py:427-533: rotary layers apply the adjacent-pair rotation and (``use_qk_norm``) the weightless
+  L2 norm to q and k; layers without rotary ("NoPE") scale the queries by the position-dependent attention temperature
+  instead.  Which kind a layer is comes from ``config.no_rope_layers[layer_idx]`` as in the reference."""
+
+  def __init__(self, config, layer_idx: int | None = None):
+    super().__init__()
+    from .llama4 import Llama4TextL2Norm
+
+    self.config = config
+    self.attention_block = AttentionModule(config)
+    self.layer_idx = layer_idx
+    self.num_attention_heads = config.num_attention_heads
+    self.num_key_value_heads = config.num_key_value_heads
+    self.num_key_value_groups = self.num_attention_heads // self.num_key_value_heads
+    self.attn_scale = config.attn_scale
+    self.floor_scale = config.floor_scale
+    self.attn_temperature_tuning = config.attn_temperature_tuning
+    no_rope = getattr(config, "no_rope_layers", None)
+    self.use_rope = bool(no_rope and layer_idx is not None and layer_idx < len(no_rope) and no_rope[layer_idx])
+    if (config.head_dim * config.num_attention_heads) != config.hidden_size:
+      raise ValueError(
+        f"hidden_size must be divisible by num_attention_heads (got `hidden_size`: {config.hidden_size}"
+        f" and `num_attention_heads`: {config.num_attention_heads})."
+      )
+    self.hidden_size = config.hidden_size
+    self.head_dim = self.hidden_size // self.num_attention_heads
+    bias = bool(getattr(config, "attention_bias", False))
+    self.q_proj = nn.Linear(self.hidden_size, self.num_attention_heads * self.head_dim, bias=bias)
+    self.k_proj = nn.Linear(self.hidden_size, self.num_key_value_heads * self.head_dim, bias=bias)
+    self.v_proj = nn.Linear(self.hidden_size, self.num_key_value_heads * self.head_dim, bias=bias)
+    self.o_proj = nn.Linear(self.hidden_size, self.hidden_size, bias=bias)
+    if getattr(config, "use_qk_norm", False) and self.use_rope:
+      self.qk_norm = Llama4TextL2Norm(config.rms_norm_eps)
+
+  def forward(self, hidden_states, position_embeddings, attention_mask=None, position_ids=None):
+    from .llama4 import apply_attn_temperature, apply_rotary_emb
+
+    bsz, q_len, _ = hidden_states.size()
+    q = self.q_proj(hidden_states).view(bsz, q_len, -1, self.head_dim)
+    k = self.k_proj(hidden_states).view(bsz, q_len, -1, self.head_dim)
+    v = self.v_proj(hidden_states).view(bsz, q_len, -1, self.head_dim).transpose(1, 2)
+    if self.use_rope:
+      q, k = apply_rotary_emb(q, k, position_embeddings)
+    if hasattr(self, "qk_norm"):
+      q, k = self.qk_norm(q), self.qk_norm(k)
+    if self.attn_temperature_tuning and not self.use_rope:
+      q = apply_attn_temperature(q, self.floor_scale, self.attn_scale)
+    out = self.attention_block(q.transpose(1, 2), k.transpose(1, 2), v, attention_mask)
+    out = out.transpose(1, 2).contiguous().reshape(bsz, q_len, self.hidden_size)
+    return self.o_proj(out)
+
