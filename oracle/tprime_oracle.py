@@ -28,6 +28,7 @@ reference, which needs torch_xla / jax / omegaconf):
                             k_rot expanded by hand; gradient of k_rot = sum over heads       pinned
   add_rms_norm, l2_norm     F.rms_norm without a weight, explicit fp64 loops                pinned
   apply_rotary_emb_llama4   complex rotation of adjacent pairs (torch.polar), norm preservation      pinned
+  llama_decoder_layer       HuggingFace LlamaDecoderLayer (eager) where importable; composed of pinned parts  pinned
   llama4_attention          explicit loops (pair rotation, unit-RMS q/k, per-position scale, softmax);
                             = llama_attention with de-interleaved projection rows on rotary layers     pinned
   attn temperature          closed form log(floor((p+1)/f)+1) a + 1 at hand-computed positions       pinned
@@ -306,6 +307,18 @@ def llama_attention(x, wq, wk, wv, wo, n_heads, n_kv_heads, cos, sin, attention_
   mask = causal_additive_mask(S, x.dtype) if isinstance(attention_mask, str) else attention_mask
   o = eager_attention(q, k, v, mask)
   return o.transpose(1, 2).contiguous().reshape(B, S, hidden) @ wo.T
+
+
+def llama_decoder_layer(x, w, n_heads, n_kv_heads, eps, cos, sin, attention_mask="causal"):
+  """``LlamaDecoderLayer.forward`` (model/llama/model.py:276-296): norm, attention, residual add, norm, SwiGLU MLP
+  (``down(silu(gate(h)) * up(h))``, :137-139), residual add.  ``w``: weights under the reference's state-dict names."""
+  h = rms_norm(x, w["input_layernorm.weight"], eps)
+  h = llama_attention(h, w["self_attn.q_proj.weight"], w["self_attn.k_proj.weight"], w["self_attn.v_proj.weight"],
+                      w["self_attn.o_proj.weight"], n_heads, n_kv_heads, cos, sin, attention_mask)
+  h = x + h
+  m = rms_norm(h, w["post_attention_layernorm.weight"], eps)
+  m = swiglu(m @ w["mlp.gate_proj.weight"].T, m @ w["mlp.up_proj.weight"].T) @ w["mlp.down_proj.weight"].T
+  return h + m
 
 
 def mixtral_attention(x, wq, wk, wv, wo, n_heads, n_kv_heads, rope_theta, max_position_embeddings, position_ids,

@@ -168,3 +168,33 @@ def test_llama4_attention_module(layer, qk_norm, temperature):
   y_ref = orc.llama4_attention(x64, r["q_proj.weight"], r["k_proj.weight"], r["v_proj.weight"], r["o_proj.weight"], H, Hkv,
                                cos.cpu().double(), sin.cpu().double(), layer == 0, qk_norm, 1e-5, temperature, 64.0, 0.1)
   _compare(y, y_ref, xg, x64, dict(m.named_parameters()), r, do)
+
+
+@pytest.mark.parametrize("kernel", ["splash_attention", None])
+def test_llama_decoder_layer(kernel):
+  """A whole decoder layer from the package's modules (norms, attention, residual add fused into the second norm,
+  SwiGLU MLP) against the oracle's restatement of LlamaDecoderLayer: output, input gradient and every weight gradient."""
+  B, S, hidden, H, Hkv, hd, inter = 2, 160, 512, 8, 2, 64, 1024
+  cfg = _cfg(attention_kernel=kernel, hidden_size=hidden, num_attention_heads=H, num_key_value_heads=Hkv,
+             intermediate_size=inter, rms_norm_eps=1e-5, hidden_act="silu")
+  m = tpa.LlamaDecoderLayer(cfg, 0).to(DEV).to(DT)
+  w = {
+    "self_attn.q_proj.weight": randn((hidden, hidden), 51, DT, 0.02), "self_attn.k_proj.weight": randn((Hkv * hd, hidden), 52, DT, 0.02),
+    "self_attn.v_proj.weight": randn((Hkv * hd, hidden), 53, DT, 0.02), "self_attn.o_proj.weight": randn((hidden, hidden), 54, DT, 0.02),
+    "mlp.gate_proj.weight": randn((inter, hidden), 55, DT, 0.02), "mlp.up_proj.weight": randn((inter, hidden), 56, DT, 0.02),
+    "mlp.down_proj.weight": randn((hidden, inter), 57, DT, 0.02),
+    "input_layernorm.weight": (1 + randn((hidden,), 58, std=0.1)).to(DT), "post_attention_layernorm.weight": (1 + randn((hidden,), 59, std=0.1)).to(DT),
+  }
+  _load(m, w)
+  x, do = randn((B, S, hidden), 60, DT), randn((B, S, hidden), 61, DT)
+  pos = torch.arange(S)[None].float()
+  rot = tpa.LlamaRotaryEmbedding(hd, 500000.0).to(DEV)
+  xg = x.to(DEV).requires_grad_(True)
+  cos, sin = rot(xg, pos.to(DEV))
+  mask = orc.causal_additive_mask(S).to(DEV) if kernel is None else None
+  y = m(xg, attention_mask=mask, position_embeddings=(cos, sin))
+  assert y.shape == (B, S, hidden) and y.dtype == DT
+  x64 = x.double().requires_grad_(True)
+  r = {k: v.double().requires_grad_(True) for k, v in w.items()}
+  y_ref = orc.llama_decoder_layer(x64, r, H, Hkv, 1e-5, cos.cpu().double(), sin.cpu().double())
+  _compare(y, y_ref, xg, x64, dict(m.named_parameters()), r, do)

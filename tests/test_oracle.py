@@ -344,6 +344,32 @@ def test_llama_block_matches_hf_llama_when_available():
   torch.testing.assert_close(got, ref, rtol=1e-4, atol=1e-5)
 
 
+def test_llama_decoder_layer_matches_hf_when_available():
+  """The whole layer (norms, attention, SwiGLU MLP, both residual adds) against HuggingFace's LlamaDecoderLayer."""
+  try:
+    from transformers import LlamaConfig
+    from transformers.models.llama.modeling_llama import LlamaDecoderLayer, LlamaRotaryEmbedding
+    cfg = LlamaConfig(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, head_dim=64, intermediate_size=384,
+                      num_hidden_layers=1, vocab_size=128, rms_norm_eps=1e-5, rope_theta=500000.0, attention_bias=False,
+                      mlp_bias=False, hidden_act="silu", max_position_embeddings=8192)
+    cfg._attn_implementation = "eager"
+    torch.manual_seed(1)
+    layer, rot = LlamaDecoderLayer(cfg, 0).eval(), LlamaRotaryEmbedding(cfg)
+    x = randn((2, 48, 256), 29)
+    with torch.no_grad():
+      layer.input_layernorm.weight.copy_(1 + randn((256,), 30, std=0.05))
+      layer.post_attention_layernorm.weight.copy_(1 + randn((256,), 31, std=0.05))
+      pos = torch.arange(48)[None]
+      cos, sin = rot(x, pos)
+      ref = layer(x, attention_mask=orc.causal_additive_mask(48), position_ids=pos, position_embeddings=(cos, sin))
+      ref = ref[0] if isinstance(ref, tuple) else ref
+  except Exception as e:
+    pytest.skip(f"transformers Llama modules not usable here: {e}")
+  w = {k: v.detach() for k, v in layer.state_dict().items()}
+  got = orc.llama_decoder_layer(x, w, 4, 2, 1e-5, cos, sin)
+  torch.testing.assert_close(got, ref, rtol=1e-4, atol=1e-5)
+
+
 # ---- the callers ------------------------------------------------------------------------------------------
 def test_mixtral_attention_is_llama_attention_with_gathered_tables():
   B, S, H, Hkv, hd = 2, 12, 4, 2, 16

@@ -197,3 +197,31 @@ class Llama4TextAttention(nn.Module):
     out = out.transpose(1, 2).contiguous().reshape(bsz, q_len, self.hidden_size)
     return self.o_proj(out)
 
+
+class LlamaDecoderLayer(nn.Module):
+  """model/llama/model.py:241-296 with the package's modules: the residual add after the attention and the norm that
+  follows it are one kernel (``add_rms_norm``), the MLP's gate product another; the four adds / norms / products of
+  the reference's layer are evaluated in the same order and with the same roundings."""
+
+  def __init__(self, config, layer_idx: int):
+    super().__init__()
+    from .mlp import LlamaMLP
+    from .norm import LlamaRMSNorm
+
+    self.hidden_size = config.hidden_size
+    self.self_attn = LlamaAttention(config=config, layer_idx=layer_idx)
+    self.mlp = LlamaMLP(config)
+    self.input_layernorm = LlamaRMSNorm(config.hidden_size, eps=config.rms_norm_eps)
+    self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, eps=config.rms_norm_eps)
+
+  def forward(self, hidden_states, attention_mask=None, position_ids=None, position_embeddings=None):
+    from .norm import add_rms_norm
+
+    residual = hidden_states
+    hidden_states = self.input_layernorm(hidden_states)
+    hidden_states = self.self_attn(hidden_states, position_embeddings, attention_mask, position_ids)
+    # residual + hidden_states, then post_attention_layernorm of the sum, in one pass
+    hidden_states, residual = add_rms_norm(hidden_states, residual, self.post_attention_layernorm)
+    hidden_states = self.mlp(hidden_states)
+    return residual + hidden_states
+
