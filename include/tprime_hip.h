@@ -152,6 +152,7 @@ size_t tp_attn_bwd_workspace_bytes(int B, int Hq, int Sq);
  *   dout, out (B,Hq,Sq,Dv), each with its own stride array (do_strides, o_strides)
  *   dq/dk/dv  strided like q/k/v but with their own stride arrays
  *   ws        fp32 workspace of tp_attn_bwd_workspace_bytes(B,Hq,Sq) bytes
+ *   dtype     TP_BF16 / TP_F16 (head dims (64,64), (128,128), (192,128)) or TP_F32 (head dims 64 and 128)
  * ---------------------------------------------------------------------------------------------- */
 int tp_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
                 const float* lse, const int32_t* seg, void* dq, void* dk, void* dv, float* ws, int B,

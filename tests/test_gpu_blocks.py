@@ -198,3 +198,41 @@ def test_llama_decoder_layer(kernel):
   r = {k: v.double().requires_grad_(True) for k, v in w.items()}
   y_ref = orc.llama_decoder_layer(x64, r, H, Hkv, 1e-5, cos.cpu().double(), sin.cpu().double())
   _compare(y, y_ref, xg, x64, dict(m.named_parameters()), r, do)
+
+
+def test_llama_attention_module_fp32_forward_and_backward():
+  """benchmark configuration 1's block in fp32 end to end on the GPU (fp32 RMSNorm-free attention block: projections,
+  RoPE, fp32 attention forward and backward, output projection): output, input gradient and weight gradients against
+  the fp64 oracle at the fp32 class of tolerance (relative-L2 2e-5, 2e-5 of the tensor's largest value per element)."""
+  B, S, hidden, H, hd = 2, 128, 512, 8, 64
+  cfg = _cfg(attention_kernel=None, hidden_size=hidden, num_attention_heads=H, num_key_value_heads=H)
+  m = tpa.LlamaAttention(cfg).to(DEV)
+  w = {
+    "q_proj.weight": randn((hidden, hidden), 71, std=0.02), "k_proj.weight": randn((hidden, hidden), 72, std=0.02),
+    "v_proj.weight": randn((hidden, hidden), 73, std=0.02), "o_proj.weight": randn((hidden, hidden), 74, std=0.02),
+  }
+  _load(m, w)
+  x, do = randn((B, S, hidden), 75), randn((B, S, hidden), 76)
+  pos = torch.arange(S)[None].float()
+  rot = tpa.LlamaRotaryEmbedding(hd, 500000.0).to(DEV)
+  xg = x.to(DEV).requires_grad_(True)
+  cos, sin = rot(xg, pos.to(DEV))
+  old = torch.backends.cuda.matmul.allow_tf32
+  torch.backends.cuda.matmul.allow_tf32 = False
+  try:
+    y = m(xg, (cos, sin), orc.causal_additive_mask(S).to(DEV))
+    assert y.dtype == torch.float32
+    y.backward(do.to(DEV))
+  finally:
+    torch.backends.cuda.matmul.allow_tf32 = old
+  x64 = x.double().requires_grad_(True)
+  r = {k: v.double().requires_grad_(True) for k, v in w.items()}
+  y_ref = orc.llama_attention(x64, r["q_proj.weight"], r["k_proj.weight"], r["v_proj.weight"], r["o_proj.weight"], H, H,
+                              cos.cpu().double(), sin.cpu().double())
+  y_ref.backward(do.double())
+  def tight(got, ref, name):
+    assert_close(got, ref, name, max_abs=2e-5 * max(1.0, ref.abs().max().item()), rel_l2=2e-5)
+  tight(y, y_ref, "out")
+  tight(xg.grad, x64.grad, "dx")
+  for name, p in m.named_parameters():
+    tight(p.grad, r[name].grad, f"d{name}")

@@ -274,7 +274,7 @@ def rope_apply(q: Tensor, k: Tensor, cos: Tensor, sin: Tensor, pos: Tensor | Non
 # attention
 # ------------------------------------------------------------------------------------------------
 _SUPPORTED_HEAD_DIMS = ((64, 64), (128, 128), (192, 128))
-_SUPPORTED_HEAD_DIMS_F32 = ((64, 64), (128, 128))  # fp32 operands: forward only (the small fp32 configurations)
+_SUPPORTED_HEAD_DIMS_F32 = ((64, 64), (128, 128))  # fp32 operands (the small fp32 configurations)
 
 
 def _check_attn(q, k, v, seg):
@@ -333,8 +333,6 @@ def attn_bwd(
   dout: Tensor, q: Tensor, k: Tensor, v: Tensor, out: Tensor, lse: Tensor, seg: Tensor | None, sm_scale: float, causal: bool
 ) -> tuple[Tensor, Tensor, Tensor]:
   dev = _lib.require_gpu(dout, q, k, v, out, lse, seg)
-  if q.dtype == torch.float32:
-    raise NotImplementedError("fp32 attention is forward-only; run the backward in bfloat16 or float16")
   B, Hq, Hkv, Sq, Skv, Dqk, Dv = _check_attn(q, k, v, seg)
   q, k, v, out, dout = _prep_heads(q), _prep_heads(k), _prep_heads(v), _prep_heads(out), _prep_heads(dout)
   lse = lse.contiguous()
@@ -429,7 +427,7 @@ def attn_bwd_masked(
 ) -> tuple[Tensor, Tensor, Tensor]:  # fmt: skip
   dev = _lib.require_gpu(dout, q, k, v, out, lse, seg, qpos)
   if q.dtype == torch.float32:
-    raise NotImplementedError("fp32 attention is forward-only; run the backward in bfloat16 or float16")
+    raise NotImplementedError("windows, soft cap and query positions are built for bfloat16 and float16 tensors")
   B, Hq, Hkv, Sq, Skv, Dqk, Dv = _check_attn(q, k, v, seg)
   q, k, v, out, dout = _prep_heads(q), _prep_heads(k), _prep_heads(v), _prep_heads(out), _prep_heads(dout)
   lse = lse.contiguous()
