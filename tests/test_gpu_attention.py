@@ -3,6 +3,7 @@ against the fp32/fp64 CPU oracle on the same seeded inputs.  Tolerance for 16-bi
 gradients: max-abs <= 2e-2 and relative-L2 <= 1e-2 (tests/util.py)."""
 
 import math
+import random
 
 import pytest
 import torch
@@ -61,6 +62,33 @@ def _check(B, Hq, Hkv, S, Dqk, Dv, dtype, causal, seg=None, layout="bshd", seed=
 )
 def test_causal_fwd_bwd(dtype, B, Hq, Hkv, S, Dqk, Dv):
   _check(B, Hq, Hkv, S, Dqk, Dv, dtype, True)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_randomised_shapes_and_segment_layouts(seed):
+  """Seeded random draws over what the kernels branch on: length (around tile edges too), GQA ratio, head dims, dtype,
+  causality, and the id layout (none, packed documents, short documents of a few rows, unsorted ids with repeats):
+  masked tiles are resolved through per-tile bit masks and per-workgroup tile lists, whose corner cases are lengths
+  and document boundaries that fall on or next to tile and wave boundaries."""
+  rng = random.Random(1000 + seed)
+  Dqk, Dv = rng.choice([(64, 64), (128, 128), (128, 128), (192, 128)])
+  Hkv = rng.choice([1, 2])
+  Hq = Hkv * rng.choice([1, 2, 4])
+  S = rng.choice([31, 32, 33, 63, 64, 65, 127, 128, 129, 191, 255, 256, 257, 300, 383, 448, 513])
+  causal = rng.random() < 0.6
+  dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+  B = rng.choice([1, 2])
+  kind = rng.choice(["none", "packed", "tiny", "unsorted"])
+  if kind == "none":
+    seg = None
+  elif kind == "packed":
+    seg = packed_segment_ids(B, S, 1, max(2, S // 2), seed=seed)[0]
+  elif kind == "tiny":
+    seg = packed_segment_ids(B, S, 1, 9, seed=seed)[0]
+  else:
+    g = torch.Generator().manual_seed(seed)
+    seg = torch.randint(-3, 4, (B, S), generator=g, dtype=torch.int32)
+  _check(B, Hq, Hkv, S, Dqk, Dv, dtype, causal, seg=seg, seed=10 * seed)
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,S,Skv,Dqk,Dv", [(1, 4, 2, 130, 130, 128, 128), (2, 2, 2, 64, 300, 64, 64), (1, 2, 1, 257, 100, 128, 128)])
