@@ -314,6 +314,29 @@ def test_fp32_attention_backward(B, Hq, Hkv, S, Skv, D, causal, use_seg):
     assert_close(got, ref, name, max_abs=2e-5 * max(1.0, ref.abs().max().item()), rel_l2=1e-5)
 
 
+def test_long_packed_sequence_65536_rows():
+  """S = 65536 with 96 packed documents, one head of 128: 1024 query tiles per workgroup list (the longest the dK/dV
+  kernel's LDS holds at this head dim).  A packed row is a set of independent causal problems, so three documents
+  are checked against the oracle run on each of them alone; everything else must be finite."""
+  B, H, S, D = 1, 1, 65536, 128
+  seg, lengths = packed_segment_ids(B, S, 300, 1000, seed=11)
+  q, k, v, do = (heads_view(B, H, S, D, 20 + i, torch.bfloat16) for i in range(4))
+  out, lse, dq, dk, dv = _run(q, k, v, do, seg, True, D**-0.5)
+  for t in (out, dq, dk, dv):
+    assert torch.isfinite(t.float()).all()
+  starts = [0]
+  for L in lengths[0]:
+    starts.append(starts[-1] + L)
+  for d in (0, len(lengths[0]) // 2, len(lengths[0]) - 1):
+    a, b_ = starts[d], starts[d + 1]
+    sl = (slice(None), slice(None), slice(a, b_))
+    o_ref, dq_ref, dk_ref, dv_ref = orc.attention_grads_ref(q[sl], k[sl], v[sl], do[sl], None, True, D**-0.5, torch.float32)
+    assert_close(out[sl], o_ref, f"out, document {d}")
+    assert_close(dq[sl], dq_ref, f"dq, document {d}", scale_abs=True)
+    assert_close(dk[sl], dk_ref, f"dk, document {d}", scale_abs=True)
+    assert_close(dv[sl], dv_ref, f"dv, document {d}", scale_abs=True)
+
+
 def test_unsupported_inputs_raise():
   q = torch.zeros((1, 2, 16, 96), dtype=torch.bfloat16, device=DEV)
   with pytest.raises(NotImplementedError):

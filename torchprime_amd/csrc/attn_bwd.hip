@@ -426,15 +426,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   const int nqt_all = (Sq + BMQ - 1) / BMQ;
   const int qt_first = CAUSAL ? min(kv0 / BMQ, nqt_all) : 0;
   const int nqt = nqt_all - qt_first;
-  int* qmin = (int*)(smem + NBUF * BUF_BYTES + 3 * ROW_BYTES);
+  // id ranges of all query tiles and the list of those to visit: only needed until the control entries below are
+  // built, so they borrow the tile buffers, which nothing has been loaded into yet
+  int* qmin = (int*)smem;
   int* qmax = qmin + nqt;
   int* active = qmax + nqt;
-  int* bk = active + nqt;  // 8 ints: per-wave (min,max) of kv ids
+  int* bk = (int*)(smem + NBUF * BUF_BYTES + 3 * ROW_BYTES);  // 8 ints: per-wave (min,max) of kv ids
   int* pmin = bk + 8;      // per query tile: (min,max) of the rows' positions in the key order (mask extensions)
   int* pmax = pmin + nqt;
-  // per visited tile, in visiting order: (query tile, min id, max id, index into the range arrays), 16 bytes that one
-  // LDS read fetches a whole tile ahead of their use (the tile loop would otherwise start every tile by waiting out
-  // a chain of dependent LDS reads: list entry -> its ranges -> which body to run)
+  // per visited tile, in visiting order: (query tile, min id, max id, index into the position ranges), 16 bytes that
+  // one LDS read fetches a whole tile ahead of their use (the tile loop would otherwise start every tile by waiting
+  // out a chain of dependent LDS reads: list entry -> its ranges -> which body to run)
   int* ctl = (int*)(((size_t)(pmax + nqt) + 15) & ~(size_t)15);
   int nact = nqt;
   int wkmin = 0, wkmax = 0;
@@ -493,7 +495,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   const unsigned q_tile_bytes = (unsigned)(BMQ * a.qs[2] * 2), do_tile_bytes = (unsigned)(BMQ * a.dos[2] * 2);
   const float* lse2 = a.delta + (int64_t)a.B * a.Hq * Sq;  // second half of the workspace (delta kernel)
   unsigned char* const rows_base = smem + NBUF * BUF_BYTES;
-  auto qtile_of = [&](int idx) { return qt_first + (SEG ? active[idx] : idx); };
+  auto qtile_of = [&](int idx) { return SEG ? ctl[4 * idx] : qt_first + idx; };
   auto issue_tile = [&](int hl, int idx, int buf, int rslot) {
     const int hq = hk * a.n_rep + hl;
     const int qt = qtile_of(idx);
@@ -553,8 +555,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     return skip ? 0 : (need_mask ? 2 : 1);
   };
   auto tile_mode = [&](int idx, int qi0) {
-    const int t = SEG ? active[idx] : 0;
-    return tile_mode_of(SEG ? qmin[t] : 0, SEG ? qmax[t] : 0, t, qi0);
+    const int* e = ctl + 4 * idx;
+    return tile_mode_of(SEG ? e[1] : 0, SEG ? e[2] : 0, SEG ? e[3] : 0, qi0);
   };
   // iteration -> (query head of the group, query tile): heads outer, tiles inner, no division in the loop
   auto advance = [&](int& hl, int& idx) {
@@ -1755,8 +1757,9 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
     constexpr int ROWS = 3 * BMQ * 16;
     constexpr int NBUF = (2 * BUF + ROWS + 4096 <= 160 * 1024) ? 2 : 1;
     const int nqt = (a.Sq + BMQ - 1) / BMQ;
-    const size_t smem = (size_t)NBUF * BUF + ROWS + (SEG ? (size_t)(9 * nqt + 8 + 4) * 4 : 0);
-    TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_bwd: Sq=%d needs %zu bytes of LDS (max 163840)", a.Sq, smem);
+    const size_t smem = (size_t)NBUF * BUF + ROWS + (SEG ? (size_t)(6 * nqt + 8 + 4) * 4 : 0);
+    TP_REQUIRE(smem <= 160 * 1024 && (size_t)3 * nqt * 4 <= (size_t)NBUF * BUF, TP_ERR_UNSUPPORTED,
+               "tp_attn_bwd: Sq=%d needs %zu bytes of LDS (max 163840)", a.Sq, smem);
     auto kern = attn_bwd_dkdv_kernel<T, DQK, DV, NBUF, CAUSAL, SEG>;
     static bool attr_set = false;
     if (!attr_set) {
