@@ -82,6 +82,27 @@ __device__ __forceinline__ void load_f_nt(const T* p, float (&out)[N]) {
 #pragma unroll
   for (int i = 0; i < N; i++) out[i] = Elem<T>::to_f(r.v[i]);
 }
+// The same load in two halves: the raw 16-byte words now, the conversion to floats when they are used.  A kernel that
+// walks rows can then request the next row before it works on the current one, at half the registers of holding floats.
+template <typename T, int N> struct Raw { u32x4 q[sizeof(T) * N / 16]; };
+template <typename T, int N>
+__device__ __forceinline__ Raw<T, N> load_raw_nt(const T* p) {
+  constexpr int W = sizeof(T) * N / 16;
+  const u32x4* src = reinterpret_cast<const u32x4*>(p);
+  Raw<T, N> r;
+#pragma unroll
+  for (int i = 0; i < W; i++) r.q[i] = __builtin_nontemporal_load(src + i);
+  return r;
+}
+template <typename T, int N>
+__device__ __forceinline__ void unpack_f(const Raw<T, N>& raw, float (&out)[N]) {
+  constexpr int W = sizeof(T) * N / 16;
+  union { u32x4 q[W]; T v[N]; } r;
+#pragma unroll
+  for (int i = 0; i < W; i++) r.q[i] = raw.q[i];
+#pragma unroll
+  for (int i = 0; i < N; i++) out[i] = Elem<T>::to_f(r.v[i]);
+}
 template <typename T, int N>
 __device__ __forceinline__ void store_f_nt(T* p, const float (&in)[N]) {
   constexpr int W = sizeof(T) * N / 16;

@@ -11,11 +11,17 @@
 
 namespace tp {
 
-constexpr int RMS_MAX_PARTS = 512;  // partial dw rows written by the backward (multiple of 4)
+// Partial dw rows written by the backward (a multiple of 4).  The row-walking kernel is fastest with about 512
+// blocks of four waves (two per CU) at two 16-byte vectors per thread and about twice that at one vector, and
+// slower with more (measured at 512 ... 4096 partial rows over hidden 512 ... 5120): so the count follows the
+// row length, the largest power of two within 2^21 / hidden, between 512 and 4096.
+constexpr int RMS_MIN_PARTS = 512, RMS_MAX_PARTS = 4096;
 
-static inline int rms_parts(int64_t rows) {
-  int64_t p = (rows + 3) / 4 * 4;
-  return (int)(p < RMS_MAX_PARTS ? p : RMS_MAX_PARTS);
+static inline int rms_parts(int64_t rows, int hidden) {
+  int cap = RMS_MAX_PARTS;
+  while (cap > RMS_MIN_PARTS && (int64_t)cap * hidden > (1 << 21)) cap >>= 1;
+  const int64_t p = (rows + 3) / 4 * 4;
+  return (int)(p < cap ? p : cap);
 }
 
 // sum over the WAVES waves that share a row (fixed order); `red` holds one float per wave of the block
@@ -134,7 +140,7 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_generic(const XT* __restrict_
 // Each thread owns fixed columns, so its dw partial sums stay in registers over all the rows it sees and
 // go straight to one partial row per (block, row slot): no atomics, no cross-thread fold.
 // ------------------------------------------------------------------------------------------------
-template <typename XT, typename WT, typename OT, int NV, int WAVES>
+template <typename XT, typename WT, typename OT, int NV, int WAVES, bool RES>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_vec(const OT* __restrict__ dy, const XT* __restrict__ x,
                                                        const WT* __restrict__ w, const float* __restrict__ rstd,
                                                        XT* __restrict__ dx, float* __restrict__ ws, int64_t rows,
@@ -142,6 +148,8 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_vec(const OT* __restrict__ dy
                                                        const XT* __restrict__ dres, int64_t drs) {
   constexpr int E = 16 / sizeof(XT);
   constexpr int RPB = 4 / WAVES, TPR = 64 * WAVES;
+  // Rows are requested one ahead while a thread's share of a row is small enough for both rows to sit in registers.
+  constexpr bool AHEAD = NV <= 2;
   __shared__ float red[2][4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int slot = wave / WAVES;
@@ -150,40 +158,69 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_vec(const OT* __restrict__ dy
   const float inv_h = 1.f / (float)hidden;
   const int64_t step = (int64_t)gridDim.x * RPB;
 
-  float wv[NV][E], wacc[NV][E];
+  Raw<WT, E> rw[NV];  // the weights stay packed and are converted where they are used: half the registers for 16-bit ones
+  float wacc[NV][E];
+  int off[NV];  // element offset of each of the thread's vectors (out-of-range vectors re-read the row's last one)
 #pragma unroll
   for (int i = 0; i < NV; i++) {
     const int v = t + TPR * i;
 #pragma unroll
-    for (int e = 0; e < E; e++) { wacc[i][e] = 0.f; wv[i][e] = 0.f; }
-    if (v < nvec) load_f<WT, E>(w + (int64_t)v * E, wv[i]);
+    for (int e = 0; e < E; e++) wacc[i][e] = 0.f;
+    off[i] = (v < nvec ? v : nvec - 1) * E;
+    rw[i] = load_raw_nt<WT, E>(w + off[i]);
   }
-  int it = 0;
-  // with WAVES == 4 all waves of the block share the row, so the loop bound is uniform for the barrier
-  for (int64_t row = (int64_t)blockIdx.x * RPB + slot; row < rows; row += step, it++) {
-    const float r = rstd[row];
-    const XT* xr = x + row * xs;
-    const OT* gr = dy + row * dys;
-    XT* dr = dx + row * dxs;
-    float n[NV][E], g[NV][E], a[NV][E];
-    float c = 0.f;
-    // all loads first (out-of-range vectors re-read the row's last one), then the arithmetic
+  // The words of a row are requested raw and converted when the row's turn comes.  With AHEAD the next row is
+  // requested before the arithmetic, the block-wide reduction and the stores of this one, so that a CU's resident
+  // blocks keep about twice the bytes in flight (measured: 3-4 % faster at two vectors per thread, 8 % slower at four).
+  Raw<XT, E> rx[NV], ra[RES ? NV : 1];
+  Raw<OT, E> rg[NV];
+  float r_next = 0.f;
+  auto request = [&](int64_t row) {
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-      const int v = t + TPR * i;
-      const int64_t o = (int64_t)(v < nvec ? v : nvec - 1) * E;
-      load_f_nt<XT, E>(xr + o, n[i]);
-      load_f_nt<OT, E>(gr + o, g[i]);
-      if (dres) load_f_nt<XT, E>(dres + row * drs + o, a[i]);
+      rx[i] = load_raw_nt<XT, E>(x + row * xs + off[i]);
+      rg[i] = load_raw_nt<OT, E>(dy + row * dys + off[i]);
     }
+    if (RES) {
+#pragma unroll
+      for (int i = 0; i < NV; i++) ra[RES ? i : 0] = load_raw_nt<XT, E>(dres + row * drs + off[i]);
+    }
+    r_next = rstd[row];
+  };
+  const int64_t row0 = (int64_t)blockIdx.x * RPB + slot;
+  if (AHEAD && row0 < rows) request(row0);
+  int it = 0;
+  // with WAVES == 4 all waves of the block share the row, so the loop bound is uniform for the barrier
+  for (int64_t row = row0; row < rows; row += step, it++) {
+    if (!AHEAD) request(row);
+    const float r = r_next;
+    XT* dr = dx + row * dxs;
+    float n[NV][E], g[NV][E];
+    float c = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      unpack_f<XT, E>(rx[i], n[i]);
+      unpack_f<OT, E>(rg[i], g[i]);
+    }
+    float a[RES ? NV : 1][E];
+    if (RES) {
+#pragma unroll
+      for (int i = 0; i < NV; i++) unpack_f<XT, E>(ra[RES ? i : 0], a[RES ? i : 0]);
+    }
+    if (AHEAD && row + step < rows) request(row + step);
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       if (t + TPR * i < nvec) {
+        float wv[E];
+        Raw<WT, E> q = rw[i];
+#pragma unroll
+        for (int k = 0; k < (int)(sizeof(q.q) / sizeof(q.q[0])); k++) asm volatile("" : "+v"(q.q[k]));  // (keeps the conversion inside the loop)
+        unpack_f<WT, E>(q, wv);
 #pragma unroll
         for (int e = 0; e < E; e++) {
           const float dyv = g[i][e];
           n[i][e] *= r;
-          g[i][e] = dyv * wv[i][e];
+          g[i][e] = dyv * wv[e];
           c += g[i][e] * n[i][e];
           wacc[i][e] += dyv * round_to<XT>(n[i][e]);
         }
@@ -193,18 +230,16 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_vec(const OT* __restrict__ dy
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       const int v = t + TPR * i;
-      if (v < nvec) {
-        float o[E];
+      float o[E];
 #pragma unroll
-        for (int e = 0; e < E; e++) o[e] = r * (g[i][e] - n[i][e] * c);
-        if (dres) {
-          // fused residual: the gradient that reached h through the residual path joins here, each addend rounded
-          // to the activation dtype first, as autograd's accumulation of two bf16 gradients does
+      for (int e = 0; e < E; e++) o[e] = r * (g[i][e] - n[i][e] * c);
+      if (RES) {
+        // fused residual: the gradient that reached h through the residual path joins here, each addend rounded
+        // to the activation dtype first, as autograd's accumulation of two bf16 gradients does
 #pragma unroll
-          for (int e = 0; e < E; e++) o[e] = round_to<XT>(o[e]) + a[i][e];
-        }
-        store_f_nt<XT, E>(dr + (int64_t)v * E, o);
+        for (int e = 0; e < E; e++) o[e] = round_to<XT>(o[e]) + a[RES ? i : 0][e];
       }
+      if (v < nvec) store_f_nt<XT, E>(dr + (int64_t)v * E, o);
     }
   }
   float* out = ws + ((int64_t)blockIdx.x * RPB + slot) * hidden;
@@ -318,7 +353,7 @@ static int bwd_typed(const void* dy, const void* x, const void* w, const float* 
   constexpr int E = 16 / sizeof(XT);
   const OT* gp = (const OT*)dy; const XT* xp = (const XT*)x; const WT* wp = (const WT*)w; XT* dxp = (XT*)dx;
   const XT* drp = (const XT*)dres;
-  const int parts = rms_parts(rows);
+  const int parts = rms_parts(rows, hidden);
   const int nvec = hidden / E;
   const bool vec = hidden % E == 0 && aligned16(dy) && aligned16(x) && aligned16(w) && aligned16(dx) &&
                    (dys * sizeof(OT)) % 16 == 0 && (xs * sizeof(XT)) % 16 == 0 && (dxs * sizeof(XT)) % 16 == 0 &&
@@ -326,8 +361,14 @@ static int bwd_typed(const void* dy, const void* x, const void* w, const float* 
   if (vec) {
     const dim3 block(256);
 #define TP_RMS_BWD(NV, WAVES)                                                                             \
-  rmsnorm_bwd_vec<XT, WT, OT, NV, WAVES><<<dim3(parts / (4 / WAVES)), block, 0, st>>>(gp, xp, wp, rstd, dxp, ws, rows, \
-                                                                                     hidden, dys, xs, dxs, drp, drs)
+  do {                                                                                                    \
+    if (drp)                                                                                              \
+      rmsnorm_bwd_vec<XT, WT, OT, NV, WAVES, true><<<dim3(parts / (4 / WAVES)), block, 0, st>>>(          \
+          gp, xp, wp, rstd, dxp, ws, rows, hidden, dys, xs, dxs, drp, drs);                               \
+    else                                                                                                  \
+      rmsnorm_bwd_vec<XT, WT, OT, NV, WAVES, false><<<dim3(parts / (4 / WAVES)), block, 0, st>>>(         \
+          gp, xp, wp, rstd, dxp, ws, rows, hidden, dys, xs, dxs, drp, drs);                               \
+  } while (0)
     if (nvec <= 64) TP_RMS_BWD(1, 1);
     else if (nvec <= 128) TP_RMS_BWD(2, 1);
     else if (nvec <= 256) TP_RMS_BWD(1, 4);
@@ -369,7 +410,7 @@ extern "C" int tp_rmsnorm_fwd(const void* x, const void* w, void* y, float* rstd
 
 extern "C" size_t tp_rmsnorm_bwd_workspace_bytes(int64_t rows, int hidden) {
   if (rows <= 0 || hidden <= 0) return 0;
-  return (size_t)rms_parts(rows) * (size_t)hidden * sizeof(float);
+  return (size_t)rms_parts(rows, hidden) * (size_t)hidden * sizeof(float);
 }
 
 extern "C" int tp_rmsnorm_bwd(const void* dy, const void* x, const void* w, const float* rstd, void* dx, void* dw,
@@ -448,7 +489,7 @@ extern "C" int tp_add_rmsnorm_bwd(const void* dy, const void* dh, const void* h,
 // ------------------------------------------------------------------------------------------------
 namespace tp {
 constexpr int RMS_NOALLOC_MAX_HIDDEN = 8192;
-constexpr size_t RMS_NOALLOC_BYTES = (size_t)RMS_MAX_PARTS * RMS_NOALLOC_MAX_HIDDEN * sizeof(float);  // 16 MiB
+constexpr size_t RMS_NOALLOC_BYTES = (size_t)RMS_MIN_PARTS * RMS_NOALLOC_MAX_HIDDEN * sizeof(float);  // 16 MiB
 static __device__ __align__(256) unsigned char scratch[RMS_NOALLOC_BYTES];
 
 constexpr int RMS_MAX_DEVICES = 64;
