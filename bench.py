@@ -388,6 +388,76 @@ def bench_other_configs(dev, iters=5, only=None):
   return res
 
 
+def bench_tiny_config_graph(dev, iters=200):
+  """Configuration 1 (B2, S128, hidden 512, 8 heads of 64, fp32: the reference's own CPU-runnable case) is bound by
+  launches, not by the kernels: the hot path's launches of one layer (RMSNorm, rotary, attention, and their backward)
+  timed launched one by one and replayed as one HIP graph.  Microseconds per pass, inputs resident."""
+  import torch
+
+  from torchprime_amd import _lib
+
+  lib = _lib.load()
+  B, S, H, D = 2, 128, 8, 64
+  hidden, dt = H * D, torch.float32
+  g = torch.Generator(device="cpu").manual_seed(7)
+  rnd = lambda *shape: torch.randn(shape, generator=g, dtype=dt).to(dev)  # noqa: E731
+  x, dy, w = rnd(B * S, hidden), rnd(B * S, hidden), rnd(hidden)
+  y, dx, dw = torch.empty_like(x), torch.empty_like(x), torch.empty_like(w)
+  rstd = torch.empty((B * S,), dtype=torch.float32, device=dev)
+  ws_n = torch.empty((lib.tp_rmsnorm_bwd_workspace_bytes(B * S, hidden) // 4,), dtype=torch.float32, device=dev)
+  q, k, v, do = (rnd(B, S, H, D).transpose(1, 2) for _ in range(4))
+  cos, sin = rnd(1, S, D), rnd(1, S, D)
+  qr, kr, dqr, dkr = (torch.empty_like(q.transpose(1, 2)).transpose(1, 2) for _ in range(4))
+  out, dq, dk, dv = (torch.empty_like(q.transpose(1, 2)).transpose(1, 2) for _ in range(4))
+  lse = torch.empty((B, H, S), dtype=torch.float32, device=dev)
+  ws_a = torch.empty((lib.tp_attn_bwd_workspace_bytes(B, H, S) // 4,), dtype=torch.float32, device=dev)
+  s3, code, sm = _lib.strides3, _lib.dtype_code(dt), 1.0 / math.sqrt(D)
+
+  def rope(a, b, ao, bo, backward):
+    _lib.call("tp_rope_apply", a.data_ptr(), b.data_ptr(), cos.data_ptr(), sin.data_ptr(), None, ao.data_ptr(), bo.data_ptr(),
+              B, H, H, S, D, s3(a), s3(b), s3(ao), s3(bo), 0, cos.stride(1), 0, 0, 0, int(backward), code, _lib.stream_ptr(dev))  # fmt: skip
+
+  def one_pass():
+    st = _lib.stream_ptr(dev)
+    _lib.call("tp_rmsnorm_fwd", x.data_ptr(), w.data_ptr(), y.data_ptr(), rstd.data_ptr(), B * S, hidden, hidden, hidden, 1e-5, code, code, st)
+    rope(q, k, qr, kr, False)
+    _lib.call("tp_attn_fwd", qr.data_ptr(), kr.data_ptr(), v.data_ptr(), None, out.data_ptr(), lse.data_ptr(),
+              B, H, H, S, S, D, D, s3(qr), s3(kr), s3(v), s3(out), sm, 1, code, st)  # fmt: skip
+    _lib.call("tp_attn_bwd", do.data_ptr(), qr.data_ptr(), kr.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), None,
+              dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws_a.data_ptr(), B, H, H, S, S, D, D,
+              s3(do), s3(qr), s3(kr), s3(v), s3(out), s3(dq), s3(dk), s3(dv), sm, 1, code, st)  # fmt: skip
+    rope(dq, dk, dqr, dkr, True)
+    _lib.call("tp_rmsnorm_bwd", dy.data_ptr(), x.data_ptr(), w.data_ptr(), rstd.data_ptr(), dx.data_ptr(), dw.data_ptr(),
+              ws_n.data_ptr(), B * S, hidden, hidden, hidden, hidden, code, code, st)  # fmt: skip
+
+  def timed(fn):
+    fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(iters):
+      fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters * 1e3
+
+  side = torch.cuda.Stream()
+  side.wait_stream(torch.cuda.current_stream())
+  with torch.cuda.stream(side):
+    one_pass()
+  torch.cuda.current_stream().wait_stream(side)
+  torch.cuda.synchronize()
+  eager_us = timed(one_pass)
+  ref = [t.clone() for t in (y, out, dqr, dkr, dv, dx, dw)]
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(graph):
+    one_pass()
+  graph_us = timed(graph.replay)
+  same = all(torch.equal(a, b) for a, b in zip(ref, (y, out, dqr, dkr, dv, dx, dw)))
+  return {"shape": dict(B=B, S=S, heads=H, head_dim=D, hidden=hidden, dtype="f32"), "launched_one_by_one_us": round(eager_us, 1),
+          "hip_graph_replay_us": round(graph_us, 1), "replay_equals_eager": same}  # fmt: skip
+
+
 def cpu_baseline(max_seconds=24.0):
   """The oracle's eager attention (attention.py:151-170 restated), fwd + bwd by autograd, bf16 inputs, on
   this host's cores: one batch element and one kv-head group (4 q heads) of the benchmark workload."""
@@ -456,6 +526,8 @@ def main():
   ap.add_argument("--other-configs", default=None, metavar="NAME[,NAME]",
                   help="run only the named other configurations (llama3_8b_packed_segments, llama3_70b_layer, "
                        "deepseek_v3_heads, or 'all') and print their line: the command the per-configuration kernel traces use")
+  ap.add_argument("--tiny-config", action="store_true",
+                  help="run only the tiny fp32 configuration's launch-by-launch / HIP graph comparison and print its line")
   args = ap.parse_args()
   if args.gpus != 1:
     sys.exit("bench.py measures the one-GPU hot path only: run with --gpus 1 (no multi-GPU path is part of this build)")
@@ -477,10 +549,14 @@ def main():
     names = None if args.other_configs == "all" else args.other_configs.split(",")
     print(json.dumps({"other_configs": bench_other_configs(dev, iters=args.steps, only=names)}))
     return
+  if args.tiny_config:
+    print(json.dumps({"tiny_fp32_config_hip_graph": bench_tiny_config_graph(dev, iters=args.steps)}))
+    return
   ms_per_step, flops_step, roofline, kernels, shape = bench_attention(args, dev)
   extra = None if args.no_extra else bench_norm_rope(dev)
   if extra is not None:
     extra["other_configs"] = bench_other_configs(dev)
+    extra["tiny_fp32_config_hip_graph"] = bench_tiny_config_graph(dev)
   torch.cuda.empty_cache()
   cpu = None if args.no_cpu else cpu_baseline()
   value = flops_step / (ms_per_step * 1e-3) / 1e12
