@@ -29,6 +29,8 @@ reference, which needs torch_xla / jax / omegaconf):
   add_rms_norm, l2_norm     F.rms_norm without a weight, explicit fp64 loops                pinned
   apply_rotary_emb_llama4   complex rotation of adjacent pairs (torch.polar), norm preservation      pinned
   llama_decoder_layer       HuggingFace LlamaDecoderLayer (eager) where importable; composed of pinned parts  pinned
+  llama_for_causal_lm       HuggingFace LlamaForCausalLM (eager; the reference's two test fixtures, with and without
+                            Llama 3.1 rope scaling, at its three input sizes): logits, loss, every gradient      pinned
   llama4_attention          explicit loops (pair rotation, unit-RMS q/k, per-position scale, softmax);
                             = llama_attention with de-interleaved projection rows on rotary layers     pinned
   attn temperature          closed form log(floor((p+1)/f)+1) a + 1 at hand-computed positions       pinned
@@ -319,6 +321,36 @@ def llama_decoder_layer(x, w, n_heads, n_kv_heads, eps, cos, sin, attention_mask
   m = rms_norm(h, w["post_attention_layernorm.weight"], eps)
   m = swiglu(m @ w["mlp.gate_proj.weight"].T, m @ w["mlp.up_proj.weight"].T) @ w["mlp.down_proj.weight"].T
   return h + m
+
+
+def llama_for_causal_lm(input_ids, labels, w, n_heads, n_kv_heads, eps, rope_theta, rope_scaling=None, attention_mask=None):
+  """``LlamaForCausalLM.forward`` (model/llama/model.py:386-400) over ``LlamaModel.forward`` (:333-367): embedding
+  lookup, position ids ``arange(S)`` as floats, one rotary table for all layers, the additive causal mask (times the
+  padding mask when one is given, :354-355), the decoder layers, the final norm, ``lm_head``, logits in fp32 (or the
+  weights' higher precision) and the shifted cross entropy.  ``w``: weights under the reference's state-dict names;
+  ``rope_scaling``: the four Llama 3.1 numbers (factor, low_freq_factor, high_freq_factor, original_context_len) or None.
+  Returns (logits, loss)."""
+  emb = w["model.embed_tokens.weight"]
+  x = emb[input_ids]
+  B, S, hidden = x.shape
+  hd = hidden // n_heads
+  inv_freq = default_rope_frequencies(hd, rope_theta) if rope_scaling is None else llama3_rope_frequencies(hd, rope_theta, *rope_scaling)
+  cos, sin = rotary_cos_sin(inv_freq, torch.arange(S)[None].float(), torch.float32)
+  cos, sin = cos.to(x.dtype), sin.to(x.dtype)
+  mask = causal_additive_mask(S, x.dtype)
+  if attention_mask is not None:
+    mask = mask * attention_mask[:, None, None, :].to(x.dtype)
+  n_layers = 1 + max(int(k.split(".")[2]) for k in w if k.startswith("model.layers."))
+  for i in range(n_layers):
+    pre = f"model.layers.{i}."
+    x = llama_decoder_layer(x, {k[len(pre):]: v for k, v in w.items() if k.startswith(pre)}, n_heads, n_kv_heads, eps, cos, sin, mask)
+  x = rms_norm(x, w["model.norm.weight"], eps)
+  logits = x @ w["lm_head.weight"].T
+  if logits.dtype in (torch.bfloat16, torch.float16):
+    logits = logits.float()
+  if labels is None:
+    return logits, None
+  return logits, cross_entropy_loss(logits, labels, logits.shape[-1])
 
 
 def mixtral_attention(x, wq, wk, wv, wo, n_heads, n_kv_heads, rope_theta, max_position_embeddings, position_ids,

@@ -204,3 +204,15 @@ def test_product_code_does_not_import_the_oracle():
     if fn.endswith(".py"):
       src = open(os.path.join(pkg, fn)).read()
       assert "oracle" not in src, f"{fn} mentions the oracle"
+
+
+def test_rotary_frequencies_stay_fp32_under_a_dtype_cast():
+  """``model.to(torch.bfloat16)`` must not round ``inv_freq`` (8 bits of frequency put the angle at position 300 off
+  by more than a radian for the fast dimensions); device moves still apply."""
+  import torchprime_amd as tpa
+  rot = tpa.LlamaRotaryEmbedding(128, 500000.0)
+  before = rot.inv_freq.clone()
+  holder = torch.nn.Sequential(rot).to(torch.bfloat16)
+  assert holder[0].inv_freq.dtype == torch.float32 and torch.equal(holder[0].inv_freq, before)
+  assert "inv_freq" not in rot.state_dict()
+

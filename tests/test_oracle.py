@@ -370,6 +370,54 @@ def test_llama_decoder_layer_matches_hf_when_available():
   torch.testing.assert_close(got, ref, rtol=1e-4, atol=1e-5)
 
 
+def _hf_llama_fixture(which):
+  """The two models of the reference's own test (torch_xla_models/tests/test_llama.py:26-125): its HuggingFace configs
+  (tests/hf_model_config/meta-llama-3-8b and meta-llama-3.1-405b: rope_theta 5e5, eps 1e-5, no biases, the 405B one
+  with the Llama 3.1 rope scaling) cut down to hidden 512, 8 heads of 64, intermediate 64, one / two layers,
+  vocabulary 128 / 256, seed 42."""
+  from transformers import LlamaConfig
+  from transformers import LlamaForCausalLM as HfLlamaForCausalLM
+  common = dict(hidden_size=512, num_attention_heads=8, num_key_value_heads=8, head_dim=64, intermediate_size=64, rms_norm_eps=1e-5,
+                rope_theta=500000.0, attention_bias=False, attention_dropout=0.0, hidden_act="silu", initializer_range=0.02,
+                tie_word_embeddings=False, use_cache=False)
+  if which == "llama3_8b":
+    cfg = LlamaConfig(vocab_size=128, num_hidden_layers=1, max_position_embeddings=8192, **common)
+    scaling = None
+  else:
+    cfg = LlamaConfig(vocab_size=256, num_hidden_layers=2, max_position_embeddings=131072, mlp_bias=False,
+                      rope_scaling={"factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                                    "original_max_position_embeddings": 8192, "rope_type": "llama3"}, **common)
+    scaling = (8.0, 1.0, 4.0, 8192)
+  cfg._attn_implementation = "eager"
+  torch.manual_seed(42)
+  return HfLlamaForCausalLM(cfg), cfg.vocab_size, scaling
+
+
+@pytest.mark.parametrize("which", ["llama3_8b", "llama3_1_405b"])
+@pytest.mark.parametrize("input_size", [8, 128, 256])
+def test_llama_for_causal_lm_matches_hf_when_available(which, input_size):
+  """The reference's test_forward_and_backward_our_model_against_hf_model with the oracle in the model's place: same
+  fixtures, input sizes, inputs (labels = input ids, a mask of ones) and the reference's tolerances for loss and
+  gradients (1e-4, 1e-5); logits to 2e-6 where the reference (on XLA) asks 1e-6: the softmax scale is a division in
+  the reference and the oracle, a product in HuggingFace."""
+  try:
+    hf, vocab, scaling = _hf_llama_fixture(which)
+    ids = torch.randint(vocab, (2, input_size // 2), generator=torch.Generator().manual_seed(input_size))
+    hf.zero_grad()
+    out = hf(input_ids=ids, labels=ids, attention_mask=torch.ones_like(ids))
+    out.loss.backward()
+  except Exception as e:
+    pytest.skip(f"transformers LlamaForCausalLM not usable here: {e}")
+  w = {k: v.detach().clone().requires_grad_(True) for k, v in hf.state_dict().items()}
+  logits, loss = orc.llama_for_causal_lm(ids, ids, w, 8, 8, 1e-5, 500000.0, scaling, attention_mask=torch.ones_like(ids))
+  loss.backward()
+  torch.testing.assert_close(logits, out.logits, atol=2e-6, rtol=1e-9)
+  torch.testing.assert_close(loss, out.loss, atol=1e-4, rtol=1e-7)
+  for name, p in hf.named_parameters():
+    assert w[name].grad is not None, name
+    torch.testing.assert_close(w[name].grad, p.grad, atol=1e-5, rtol=1e-9, msg=lambda m, name=name: f"{name}: {m}")
+
+
 # ---- the callers ------------------------------------------------------------------------------------------
 def test_mixtral_attention_is_llama_attention_with_gathered_tables():
   B, S, H, Hkv, hd = 2, 12, 4, 2, 16

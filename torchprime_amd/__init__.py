@@ -19,7 +19,8 @@ ops in :mod:`torchprime_amd.ops`); there is no CPU or torch-math fallback.
 
 from . import kernel_utils, ops, parallelism_utils, rope  # noqa: F401
 from .attention import AttentionModule, repeat_kv
-from .blocks import DeepseekV3Attention, Llama4TextAttention, LlamaAttention, LlamaDecoderLayer, MixtralAttention
+from .blocks import (DeepseekV3Attention, Llama4TextAttention, LlamaAttention, LlamaDecoderLayer, LlamaForCausalLM, LlamaModel,
+                     MixtralAttention)
 from .config import Config
 from .kernel_utils import SplashAttentionConfig, splash_attention_jax_wrapper, tpu_splash_attention_jax_call_wrapper
 from .llama4 import (
@@ -47,7 +48,7 @@ __all__ = [
   "SplashAttentionConfig", "LlamaRMSNorm", "MixtralRMSNorm", "DeepseekV3RMSNorm", "RopeScaling",
   "default_rope_frequencies", "llama3_rope_frequencies", "deepseek_v3_rope_init_fn", "LlamaRotaryEmbedding",
   "MixtralRotaryEmbedding", "DeepseekV3RotaryEmbedding", "rotate_half", "apply_rotary_pos_emb",
-  "apply_rotary_pos_emb_interleave", "LlamaAttention", "MixtralAttention", "DeepseekV3Attention", "Llama4TextAttention", "LlamaDecoderLayer", "Config",
+  "apply_rotary_pos_emb_interleave", "LlamaAttention", "MixtralAttention", "DeepseekV3Attention", "Llama4TextAttention", "LlamaDecoderLayer", "LlamaModel", "LlamaForCausalLM", "Config",
   "Llama4TextL2Norm", "Llama4TextRotaryEmbedding", "apply_rotary_emb", "attn_temperature_scales", "apply_attn_temperature",
   "cross_entropy_loss", "LlamaMLP", "add_rms_norm",
 ]  # fmt: skip

@@ -5,6 +5,8 @@ reference's tensor layouts; the projections are stock ``nn.Linear`` (GEMMs are o
 * LlamaAttention        torchprime/torch_xla_models/model/llama/model.py:156-238
 * MixtralAttention      model/mixtral/model.py:159-243
 * DeepseekV3Attention   model/deepseek_v3/model.py:341-455
+* LlamaDecoderLayer, LlamaModel, LlamaForCausalLM   model/llama/model.py:241-400 (the callers of the path, one and
+  two levels up: embedding, the layers, final norm, ``lm_head`` and the shifted cross entropy)
 """
 
 from __future__ import annotations
@@ -225,3 +227,109 @@ class LlamaDecoderLayer(nn.Module):
     hidden_states = self.mlp(hidden_states)
     return residual + hidden_states
 
+
+
+  def forward_deferred(self, x, residual, attention_mask=None, position_ids=None, position_embeddings=None):
+    """The same layer with the residual adds at its two ends left to the neighbours.  The layer's input is
+    ``x + residual`` (``residual`` None: ``x`` itself), added inside the first norm's kernel; the return value is
+    ``(mlp_out, h)`` whose sum is the layer's output, for the next layer (or the model's final norm) to add the same
+    way.  Same values as ``forward``, bit for bit, with one pass over the hidden states less per layer."""
+    from .norm import add_rms_norm
+
+    if residual is None:
+      residual, hidden_states = x, self.input_layernorm(x)
+    else:
+      hidden_states, residual = add_rms_norm(x, residual, self.input_layernorm)
+    hidden_states = self.self_attn(hidden_states, position_embeddings, attention_mask, position_ids)
+    hidden_states, residual = add_rms_norm(hidden_states, residual, self.post_attention_layernorm)
+    return self.mlp(hidden_states), residual
+
+
+class LlamaModel(nn.Module):
+  """model/llama/model.py:300-367: embedding, the decoder layers, the final norm; position ids ``arange(S)`` as
+  floats, one rotary table for all layers.  Parameter names are the reference's (and HuggingFace's), so
+  ``load_state_dict(hf_model.state_dict())`` works as in the reference's tests.
+
+  The (S, S) additive causal mask of :347-355 is only consumed by the eager branch of ``AttentionModule`` (the kernel
+  branches are causal by themselves), so it is built only for ``attention_kernel=None``, and kept per sequence length
+  while no padding mask multiplies it."""
+
+  def __init__(self, config):
+    super().__init__()
+    from .norm import LlamaRMSNorm
+    from .rope import RopeScaling
+    from .rotary import LlamaRotaryEmbedding
+
+    self.config = config
+    self.vocab_size = config.vocab_size
+    self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size)
+    self.layers = nn.ModuleList(LlamaDecoderLayer(config, i) for i in range(config.num_hidden_layers))
+    self.norm = LlamaRMSNorm(config.hidden_size, eps=config.rms_norm_eps)
+    rope_scaling = config.get("rope_scaling", None)
+    if rope_scaling is not None:
+      rope_scaling = RopeScaling(**dict(rope_scaling))
+    self.rope_theta = config.rope_theta
+    self.rotary_emb = LlamaRotaryEmbedding(
+      head_dim=config.hidden_size // config.num_attention_heads, rope_theta=config.rope_theta, scaling=rope_scaling
+    )
+    self._causal_masks: dict = {}
+
+  def _mask(self, seq_length, attention_mask, device):
+    if self.config.attention_kernel in ("splash_attention", "flash_attention"):
+      return None  # never read on those branches (attention.py:121-123, 144-150)
+    key = (seq_length, str(device))
+    causal = self._causal_masks.get(key)
+    if causal is None:
+      if len(self._causal_masks) > 4:
+        self._causal_masks.clear()
+      causal = torch.triu(torch.full((seq_length, seq_length), float("-inf"), device=device), diagonal=1)[None, None]
+      self._causal_masks[key] = causal
+    if attention_mask is not None:
+      causal = causal * attention_mask[:, None, None, :]
+    return causal
+
+  def forward(self, input_ids, attention_mask=None):
+    from .norm import add_rms_norm
+
+    inputs_embeds = self.embed_tokens(input_ids)
+    seq_length = inputs_embeds.size(1)
+    position_ids = torch.arange(seq_length, device=inputs_embeds.device).unsqueeze(0).float()
+    causal_mask = self._mask(seq_length, attention_mask, inputs_embeds.device)
+    position_embeddings = self.rotary_emb(inputs_embeds, position_ids)
+    x, residual = inputs_embeds, None
+    for layer in self.layers:
+      x, residual = layer.forward_deferred(x, residual, attention_mask=causal_mask, position_ids=position_ids,
+                                           position_embeddings=position_embeddings)
+    if residual is None:
+      return self.norm(x)
+    return add_rms_norm(x, residual, self.norm)[0]
+
+
+class LlamaForCausalLM(nn.Module):
+  """model/llama/model.py:370-400: the model, ``lm_head``, logits in fp32 and the shifted cross entropy; returns
+  ``(logits, loss)`` (loss None without labels).  Linear and embedding weights start from a normal distribution of
+  standard deviation ``config.initializer_range``, biases from zero (model/base_causal_lm.py:38-54)."""
+
+  def __init__(self, config):
+    super().__init__()
+    self.config = config
+    self.model = LlamaModel(config)
+    self.vocab_size = config.vocab_size
+    self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
+    self.apply(self._init_weights)
+
+  def _init_weights(self, module):
+    std = self.config.initializer_range
+    if isinstance(module, (nn.Linear, nn.Embedding)):
+      module.weight.data.normal_(mean=0.0, std=std)
+      if getattr(module, "bias", None) is not None:
+        module.bias.data.zero_()
+
+  def forward(self, input_ids, labels=None, attention_mask=None):
+    from .loss import cross_entropy_loss
+
+    hidden_states = self.model(input_ids=input_ids, attention_mask=attention_mask)
+    logits = self.lm_head(hidden_states).float()
+    if labels is None:
+      return logits, None
+    return logits, cross_entropy_loss(logits, labels=labels, vocab_size=self.config.vocab_size)

@@ -21,7 +21,21 @@ from . import _lib, ops
 from .rope import RopeScaling, deepseek_v3_rope_init_fn, llama3_rope_frequencies
 
 
-class LlamaRotaryEmbedding(nn.Module):
+class _Fp32Frequencies(nn.Module):
+  """``inv_freq`` stays fp32 whatever the module is cast to.  The reference builds its models under a default dtype
+  and never casts them, so its fp32 buffer (rope/rope.py:25-39 ends in ``.float()``) is never rounded; a
+  ``model.to(torch.bfloat16)`` would round the frequencies to 8 bits and turn the angles at a few hundred positions
+  wrong by several percent.  Device moves apply as usual."""
+
+  def _apply(self, fn, recurse=True):
+    kept = self.inv_freq
+    super()._apply(fn, recurse)
+    if self.inv_freq.dtype != kept.dtype:
+      self.inv_freq = kept.to(self.inv_freq.device)
+    return self
+
+
+class LlamaRotaryEmbedding(_Fp32Frequencies):
   inv_freq: torch.Tensor
 
   def __init__(self, head_dim, rope_theta, scaling: RopeScaling | None = None):
@@ -36,7 +50,7 @@ class LlamaRotaryEmbedding(nn.Module):
     return ops.rope_table(self.inv_freq, position_ids, 1.0, x.dtype)
 
 
-class DeepseekV3RotaryEmbedding(nn.Module):
+class DeepseekV3RotaryEmbedding(_Fp32Frequencies):
   inv_freq: torch.Tensor
 
   def __init__(self, config):
