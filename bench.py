@@ -458,6 +458,51 @@ def bench_tiny_config_graph(dev, iters=200):
           "hip_graph_replay_us": round(graph_us, 1), "replay_equals_eager": same}  # fmt: skip
 
 
+def bench_decoder_layer(dev, iters=5):
+  """One Llama-3-8B decoder layer (hidden 4096, 32 q / 8 kv heads of 128, MLP 14336; B4, S8192, bf16), forward and
+  backward through autograd: the package's modules around stock ``nn.Linear`` GEMMs.  Context for the headline
+  number: what share of a layer's step the hot path is.  Milliseconds per forward + backward, inputs resident."""
+  import torch
+
+  import torchprime_amd as tpa
+
+  B, S, hidden, H, Hkv, inter = 4, 8192, 4096, 32, 8, 14336
+  cfg = tpa.Config(attention_kernel="splash_attention", hidden_size=hidden, num_attention_heads=H, num_key_value_heads=Hkv,
+                   intermediate_size=inter, rms_norm_eps=1e-5, hidden_act="silu", attention_dropout=False, attention_bias=False)
+  torch.manual_seed(0)
+  layer = tpa.LlamaDecoderLayer(cfg, 0).to(dev).to(torch.bfloat16)
+  for p in layer.parameters():
+    if p.dim() == 2:
+      torch.nn.init.normal_(p, std=0.02)
+  g = torch.Generator(device="cpu").manual_seed(3)
+  x = torch.randn((B, S, hidden), generator=g).to(torch.bfloat16).to(dev).requires_grad_(True)
+  do = torch.randn((B, S, hidden), generator=g).to(torch.bfloat16).to(dev)
+  rot = tpa.LlamaRotaryEmbedding(hidden // H, 500000.0).to(dev)
+  pe = rot(x, torch.arange(S, device=dev)[None].float())
+
+  def step():
+    layer.zero_grad(set_to_none=True)
+    x.grad = None
+    y = layer(x, position_embeddings=pe)
+    y.backward(do)
+
+  step()
+  torch.cuda.synchronize()
+  a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+  a.record()
+  for _ in range(iters):
+    step()
+  b.record()
+  torch.cuda.synchronize()
+  ms = a.elapsed_time(b) / iters
+  params = sum(p.numel() for p in layer.parameters() if p.dim() == 2)
+  gemm_flops = 6.0 * B * S * params
+  attn_flops = 6.0 * B * H * S * S * (hidden // H)
+  return {"shape": dict(B=B, S=S, hidden=hidden, q_heads=H, kv_heads=Hkv, head_dim=hidden // H, intermediate=inter, dtype="bf16"),
+          "fwd_bwd_ms": round(ms, 3), "gemm_TFLOP": round(gemm_flops / 1e12, 2), "attention_TFLOP_counted": round(attn_flops / 1e12, 2),
+          "layer_TFLOPs": round((gemm_flops + attn_flops) / (ms * 1e-3) / 1e12, 1)}  # fmt: skip
+
+
 def cpu_baseline(max_seconds=24.0):
   """The oracle's eager attention (attention.py:151-170 restated), fwd + bwd by autograd, bf16 inputs, on
   this host's cores: one batch element and one kv-head group (4 q heads) of the benchmark workload."""
@@ -526,6 +571,8 @@ def main():
   ap.add_argument("--other-configs", default=None, metavar="NAME[,NAME]",
                   help="run only the named other configurations (llama3_8b_packed_segments, llama3_70b_layer, "
                        "deepseek_v3_heads, or 'all') and print their line: the command the per-configuration kernel traces use")
+  ap.add_argument("--decoder-layer", action="store_true",
+                  help="run only one Llama-3-8B decoder layer forward + backward (GEMMs included) and print its line")
   ap.add_argument("--tiny-config", action="store_true",
                   help="run only the tiny fp32 configuration's launch-by-launch / HIP graph comparison and print its line")
   args = ap.parse_args()
@@ -548,6 +595,9 @@ def main():
   if args.other_configs:
     names = None if args.other_configs == "all" else args.other_configs.split(",")
     print(json.dumps({"other_configs": bench_other_configs(dev, iters=args.steps, only=names)}))
+    return
+  if args.decoder_layer:
+    print(json.dumps({"llama3_8b_decoder_layer": bench_decoder_layer(dev, iters=args.steps)}))
     return
   if args.tiny_config:
     print(json.dumps({"tiny_fp32_config_hip_graph": bench_tiny_config_graph(dev, iters=args.steps)}))
