@@ -60,7 +60,8 @@ def test_c_abi_validates_arguments_before_launching():
   assert lib.tp_rmsnorm_bwd_workspace_bytes(32768, 4096) == 512 * 4096 * 4
   assert lib.tp_rmsnorm_bwd_workspace_bytes(10, 64) == 12 * 64 * 4
   assert lib.tp_rmsnorm_bwd_workspace_bytes(32768, 512) == 4096 * 512 * 4   # short rows: more partial rows
-  assert lib.tp_rmsnorm_bwd_workspace_bytes(32768, 1536) == 1024 * 1536 * 4
+  assert lib.tp_rmsnorm_bwd_workspace_bytes(32768, 1536) == 2048 * 1536 * 4
+  assert lib.tp_rmsnorm_bwd_workspace_bytes(32768, 2048) == 1024 * 2048 * 4
   assert lib.tp_rmsnorm_bwd_workspace_bytes(32768, 16384) == 512 * 16384 * 4
   assert lib.tp_attn_bwd_workspace_bytes(4, 32, 8192) == 2 * 4 * 32 * 8192 * 4
 

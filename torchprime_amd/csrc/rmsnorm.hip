@@ -13,13 +13,13 @@ namespace tp {
 
 // Partial dw rows written by the backward (a multiple of 4).  The row-walking kernel is fastest with about 512
 // blocks of four waves (two per CU) at two 16-byte vectors per thread and about twice that at one vector, and
-// slower with more (measured at 512 ... 4096 partial rows over hidden 512 ... 5120): so the count follows the
-// row length, the largest power of two within 2^21 / hidden, between 512 and 4096.
+// slower with more (measured at 512 ... 4096 partial rows over hidden 512 ... 5120).  Rows short enough for a
+// single wave go four to a block, so they need four times the partial rows for the same number of blocks: the
+// count follows the row length.
 constexpr int RMS_MIN_PARTS = 512, RMS_MAX_PARTS = 4096;
 
 static inline int rms_parts(int64_t rows, int hidden) {
-  int cap = RMS_MAX_PARTS;
-  while (cap > RMS_MIN_PARTS && (int64_t)cap * hidden > (1 << 21)) cap >>= 1;
+  const int cap = hidden <= 512 ? 4096 : hidden <= 1536 ? 2048 : hidden <= 2048 ? 1024 : RMS_MIN_PARTS;
   const int64_t p = (rows + 3) / 4 * 4;
   return (int)(p < cap ? p : cap);
 }
@@ -141,16 +141,17 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_generic(const XT* __restrict_
 // go straight to one partial row per (block, row slot): no atomics, no cross-thread fold.
 // ------------------------------------------------------------------------------------------------
 template <typename XT, typename WT, typename OT, int NV, int WAVES, bool RES>
-__global__ __launch_bounds__(256) void rmsnorm_bwd_vec(const OT* __restrict__ dy, const XT* __restrict__ x,
+__global__ __launch_bounds__(64 * (WAVES > 4 ? WAVES : 4)) void rmsnorm_bwd_vec(const OT* __restrict__ dy, const XT* __restrict__ x,
                                                        const WT* __restrict__ w, const float* __restrict__ rstd,
                                                        XT* __restrict__ dx, float* __restrict__ ws, int64_t rows,
                                                        int hidden, int64_t dys, int64_t xs, int64_t dxs,
                                                        const XT* __restrict__ dres, int64_t drs) {
   constexpr int E = 16 / sizeof(XT);
-  constexpr int RPB = 4 / WAVES, TPR = 64 * WAVES;
+  constexpr int BW = WAVES > 4 ? WAVES : 4;  // waves per block: four, or all the waves of a long row
+  constexpr int RPB = BW / WAVES, TPR = 64 * WAVES;
   // Rows are requested one ahead while a thread's share of a row is small enough for both rows to sit in registers.
-  constexpr bool AHEAD = NV <= 2;
-  __shared__ float red[2][4];
+  constexpr bool AHEAD = NV <= 2 && !(WAVES == 16 && RES && sizeof(OT) > sizeof(XT));  // (that one would spill at 128 registers)
+  __shared__ float red[2][BW];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int slot = wave / WAVES;
   const int t = (wave % WAVES) * 64 + lane;
@@ -335,6 +336,7 @@ static int fwd_typed(const void* x, const void* w, void* y, float* rstd, int64_t
     // 512 threads, or a wave per row)
     if (nvec <= 64) TP_RMS_FWD(1, 1);
     else if (nvec <= 128) TP_RMS_FWD(2, 1);
+    else if (nvec <= 192) TP_RMS_FWD(3, 1);  // (a 256-thread row would leave a quarter of its lanes idle: hidden 1536)
     else if (nvec <= 256) TP_RMS_FWD(1, 4);
     else if (nvec <= 512) TP_RMS_FWD(2, 4);
     else if (nvec <= 1024) TP_RMS_FWD(4, 4);
@@ -359,22 +361,28 @@ static int bwd_typed(const void* dy, const void* x, const void* w, const float* 
                    (dys * sizeof(OT)) % 16 == 0 && (xs * sizeof(XT)) % 16 == 0 && (dxs * sizeof(XT)) % 16 == 0 &&
                    aligned16(dres) && (drs * sizeof(XT)) % 16 == 0 && nvec <= 256 * 8;
   if (vec) {
-    const dim3 block(256);
 #define TP_RMS_BWD(NV, WAVES)                                                                             \
   do {                                                                                                    \
+    constexpr int BW = WAVES > 4 ? WAVES : 4;                                                             \
+    const dim3 grid(parts / (BW / WAVES)), block(64 * BW);                                                \
     if (drp)                                                                                              \
-      rmsnorm_bwd_vec<XT, WT, OT, NV, WAVES, true><<<dim3(parts / (4 / WAVES)), block, 0, st>>>(          \
+      rmsnorm_bwd_vec<XT, WT, OT, NV, WAVES, true><<<grid, block, 0, st>>>(                               \
           gp, xp, wp, rstd, dxp, ws, rows, hidden, dys, xs, dxs, drp, drs);                               \
     else                                                                                                  \
-      rmsnorm_bwd_vec<XT, WT, OT, NV, WAVES, false><<<dim3(parts / (4 / WAVES)), block, 0, st>>>(         \
+      rmsnorm_bwd_vec<XT, WT, OT, NV, WAVES, false><<<grid, block, 0, st>>>(                              \
           gp, xp, wp, rstd, dxp, ws, rows, hidden, dys, xs, dxs, drp, drs);                               \
   } while (0)
+    // Measured per shape (same box, 128 Mi elements): up to two vectors per thread a row spreads over more waves
+    // rather than more vectors per thread - 16 waves for rows beyond 1024 vectors (hidden 16384 in bf16: 178 -> 151 us
+    // against four waves of eight vectors), eight for the fused-residual form beyond 512 (hidden 7168: 202 -> 180 us);
+    // the plain form is faster with four waves of four vectors there (141 against 149 us).
     if (nvec <= 64) TP_RMS_BWD(1, 1);
     else if (nvec <= 128) TP_RMS_BWD(2, 1);
+    else if (nvec <= 192) TP_RMS_BWD(3, 1);
     else if (nvec <= 256) TP_RMS_BWD(1, 4);
     else if (nvec <= 512) TP_RMS_BWD(2, 4);
-    else if (nvec <= 1024) TP_RMS_BWD(4, 4);
-    else TP_RMS_BWD(8, 4);
+    else if (nvec <= 1024) { if (drp) TP_RMS_BWD(2, 8); else TP_RMS_BWD(4, 4); }
+    else TP_RMS_BWD(2, 16);
 #undef TP_RMS_BWD
   } else {
     rmsnorm_bwd_dx_generic<XT, WT, OT><<<dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st>>>(gp, xp, wp, rstd, dxp, rows,
