@@ -17,6 +17,7 @@ DEV = "cuda"
 # ---- residual add + RMSNorm -----------------------------------------------------------------------------------
 @pytest.mark.parametrize("shape,dtype,wdtype", [((2, 128, 512), torch.float32, torch.float32), ((2, 256, 4096), torch.bfloat16, torch.bfloat16),
                                                 ((3, 50, 8192), torch.bfloat16, torch.bfloat16), ((5, 333), torch.float16, torch.float16),
+                                                ((1, 33, 16384), torch.bfloat16, torch.bfloat16), ((2, 17, 16384), torch.bfloat16, torch.float32), ((2, 700, 7168), torch.bfloat16, torch.bfloat16),
                                                 ((4, 7, 1536), torch.bfloat16, torch.float32)])
 def test_add_rmsnorm_fwd_bwd(shape, dtype, wdtype):
   hidden, eps = shape[-1], 1e-5

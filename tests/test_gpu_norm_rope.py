@@ -21,6 +21,11 @@ DEV = "cuda"
     ((1, 512, 1536), torch.bfloat16, torch.bfloat16, 1e-6),   # DeepSeek q latent
     ((1, 512, 512), torch.bfloat16, torch.bfloat16, 1e-6),    # DeepSeek kv latent
     ((3, 7, 4096), torch.bfloat16, torch.float32, 1e-5),      # fp32 weight: result promotes to fp32
+    ((1, 40, 16384), torch.bfloat16, torch.bfloat16, 1e-5),   # Llama-3.1-405B hidden: 16 waves per row in the backward
+    ((2, 9, 16384), torch.bfloat16, torch.float32, 1e-5),     # the same with fp32 weight and dy
+    ((1, 70, 7168), torch.bfloat16, torch.bfloat16, 1e-6),    # DeepSeek-V3 hidden
+    ((3, 900, 5120), torch.float16, torch.float16, 1e-5),     # Llama-4 hidden; more rows than partial dw rows
+    ((1, 5000, 1024), torch.bfloat16, torch.bfloat16, 1e-5),  # single-wave rows, more rows than partial dw rows
     ((5, 333), torch.float16, torch.float16, 1e-6),           # ragged hidden: scalar path
     ((4, 3, 100), torch.float32, torch.float32, 1e-6),
     ((0, 512), torch.bfloat16, torch.bfloat16, 1e-6),         # empty
