@@ -265,4 +265,71 @@ __device__ __forceinline__ u32x2 transpose_col(const u32x4 (&r)[4], int j) {
   return o;
 }
 
+// ------------------------------------------------------------------------------------------------
+// row-major tiles filled by buffer loads that write LDS directly (no staging registers)
+// ------------------------------------------------------------------------------------------------
+// One such load moves 16 bytes per lane to LDS address  base + 16 * lane: where a chunk lands is fixed by
+// the lane, which global chunk it carries is free.  A tile of 64 rows x D 16-bit elements is stored
+// densely (row r at r * D*2) with the 16-byte chunks of a row XOR-swizzled by the row, so that the MFMA
+// fragment reads (lanes = consecutive rows, same logical chunk) fall into different banks.
+template <int D>
+struct DmaTile {
+  static constexpr int CPR = D / 8;              // 16-byte chunks per row
+  static constexpr int ROWB = D * 2;             // bytes per row
+  static constexpr int BYTES = 64 * ROWB;
+  static constexpr int PER_WAVE = CPR / 4;       // load instructions per wave for one tile (4 waves)
+  static_assert(CPR % 8 == 0, "head dim must be a multiple of 64");
+  static __device__ __forceinline__ int swz(int row) { return (CPR % 16 == 0) ? (row & 15) : ((row >> 1) & 7); }
+  // byte offset of logical chunk c of a row
+  static __device__ __forceinline__ int off(int row, int c) { return row * ROWB + ((c ^ swz(row)) << 4); }
+
+  unsigned vo[PER_WAVE];  // global byte offset (inside a tile) of the chunk this lane carries, per instruction
+
+  __device__ __forceinline__ void init(int64_t row_stride, int wave, int lane) {
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; i++) {
+      const int slot = (wave * PER_WAVE + i) * 64 + lane;  // 16-byte slot inside the LDS tile
+      const int row = slot / CPR, c = (slot % CPR) ^ swz(row);
+      vo[i] = (unsigned)((row * row_stride + c * 8) * 2);
+    }
+  }
+  // Issue this wave's share of the tile.  The loads are written as assembly on purpose: the compiler
+  // orders every later LDS read behind an LDS-writing load it knows of, which would stall the tile being
+  // computed on the one in flight; the caller waits (s_waitcnt 0 + barrier) before the tile is read.
+  // Rows past the end of the tensor (offset >= rs.z) arrive as zeros.
+  template <int I>
+  __device__ __forceinline__ void issue_one(u32x4 rs, unsigned tile_byte_offset, unsigned char* lds_tile, int wave) const {
+    const unsigned dst = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(lds_tile + (wave * PER_WAVE + I) * 1024));
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(dst), "v"(vo[I]), "s"(rs), "s"(tile_byte_offset) : "memory", "m0");
+  }
+  // same, with the wave's first LDS destination given as a scalar byte address (keeps the address
+  // arithmetic on the scalar unit)
+  template <int I>
+  __device__ __forceinline__ void issue_one_at(u32x4 rs, unsigned tile_byte_offset, unsigned wave_dst) const {
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(wave_dst + I * 1024), "v"(vo[I]), "s"(rs), "s"(tile_byte_offset) : "memory", "m0");
+  }
+  __device__ __forceinline__ void issue(u32x4 rs, unsigned tile_byte_offset, unsigned char* lds_tile, int wave) const {
+    tile_byte_offset = __builtin_amdgcn_readfirstlane(tile_byte_offset);
+    if constexpr (PER_WAVE > 0) issue_one<0>(rs, tile_byte_offset, lds_tile, wave);
+    if constexpr (PER_WAVE > 1) issue_one<1>(rs, tile_byte_offset, lds_tile, wave);
+    if constexpr (PER_WAVE > 2) issue_one<2>(rs, tile_byte_offset, lds_tile, wave);
+    if constexpr (PER_WAVE > 3) issue_one<3>(rs, tile_byte_offset, lds_tile, wave);
+    if constexpr (PER_WAVE > 4) issue_one<4>(rs, tile_byte_offset, lds_tile, wave);
+    if constexpr (PER_WAVE > 5) issue_one<5>(rs, tile_byte_offset, lds_tile, wave);
+    static_assert(PER_WAVE <= 6, "head dim above 192");
+  }
+};
+// buffer resource words for the assembly loads: base, stride 0, size in bytes, raw-buffer flags
+__device__ __forceinline__ u32x4 make_rsrc_words(const void* base, unsigned bytes) {
+  const unsigned long long p = (unsigned long long)base;
+  u32x4 r;
+  r.x = __builtin_amdgcn_readfirstlane((unsigned)p);
+  r.y = __builtin_amdgcn_readfirstlane((unsigned)(p >> 32));
+  r.z = __builtin_amdgcn_readfirstlane(bytes);
+  r.w = 0x00020000u;
+  return r;
+}
+
 }  // namespace tp

@@ -34,21 +34,31 @@ struct FwdArgs {
   MaskExt mx;
 };
 
-// Two workgroups per CU (256 registers per lane) where the kernel fits them; the 192-wide heads and the 128-wide
-// non-causal variants (run-time buffer index, mask extensions) need more and take one workgroup per CU instead of
-// spilling a hundred registers.
-template <int DQK, bool CAUSAL>
-constexpr int fwd_blocks_per_cu() { return (DQK > 128 || (DQK == 128 && !CAUSAL)) ? 1 : 2; }
+// Two workgroups per CU (256 registers per lane) where the kernel fits them; the non-causal variants at head dims of
+// 128 and more (run-time buffer index, mask extensions) and the 192-wide heads with segment ids need more registers
+// or LDS and take one workgroup per CU instead of spilling a hundred registers.
+template <int DQK, bool CAUSAL, bool SEG>
+constexpr int fwd_blocks_per_cu() { return (DQK >= 128 && !CAUSAL) || (DQK > 128 && SEG) ? 1 : 2; }
+// The causal kernels fill their K tiles with buffer loads that write LDS directly: no staging registers for K, no
+// LDS stores for it, and dense swizzled rows instead of padded ones.  For the 192-wide heads that is what lets two
+// workgroups share a CU: 254 registers instead of 289, and two double-buffered tile sets of 81920 bytes fill the
+// CU's 160 KB exactly (forward at 128 heads x 4096 rows: 1.16 -> 0.89 ms).  At head dim 128 it is worth 3 %.
+// (The head-dim-128 kernel with segment ids keeps the staged path: its run-time buffer index would turn the
+// swizzled fragment offsets into eight more live registers, which it does not have.)
+template <int DQK, bool CAUSAL, bool SEG>
+constexpr bool fwd_k_dma() { return CAUSAL && (DQK > 128 || (DQK == 128 && !SEG)); }
 
 template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
-__global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_fwd_kernel(const FwdArgs a) {
+__global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void attn_fwd_kernel(const FwdArgs a) {
   typedef typename MT<T>::v8 v8;
   constexpr int BN = 64;              // kv rows per LDS tile, processed as two halves of 32
   constexpr int BM = 128;             // q rows per workgroup, 32 per wave
   constexpr int KSTEPS = DQK / 16;    // MFMA k-steps over the qk head dim
   constexpr int DVB = DV / 32;        // 32-column blocks of the v head dim
   typedef RowTile<DQK> KT;
-  constexpr int K_BYTES = BN * KT::STRIDE;
+  typedef DmaTile<DQK> KD;
+  constexpr bool KDMA = fwd_k_dma<DQK, CAUSAL, SEG>();
+  constexpr int K_BYTES = KDMA ? KD::BYTES : BN * KT::STRIDE;
   constexpr int V_BYTES = DV * TrTile64::ROW_BYTES;
   constexpr int SEG_BYTES = SEG ? BN * 4 : 0;
   constexpr int BUF_BYTES = K_BYTES + V_BYTES + SEG_BYTES;
@@ -61,7 +71,8 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
   constexpr int V_AT = STATIC_BUF ? 2 * K_BYTES : K_BYTES, V_STEP = STATIC_BUF ? V_BYTES : BUF_BYTES;
   constexpr int SEG_AT = STATIC_BUF ? 2 * (K_BYTES + V_BYTES) : K_BYTES + V_BYTES, SEG_STEP = STATIC_BUF ? SEG_BYTES : BUF_BYTES;
   constexpr int KCH = DQK / 8;                      // 16-byte chunks per K row
-  constexpr int K_ITEMS = BN * KCH / 256;           // chunks per thread
+  constexpr int K_ITEMS = BN * KCH / 256;           // chunks per thread (KDMA: LDS-writing loads per wave)
+  static_assert(!KDMA || K_ITEMS == KD::PER_WAVE, "one load instruction per staged chunk");
   constexpr int V_TOT = (DV / 8) * (BN / 4);        // 4x8 blocks of the V tile
   constexpr int V_ITEMS = (V_TOT + 255) / 256;
   static_assert(BN * KCH % 256 == 0, "K tile must split evenly over 256 threads");
@@ -166,11 +177,19 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
   const rsrc_t krs = make_rsrc(kb, span_bytes(Skv, a.ks[2], DQK));
   const rsrc_t vrs = make_rsrc(vb, span_bytes(Skv, a.vs[2], DV));
   const unsigned k_tile_bytes = (unsigned)(BN * a.ks[2] * 2), v_tile_bytes = (unsigned)(BN * a.vs[2] * 2);
-  unsigned kvo[K_ITEMS], vvo[V_ITEMS][4];
+  constexpr int K_REGS = KDMA ? 1 : K_ITEMS;
+  unsigned kvo[K_REGS], vvo[V_ITEMS][4];
+  KD kdma;
+  u32x4 krw = {0u, 0u, 0u, 0u};
+  if constexpr (KDMA) {
+    kdma.init(a.ks[2], wave, lane);
+    krw = make_rsrc_words(kb, span_bytes(Skv, a.ks[2], DQK));
+  } else {
 #pragma unroll
-  for (int i = 0; i < K_ITEMS; i++) {
-    const int item = tid + 256 * i;
-    kvo[i] = (unsigned)(((item / KCH) * a.ks[2] + (item % KCH) * 8) * 2);
+    for (int i = 0; i < K_ITEMS; i++) {
+      const int item = tid + 256 * i;
+      kvo[i] = (unsigned)(((item / KCH) * a.ks[2] + (item % KCH) * 8) * 2);
+    }
   }
 #pragma unroll
   for (int i = 0; i < V_ITEMS; i++) {
@@ -179,13 +198,18 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
 #pragma unroll
     for (int ii = 0; ii < 4; ii++) vvo[i][ii] = (unsigned)(((4 * rq + ii) * a.vs[2] + c8 * 8) * 2);
   }
-  u32x4 kreg[K_ITEMS];
+  u32x4 kreg[K_REGS];
   u32x4 vreg[V_ITEMS][4];
   int sreg = 0;
-  auto load_tile = [&](int t) {
+  // (KDMA: the K tile goes straight into buffer `kbuf`, which nobody reads before the next barrier)
+  auto load_tile = [&](int t, int kbuf) {
     const unsigned kso = (unsigned)t * k_tile_bytes, vso = (unsigned)t * v_tile_bytes;
+    if constexpr (KDMA) {
+      kdma.issue(krw, kso, smem + K_AT + kbuf * K_STEP, wave);
+    } else {
 #pragma unroll
-    for (int i = 0; i < K_ITEMS; i++) kreg[i] = buf_load16(krs, kvo[i], kso);
+      for (int i = 0; i < K_ITEMS; i++) kreg[i] = buf_load16(krs, kvo[i], kso);
+    }
 #pragma unroll
     for (int i = 0; i < V_ITEMS; i++) {
       if (tid + 256 * i < V_TOT) {
@@ -196,10 +220,11 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
     if (has_seg && tid < BN) sreg = segb[min(t * BN + tid, Skv - 1)];
   };
   // the same loads one at a time (piece P of K_ITEMS + 4 V_ITEMS), for issuing between MFMAs
-  auto load_piece = [&](auto Pc, int t) {
+  auto load_piece = [&](auto Pc, int t, int kbuf) {
     constexpr int p = decltype(Pc)::value;
     if constexpr (p < K_ITEMS) {
-      kreg[p] = buf_load16(krs, kvo[p], (unsigned)t * k_tile_bytes);
+      if constexpr (KDMA) kdma.template issue_one<p>(krw, __builtin_amdgcn_readfirstlane((unsigned)t * k_tile_bytes), smem + K_AT + kbuf * K_STEP, wave);
+      else kreg[p] = buf_load16(krs, kvo[p], (unsigned)t * k_tile_bytes);
     } else {
       constexpr int i = (p - K_ITEMS) / 4, ii = (p - K_ITEMS) % 4;
       if (tid + 256 * i < V_TOT) vreg[i][ii] = buf_load16(vrs, vvo[i][ii], (unsigned)t * v_tile_bytes);
@@ -208,10 +233,12 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
   auto store_tile = [&](int buf) {
     unsigned char* kl = smem + K_AT + buf * K_STEP;
     unsigned char* vl = kl + (V_AT - K_AT) + buf * (V_STEP - K_STEP);
+    if constexpr (!KDMA) {
 #pragma unroll
-    for (int i = 0; i < K_ITEMS; i++) {
-      const int item = tid + 256 * i;
-      *(u32x4*)(kl + KT::off(item / KCH, (item % KCH) * 8)) = kreg[i];
+      for (int i = 0; i < K_ITEMS; i++) {
+        const int item = tid + 256 * i;
+        *(u32x4*)(kl + KT::off(item / KCH, (item % KCH) * 8)) = kreg[i];
+      }
     }
 #pragma unroll
     for (int i = 0; i < V_ITEMS; i++) {
@@ -234,6 +261,8 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
       }
     }
     if (SEG && tid < BN) ((int*)(smem + SEG_AT + buf * SEG_STEP))[tid] = sreg;
+    // the LDS-writing K loads are outside the compiler's bookkeeping: they have landed before the barrier that follows
+    if constexpr (KDMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
 
   // ---- accumulators: O^T blocks, running max (log2 units), per-lane partial row sum
@@ -294,6 +323,17 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
 #pragma unroll
     for (int m = 0; m < 4; m++) tb[m] = (unsigned)TrTile64::chunk_off(ln, m, g) + v_at;
   }
+  // KDMA: per-lane offsets of the K fragments in the swizzled tile.  Row hf*32 + ln, chunk 2 ks + g lies at
+  // (hf*32 + ln) * ROWB + ((2 ks + g) ^ swz) * 16.  With 24 chunks per row the swizzle has three bits,
+  // (ln >> 1) & 7, so only the low three bits of the chunk depend on the lane: four offsets (ks & 3), the rest is an
+  // immediate.  With 16 chunks per row it has four bits (ln & 15): one offset per k-step.
+  constexpr bool KSWZ3 = KD::CPR % 16 != 0;
+  constexpr int NKFO = KDMA ? (KSWZ3 ? 4 : KSTEPS) : 1;
+  unsigned kfo[NKFO];
+  if constexpr (KDMA) {
+#pragma unroll
+    for (int j = 0; j < NKFO; j++) kfo[j] = (unsigned)(ln * KD::ROWB + (((2 * j + g) ^ KD::swz(ln)) << 4));
+  }
   auto tile_body = [&](auto masked_c, auto BUFc, int buf_rt, int t, bool has_next, int t_next) {
     constexpr bool MASKED = decltype(masked_c)::value;
     // the buffer index: a constant, or (-1) the run-time one
@@ -345,7 +385,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
       }
     };
     constexpr int S1 = KSTEPS, PV0 = 2 * KSTEPS, PV1 = PV0 + 2 * DVB, NS = PV1 + 2 * DVB;
-    constexpr int AHEAD = STATIC_BUF ? 5 : 3, NF = AHEAD + 1;  // (the plain causal kernel has registers left for a deeper ring)
+    constexpr int AHEAD = (STATIC_BUF && DQK <= 128) ? 5 : 3, NF = AHEAD + 1;  // (the plain causal kernel up to head dim 128 has registers left for a deeper ring; seven slots gain nothing)
     v8 fr[NF];
     f32x16 s[2];
     v8 pf[2][2];
@@ -355,7 +395,8 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
       constexpr int i = decltype(I)::value;
       if constexpr (i < PV0) {
         constexpr int hf = i / KSTEPS, ks = i % KSTEPS;
-        return *(const v8*)(kl + KT::off(hf * 32 + ln, 16 * ks + 8 * g));
+        if constexpr (KDMA) return *(const v8*)(kl + kfo[KSWZ3 ? (ks & 3) : ks] + hf * 32 * KD::ROWB + (KSWZ3 ? 128 * (ks >> 2) : 0));
+        else return *(const v8*)(kl + KT::off(hf * 32 + ln, 16 * ks + 8 * g));
       } else {
         constexpr int hf = (i - PV0) / (2 * DVB), j = (i - PV0) % (2 * DVB), kk = j / DVB, d = j % DVB;
         if constexpr (STATIC_BUF) return *(const v8*)(vl + tb[(2 * hf + kk) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
@@ -405,7 +446,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
       if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
       mma(I, fr[i % NF]);
       // the next tile's loads, one per slot (past the last tile they re-read the last one: no branch here)
-      if constexpr (i < K_ITEMS + 4 * V_ITEMS) load_piece(I, t_next);
+      if constexpr (i < K_ITEMS + 4 * V_ITEMS) load_piece(I, t_next, buf ^ 1);
       if constexpr (i == 0) {
         if (has_seg && tid < BN) sreg = segb[min(t_next * BN + tid, Skv - 1)];
       }
@@ -439,7 +480,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
   // loop over its distinct values
   auto tile_at = [&](int i) { return SEG ? __builtin_amdgcn_readfirstlane(active[i]) : i; };
   if (nact > 0) {
-    load_tile(tile_at(0));
+    load_tile(tile_at(0), 0);
     store_tile(0);
   }
   // Everything loaded so far (the Q fragments above all) has landed before the loop starts.  Without
@@ -468,7 +509,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
     }
     if (skip) {
       if (has_next) {
-        load_tile(t_next);
+        load_tile(t_next, buf ^ 1);
         store_tile(buf ^ 1);
       }
     } else if (need_mask) {
@@ -508,7 +549,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
       typedef std::integral_constant<int, -1> RT;
       if (skip) {
         if (has_next) {
-          load_tile(t_next);
+          load_tile(t_next, buf ^ 1);
           store_tile(buf ^ 1);
         }
       } else if (need_mask) {
@@ -520,6 +561,9 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
     }
   }
 
+  // (the last tile's body issues its loads without a successor to wait for them: no LDS-writing load may be in flight
+  // when the workgroup's LDS is handed to the next one)
+  if constexpr (KDMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   // ---- epilogue: normalise, write O (row = query, 4 consecutive v-dims per store) and LSE
   T* ob = (T*)a.out + b * a.os[0] + h * a.os[1];
   float* lb = a.lse + ((int64_t)b * a.Hq + h) * Sq;
@@ -547,7 +591,8 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL>())) void attn_
 template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
 static int launch_fwd(const FwdArgs& a, int B, hipStream_t st) {
   constexpr int BN = 64, BM = 128;
-  constexpr int BUF = BN * RowTile<DQK>::STRIDE + DV * TrTile64::ROW_BYTES + (SEG ? BN * 4 : 0);
+  constexpr int K_TILE = fwd_k_dma<DQK, CAUSAL, SEG>() ? DmaTile<DQK>::BYTES : BN * RowTile<DQK>::STRIDE;
+  constexpr int BUF = K_TILE + DV * TrTile64::ROW_BYTES + (SEG ? BN * 4 : 0);
   const int ntiles_max = (a.Skv + BN - 1) / BN;
   const size_t smem = 2 * (size_t)BUF + (SEG ? (size_t)(3 * ntiles_max + 16) * 4 : 0);
   TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_fwd: Skv=%d needs %zu bytes of LDS (max 163840)", a.Skv, smem);
