@@ -8,10 +8,11 @@
 //     one query column and 16 key rows per 32x32 block: row max / sum / rescale are per-lane scalars
 //     (one half-wave exchange per tile), and exp(S^T) converted to 16 bit is already the B operand of
 //     O^T += V^T P^T - P never goes through LDS;
-//   * Q fragments stay in registers for the whole KV loop; K tiles are staged row-major in LDS, V tiles
-//     are transposed while being written to LDS so both are read with conflict-free 16-byte loads;
-//   * the next K/V tile is fetched from HBM into registers while the current one is being multiplied
-//     (LDS double buffer, one barrier per tile);
+//   * Q fragments stay in registers for the whole KV loop; K tiles are row-major in LDS (dense rows, 16-byte
+//     chunks XOR-swizzled by the row), V tiles are transposed while being written to LDS, so both are read with
+//     conflict-free 16-byte loads;
+//   * the next tile is fetched while the current one is being multiplied: K by buffer loads that write LDS
+//     directly, V from HBM into registers (its transposition needs them); LDS double buffer, one barrier per tile;
 //   * causal: the KV loop ends at the diagonal, element masks only on tiles that straddle it;
 //     segments: per-tile [min,max] of the ids is computed once per workgroup, tiles whose id range
 //     misses the query rows' range are skipped, element compares only where ranges are not one id.
@@ -39,14 +40,12 @@ struct FwdArgs {
 // or LDS and take one workgroup per CU instead of spilling a hundred registers.
 template <int DQK, bool CAUSAL, bool SEG>
 constexpr int fwd_blocks_per_cu() { return (DQK >= 128 && !CAUSAL) || (DQK > 128 && SEG) ? 1 : 2; }
-// The causal kernels fill their K tiles with buffer loads that write LDS directly: no staging registers for K, no
-// LDS stores for it, and dense swizzled rows instead of padded ones.  For the 192-wide heads that is what lets two
+// K tiles are filled by buffer loads that write LDS directly (DmaTile): no staging registers for K, no LDS stores
+// for it, and dense swizzled rows instead of padded ones.  For the causal 192-wide heads that is what lets two
 // workgroups share a CU: 254 registers instead of 289, and two double-buffered tile sets of 81920 bytes fill the
-// CU's 160 KB exactly (forward at 128 heads x 4096 rows: 1.16 -> 0.89 ms).  At head dim 128 it is worth 3 %.
-// (The head-dim-128 kernel with segment ids keeps the staged path: its run-time buffer index would turn the
-// swizzled fragment offsets into eight more live registers, which it does not have.)
-template <int DQK, bool CAUSAL, bool SEG>
-constexpr bool fwd_k_dma() { return CAUSAL && (DQK > 128 || (DQK == 128 && !SEG)); }
+// CU's 160 KB exactly (forward at 128 heads x 4096 rows: 1.16 -> 0.89 ms).  The other variants gain 2-7 % over staging
+// K through registers (same-box A/B: head dim 64 causal 2.6 %, 128 causal 3 %, 128 causal with segment ids 7 % - it
+// also stopped spilling -, 128 and 192 non-causal 3.4 and 3.9 %).
 
 template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
 __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void attn_fwd_kernel(const FwdArgs a) {
@@ -55,10 +54,8 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   constexpr int BM = 128;             // q rows per workgroup, 32 per wave
   constexpr int KSTEPS = DQK / 16;    // MFMA k-steps over the qk head dim
   constexpr int DVB = DV / 32;        // 32-column blocks of the v head dim
-  typedef RowTile<DQK> KT;
   typedef DmaTile<DQK> KD;
-  constexpr bool KDMA = fwd_k_dma<DQK, CAUSAL, SEG>();
-  constexpr int K_BYTES = KDMA ? KD::BYTES : BN * KT::STRIDE;
+  constexpr int K_BYTES = KD::BYTES;
   constexpr int V_BYTES = DV * TrTile64::ROW_BYTES;
   constexpr int SEG_BYTES = SEG ? BN * 4 : 0;
   constexpr int BUF_BYTES = K_BYTES + V_BYTES + SEG_BYTES;
@@ -70,12 +67,9 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   constexpr int K_AT = 0, K_STEP = STATIC_BUF ? K_BYTES : BUF_BYTES;
   constexpr int V_AT = STATIC_BUF ? 2 * K_BYTES : K_BYTES, V_STEP = STATIC_BUF ? V_BYTES : BUF_BYTES;
   constexpr int SEG_AT = STATIC_BUF ? 2 * (K_BYTES + V_BYTES) : K_BYTES + V_BYTES, SEG_STEP = STATIC_BUF ? SEG_BYTES : BUF_BYTES;
-  constexpr int KCH = DQK / 8;                      // 16-byte chunks per K row
-  constexpr int K_ITEMS = BN * KCH / 256;           // chunks per thread (KDMA: LDS-writing loads per wave)
-  static_assert(!KDMA || K_ITEMS == KD::PER_WAVE, "one load instruction per staged chunk");
+  constexpr int K_ITEMS = KD::PER_WAVE;             // LDS-writing K loads per wave and tile
   constexpr int V_TOT = (DV / 8) * (BN / 4);        // 4x8 blocks of the V tile
   constexpr int V_ITEMS = (V_TOT + 255) / 256;
-  static_assert(BN * KCH % 256 == 0, "K tile must split evenly over 256 threads");
 
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -174,23 +168,12 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   // V row quads are dealt to threads so that the 32 lanes whose transposed 8-byte stores are served
   // together fall into 32 different bank pairs
   auto v_quad = [](int rqi) { return (rqi & ~3) | ((rqi & 1) << 1) | ((rqi >> 1) & 1); };
-  const rsrc_t krs = make_rsrc(kb, span_bytes(Skv, a.ks[2], DQK));
   const rsrc_t vrs = make_rsrc(vb, span_bytes(Skv, a.vs[2], DV));
   const unsigned k_tile_bytes = (unsigned)(BN * a.ks[2] * 2), v_tile_bytes = (unsigned)(BN * a.vs[2] * 2);
-  constexpr int K_REGS = KDMA ? 1 : K_ITEMS;
-  unsigned kvo[K_REGS], vvo[V_ITEMS][4];
+  unsigned vvo[V_ITEMS][4];
   KD kdma;
-  u32x4 krw = {0u, 0u, 0u, 0u};
-  if constexpr (KDMA) {
-    kdma.init(a.ks[2], wave, lane);
-    krw = make_rsrc_words(kb, span_bytes(Skv, a.ks[2], DQK));
-  } else {
-#pragma unroll
-    for (int i = 0; i < K_ITEMS; i++) {
-      const int item = tid + 256 * i;
-      kvo[i] = (unsigned)(((item / KCH) * a.ks[2] + (item % KCH) * 8) * 2);
-    }
-  }
+  kdma.init(a.ks[2], wave, lane);
+  const u32x4 krw = make_rsrc_words(kb, span_bytes(Skv, a.ks[2], DQK));
 #pragma unroll
   for (int i = 0; i < V_ITEMS; i++) {
     const int item = tid + 256 * i;
@@ -198,18 +181,12 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
 #pragma unroll
     for (int ii = 0; ii < 4; ii++) vvo[i][ii] = (unsigned)(((4 * rq + ii) * a.vs[2] + c8 * 8) * 2);
   }
-  u32x4 kreg[K_REGS];
   u32x4 vreg[V_ITEMS][4];
   int sreg = 0;
-  // (KDMA: the K tile goes straight into buffer `kbuf`, which nobody reads before the next barrier)
+  // the K tile goes straight into buffer `kbuf`, which nobody reads before the next barrier
   auto load_tile = [&](int t, int kbuf) {
     const unsigned kso = (unsigned)t * k_tile_bytes, vso = (unsigned)t * v_tile_bytes;
-    if constexpr (KDMA) {
-      kdma.issue(krw, kso, smem + K_AT + kbuf * K_STEP, wave);
-    } else {
-#pragma unroll
-      for (int i = 0; i < K_ITEMS; i++) kreg[i] = buf_load16(krs, kvo[i], kso);
-    }
+    kdma.issue(krw, kso, smem + K_AT + kbuf * K_STEP, wave);
 #pragma unroll
     for (int i = 0; i < V_ITEMS; i++) {
       if (tid + 256 * i < V_TOT) {
@@ -223,8 +200,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   auto load_piece = [&](auto Pc, int t, int kbuf) {
     constexpr int p = decltype(Pc)::value;
     if constexpr (p < K_ITEMS) {
-      if constexpr (KDMA) kdma.template issue_one<p>(krw, __builtin_amdgcn_readfirstlane((unsigned)t * k_tile_bytes), smem + K_AT + kbuf * K_STEP, wave);
-      else kreg[p] = buf_load16(krs, kvo[p], (unsigned)t * k_tile_bytes);
+      kdma.template issue_one<p>(krw, __builtin_amdgcn_readfirstlane((unsigned)t * k_tile_bytes), smem + K_AT + kbuf * K_STEP, wave);
     } else {
       constexpr int i = (p - K_ITEMS) / 4, ii = (p - K_ITEMS) % 4;
       if (tid + 256 * i < V_TOT) vreg[i][ii] = buf_load16(vrs, vvo[i][ii], (unsigned)t * v_tile_bytes);
@@ -233,13 +209,6 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   auto store_tile = [&](int buf) {
     unsigned char* kl = smem + K_AT + buf * K_STEP;
     unsigned char* vl = kl + (V_AT - K_AT) + buf * (V_STEP - K_STEP);
-    if constexpr (!KDMA) {
-#pragma unroll
-      for (int i = 0; i < K_ITEMS; i++) {
-        const int item = tid + 256 * i;
-        *(u32x4*)(kl + KT::off(item / KCH, (item % KCH) * 8)) = kreg[i];
-      }
-    }
 #pragma unroll
     for (int i = 0; i < V_ITEMS; i++) {
       const int item = tid + 256 * i;
@@ -262,7 +231,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
     }
     if (SEG && tid < BN) ((int*)(smem + SEG_AT + buf * SEG_STEP))[tid] = sreg;
     // the LDS-writing K loads are outside the compiler's bookkeeping: they have landed before the barrier that follows
-    if constexpr (KDMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
 
   // ---- accumulators: O^T blocks, running max (log2 units), per-lane partial row sum
@@ -323,17 +292,15 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
 #pragma unroll
     for (int m = 0; m < 4; m++) tb[m] = (unsigned)TrTile64::chunk_off(ln, m, g) + v_at;
   }
-  // KDMA: per-lane offsets of the K fragments in the swizzled tile.  Row hf*32 + ln, chunk 2 ks + g lies at
+  // Per-lane offsets of the K fragments in the swizzled tile.  Row hf*32 + ln, chunk 2 ks + g lies at
   // (hf*32 + ln) * ROWB + ((2 ks + g) ^ swz) * 16.  With 24 chunks per row the swizzle has three bits,
   // (ln >> 1) & 7, so only the low three bits of the chunk depend on the lane: four offsets (ks & 3), the rest is an
   // immediate.  With 16 chunks per row it has four bits (ln & 15): one offset per k-step.
   constexpr bool KSWZ3 = KD::CPR % 16 != 0;
-  constexpr int NKFO = KDMA ? (KSWZ3 ? 4 : KSTEPS) : 1;
+  constexpr int NKFO = KSWZ3 ? (KSTEPS < 4 ? KSTEPS : 4) : KSTEPS;
   unsigned kfo[NKFO];
-  if constexpr (KDMA) {
 #pragma unroll
-    for (int j = 0; j < NKFO; j++) kfo[j] = (unsigned)(ln * KD::ROWB + (((2 * j + g) ^ KD::swz(ln)) << 4));
-  }
+  for (int j = 0; j < NKFO; j++) kfo[j] = (unsigned)(ln * KD::ROWB + (((2 * j + g) ^ KD::swz(ln)) << 4));
   auto tile_body = [&](auto masked_c, auto BUFc, int buf_rt, int t, bool has_next, int t_next) {
     constexpr bool MASKED = decltype(masked_c)::value;
     // the buffer index: a constant, or (-1) the run-time one
@@ -395,8 +362,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
       constexpr int i = decltype(I)::value;
       if constexpr (i < PV0) {
         constexpr int hf = i / KSTEPS, ks = i % KSTEPS;
-        if constexpr (KDMA) return *(const v8*)(kl + kfo[KSWZ3 ? (ks & 3) : ks] + hf * 32 * KD::ROWB + (KSWZ3 ? 128 * (ks >> 2) : 0));
-        else return *(const v8*)(kl + KT::off(hf * 32 + ln, 16 * ks + 8 * g));
+        return *(const v8*)(kl + kfo[KSWZ3 ? (ks & 3) : ks] + hf * 32 * KD::ROWB + (KSWZ3 ? 128 * (ks >> 2) : 0));
       } else {
         constexpr int hf = (i - PV0) / (2 * DVB), j = (i - PV0) % (2 * DVB), kk = j / DVB, d = j % DVB;
         if constexpr (STATIC_BUF) return *(const v8*)(vl + tb[(2 * hf + kk) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
@@ -563,7 +529,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
 
   // (the last tile's body issues its loads without a successor to wait for them: no LDS-writing load may be in flight
   // when the workgroup's LDS is handed to the next one)
-  if constexpr (KDMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   // ---- epilogue: normalise, write O (row = query, 4 consecutive v-dims per store) and LSE
   T* ob = (T*)a.out + b * a.os[0] + h * a.os[1];
   float* lb = a.lse + ((int64_t)b * a.Hq + h) * Sq;
@@ -591,8 +557,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
 template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
 static int launch_fwd(const FwdArgs& a, int B, hipStream_t st) {
   constexpr int BN = 64, BM = 128;
-  constexpr int K_TILE = fwd_k_dma<DQK, CAUSAL, SEG>() ? DmaTile<DQK>::BYTES : BN * RowTile<DQK>::STRIDE;
-  constexpr int BUF = K_TILE + DV * TrTile64::ROW_BYTES + (SEG ? BN * 4 : 0);
+  constexpr int BUF = DmaTile<DQK>::BYTES + DV * TrTile64::ROW_BYTES + (SEG ? BN * 4 : 0);
   const int ntiles_max = (a.Skv + BN - 1) / BN;
   const size_t smem = 2 * (size_t)BUF + (SEG ? (size_t)(3 * ntiles_max + 16) * 4 : 0);
   TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_fwd: Skv=%d needs %zu bytes of LDS (max 163840)", a.Skv, smem);
