@@ -607,6 +607,8 @@ def main():
   if extra is not None:
     extra["other_configs"] = bench_other_configs(dev)
     extra["tiny_fp32_config_hip_graph"] = bench_tiny_config_graph(dev)
+    extra["llama3_8b_decoder_layer"] = bench_decoder_layer(dev, iters=3)
+    torch.cuda.empty_cache()
   torch.cuda.empty_cache()
   cpu = None if args.no_cpu else cpu_baseline()
   value = flops_step / (ms_per_step * 1e-3) / 1e12
