@@ -17,10 +17,12 @@ DEV = "cuda"
 
 
 def _check(B, Hq, Hkv, S, D, dtype=torch.bfloat16, causal=True, seg=None, window=None, soft_cap=None, q_positions=None,
-           causal_offset=0, Skv=None, seed=0):
+           causal_offset=0, Skv=None, seed=0, Dv=None):
   Skv = S if Skv is None else Skv
-  q, k, v, do = (heads_view(B, h, s_, D, seed + i, dtype) for i, (h, s_) in enumerate(((Hq, S), (Hkv, Skv), (Hkv, Skv), (Hq, S))))
-  sm = 1.0 / math.sqrt(D)
+  Dv = D if Dv is None else Dv
+  q, k, v, do = (heads_view(B, h, s_, d, seed + i, dtype)
+                 for i, (h, s_, d) in enumerate(((Hq, S, D), (Hkv, Skv, D), (Hkv, Skv, Dv), (Hq, S, Dv))))
+  sm = 1.0 / math.sqrt(Dv)
   qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
   qp = None if q_positions is None else torch.as_tensor(q_positions).to(DEV)
   out = tpa.ops.attention(qd, kd, vd, None if seg is None else seg.to(DEV), sm, causal, window=window, soft_cap=soft_cap,
@@ -52,6 +54,20 @@ def test_sliding_window_with_segments_and_ragged_kv(dtype):
 def test_soft_cap_fwd_bwd(D, causal):
   _check(1, 4, 2, 300, D, causal=causal, soft_cap=2.0)       # caps visibly: |logit| reaches ~3 with N(0,1) inputs
   _check(1, 2, 2, 200, D, causal=causal, soft_cap=30.0, window=(64, 64) if not causal else None)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mask_extensions_with_wide_heads(dtype):
+  """qk head dim 192, v head dim 128 (the single-buffer dK/dV path and the four-wave dQ kernel): window, window with
+  segment ids and a ragged kv length, soft cap, and the load-balanced causal order."""
+  _check(1, 4, 4, 330, 192, dtype=dtype, causal=True, window=(70, 70), Dv=128, seed=3)
+  _check(1, 4, 2, 200, 192, dtype=dtype, causal=False, window=(50, 20), Dv=128, Skv=300, seed=4)
+  seg, _ = packed_segment_ids(2, 260, 10, 120, seed=5)
+  _check(2, 4, 4, 260, 192, dtype=dtype, causal=True, seg=seg, window=(40, 40), Dv=128, seed=6)
+  _check(1, 4, 2, 300, 192, dtype=dtype, causal=True, soft_cap=2.0, Dv=128, seed=7)
+  _check(1, 2, 2, 200, 192, dtype=dtype, causal=False, soft_cap=5.0, window=(64, 64), Dv=128, seed=8)
+  mask = pu.LoadBalancedCausalMask(shape=(256, 256), cp_size=4)
+  _check(1, 4, 4, 256, 192, dtype=dtype, causal=True, q_positions=mask.q_sequence, Dv=128, seed=9)
 
 
 @pytest.mark.parametrize("cp_size,D", [(2, 128), (4, 128), (4, 64)])

@@ -890,7 +890,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       const float* lsel = (const float*)(rows_base + (it & 1) * ROW_BYTES);
       const float* deltal = lsel + BMQ;
       const int* segl = (const int*)(deltal + BMQ);
+      const int* posl = segl + BMQ;  // query positions of the tile's rows (mask extensions)
       f32x16 sacc[QB], dpacc[QB];
+      float fcap[GEN ? QB : 1][16];  // soft cap: 1 - tanh^2 of every score, kept from P to dS
       v8 pfr[BMQ / 16];
       u32x4 trd[4];
       // transposition of this tile in 3 reads and 12 double stores, placed at steps T0.. of part 1
@@ -920,7 +922,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         f32x4 l4[NCH / 4];
         // masked tiles: one bit per query row of the tile for this lane's kv column (see the pipelined path)
         unsigned rowbits[2] = {0u, 0u};
-        if constexpr (MASKED) {
+        const bool by_bits = MASKED && !(GEN && ext);  // (the mask extensions are evaluated element by element)
+        if (MASKED && by_bits) {
           const int lo_r = CAUSAL ? max(kvcol - qi0, 0) : 0;
           const int hi_r = kvcol < Skv ? min(Sq - qi0, BMQ) : 0;
           unsigned long long m = 0ull;
@@ -958,9 +961,27 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
 #pragma unroll
             for (int idx = 2 * k; idx < 2 * k + 2; idx++) {
               const int qb = idx / 16, v = idx % 16, m = idx / 4, e = idx % 4;
-              float pv = fast_exp2(__builtin_fmaf(sacc[qb][v], c, l4[m][e]));
-              if constexpr (MASKED)
-                pv = __uint_as_float(__float_as_uint(pv) & (unsigned)__builtin_amdgcn_sbfe((int)rowbits[qb], 8 * (v / 4) + e, 1));
+              float sval = sacc[qb][v];
+              if constexpr (GEN && MASKED) {
+                if (capped) {
+                  const float th = fast_tanh(sval * a.mx.cap_in);
+                  fcap[GEN ? qb : 0][v] = 1.f - th * th;
+                  sval = a.mx.cap_out * th;
+                }
+              }
+              float pv = fast_exp2(__builtin_fmaf(sval, c, l4[m][e]));
+              if constexpr (MASKED) {
+                if (by_bits) {
+                  pv = __uint_as_float(__float_as_uint(pv) & (unsigned)__builtin_amdgcn_sbfe((int)rowbits[qb], 8 * (v / 4) + e, 1));
+                } else {
+                  const int r = qb * 32 + 8 * (v / 4) + 4 * g + e;
+                  const int qrow = qi0 + r;
+                  bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || !has_seg || segl[r] == segk);
+                  const int qp = has_pos ? posl[r] : qrow;
+                  ok = ok && kvcol >= qp - a.mx.lo_off && kvcol <= qp + a.mx.hi_off;
+                  pv = ok ? pv : 0.f;
+                }
+              }
               asm volatile("" : "+v"(pv));  // keeps the computation in this step
               sacc[qb][v] = pv;
             }
@@ -1022,6 +1043,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
             for (int idx = 2 * i; idx < 2 * i + 2; idx++) {
               const int qb = idx / 16, v = idx % 16, m = idx / 4, e = idx % 4;
               float dsv = sacc[qb][v] * (dpacc[qb][v] + d4[m][e]);
+              if constexpr (GEN) {
+                if (mode == 2 && capped) dsv *= fcap[GEN ? qb : 0][v];  // derivative of the capped score
+              }
               asm volatile("" : "+v"(dsv));
               dpacc[qb][v] = dsv;
             }
@@ -1736,8 +1760,7 @@ template <typename T, int DQK, int DV>
 static int dispatch_bwd(const BwdArgs& a, int causal, hipStream_t st, void* const* ev) {
   if (a.mx.on) {
     // mask extensions: the general instantiation (causality is part of the band then)
-    if constexpr (DQK == DV && DQK <= 128) return launch_bwd<T, DQK, DV, false, true>(a, st, ev);
-    else TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_attn_bwd_masked: windows, soft cap and query positions are built for head dims 64 and 128");
+    return launch_bwd<T, DQK, DV, false, true>(a, st, ev);
   }
   if (causal) {
     if (a.seg) return launch_bwd<T, DQK, DV, true, true>(a, st, ev);

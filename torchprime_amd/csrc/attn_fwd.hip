@@ -577,8 +577,7 @@ template <typename T, int DQK, int DV>
 static int dispatch_fwd(const FwdArgs& a, int B, int causal, hipStream_t st) {
   if (a.mx.on) {
     // mask extensions: the general instantiation (causality is part of the band then)
-    if constexpr (DQK == DV && DQK <= 128) return launch_fwd<T, DQK, DV, false, true>(a, B, st);
-    else TP_REQUIRE(false, TP_ERR_UNSUPPORTED, "tp_attn_fwd_masked: windows, soft cap and query positions are built for head dims 64 and 128");
+    return launch_fwd<T, DQK, DV, false, true>(a, B, st);
   }
   if (causal) {
     if (a.seg) return launch_fwd<T, DQK, DV, true, true>(a, B, st);
