@@ -185,7 +185,7 @@ int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, const void* v
  *   logits_soft_cap > 0: scores become cap * tanh(sm_scale * q.k / cap) before masking and softmax
  *                   (attn_logits_soft_cap, kernel_utils.py:292); <= 0: none
  * Tiles outside every row's band are skipped.  Rows left without any allowed key give out = 0, lse = -inf and
- * zero gradients.  bf16 / fp16, head dims as tp_attn_fwd.  With none of the extensions in use the calls are
+ * zero gradients.  Dtypes and head dims as tp_attn_fwd.  With none of the extensions in use the calls are
  * tp_attn_fwd / tp_attn_bwd.
  * ---------------------------------------------------------------------------------------------- */
 int tp_attn_fwd_masked(const void* q, const void* k, const void* v, const int32_t* seg,

@@ -344,9 +344,9 @@ def test_unsupported_inputs_raise():
   q64 = torch.zeros((1, 2, 16, 64), dtype=torch.float64, device=DEV)
   with pytest.raises(TypeError):
     tpa.ops.attention(q64, q64, q64)
-  q32 = torch.zeros((1, 2, 16, 64), dtype=torch.float32, device=DEV)
-  with pytest.raises(NotImplementedError):  # the mask extensions are built for 16-bit tensors
-    tpa.ops.attention(q32, q32, q32, window=(4, 0))
+  q32 = torch.zeros((1, 2, 16, 192), dtype=torch.float32, device=DEV)
+  with pytest.raises(NotImplementedError):  # fp32 tensors: head dims 64 and 128
+    tpa.ops.attention(q32, q32, q32[..., :128])
   with pytest.raises(RuntimeError):
     tpa.ops.attention(q.cpu(), q.cpu(), q.cpu())
 

@@ -70,6 +70,37 @@ def test_mask_extensions_with_wide_heads(dtype):
   _check(1, 4, 4, 256, 192, dtype=dtype, causal=True, q_positions=mask.q_sequence, Dv=128, seed=9)
 
 
+@pytest.mark.parametrize("D", [64, 128])
+def test_mask_extensions_fp32(D):
+  """fp32 tensors through the fp32 kernels: window, window with segment ids and a ragged kv length, soft cap, the
+  load-balanced causal order; fp32 class of tolerance against the fp64 oracle."""
+  def check32(B, Hq, Hkv, S, seed, Skv=None, **kw):
+    Skv_ = S if Skv is None else Skv
+    q, k, v, do = (heads_view(B, h, s_, D, seed + i, torch.float32) for i, (h, s_) in enumerate(((Hq, S), (Hkv, Skv_), (Hkv, Skv_), (Hq, S))))
+    sm = 1.0 / math.sqrt(D)
+    qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    seg = kw.pop("seg", None)
+    causal = kw.pop("causal", True)
+    qp = kw.get("q_positions")
+    out = tpa.ops.attention(qd, kd, vd, None if seg is None else seg.to(DEV), sm, causal, window=kw.get("window"), soft_cap=kw.get("soft_cap"),
+                            q_positions=None if qp is None else torch.as_tensor(qp).to(DEV), causal_offset=kw.get("causal_offset", 0))
+    assert out.dtype == torch.float32
+    out.backward(do.to(DEV))
+    o_ref, dq_ref, dk_ref, dv_ref = orc.attention_grads_ref(q, k, v, do, seg, causal, sm, torch.float64, **kw)
+    for got, ref, name in ((out, o_ref, "out"), (qd.grad, dq_ref, "dq"), (kd.grad, dk_ref, "dk"), (vd.grad, dv_ref, "dv")):
+      assert_close(got, ref, name, max_abs=2e-5 * max(1.0, ref.abs().max().item()), rel_l2=2e-5)
+
+  check32(2, 4, 2, 200, 1, window=(50, 50))
+  check32(1, 2, 1, 130, 2, causal=False, window=(50, 20), Skv=260)
+  seg, _ = packed_segment_ids(2, 160, 10, 80, seed=3)
+  check32(2, 4, 4, 160, 3, seg=seg, window=(30, 30))
+  check32(1, 4, 2, 150, 4, soft_cap=2.0)
+  check32(1, 2, 2, 140, 5, causal=False, soft_cap=5.0, window=(40, 40))
+  mask = pu.LoadBalancedCausalMask(shape=(128, 128), cp_size=4)
+  check32(1, 4, 2, 128, 6, q_positions=mask.q_sequence)
+  check32(1, 2, 2, 128, 7, q_positions=mask.q_sequence, causal_offset=5)
+
+
 @pytest.mark.parametrize("cp_size,D", [(2, 128), (4, 128), (4, 64)])
 def test_load_balanced_causal_mask_fwd_bwd(cp_size, D):
   S = 512

@@ -51,7 +51,6 @@ def test_c_abi_validates_arguments_before_launching():
   assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 128, 128, z3, z3, z3, z3, 0.1, 1, 7, None) == -2  # unknown dtype
   s192, s128 = _lib._I64x3(8 * 2 * 192, 192, 2 * 192), _lib._I64x3(8 * 2 * 128, 128, 2 * 128)
   assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 192, 128, s192, s192, s128, s128, 0.1, 1, 2, None) == -2  # fp32: dims 64 / 128 only
-  assert lib.tp_attn_fwd_masked(p, p, p, None, None, p, p, 1, 2, 2, 8, 8, 128, 128, s128, s128, s128, s128, 0.1, 1, 0, 4, -1, 0.0, 2, None) == -2  # window in fp32
   assert lib.tp_attn_fwd(p, p, p, None, p, p, 1, 2, 2, 8, 8, 128, 128, z3, z3, z3, z3, -1.0, 1, 0, None) == -1  # scale
   assert lib.tp_attn_fwd(p, p, p, p, p, p, 1, 2, 2, 8, 16, 128, 128, z3, z3, z3, z3, 0.1, 1, 0, None) == -1  # seg, Sq != Skv
   assert lib.tp_rope_apply(p, None, p, p, None, p, None, 1, 2, 0, 8, 24, z3, z3, z3, z3, 0, 24, 0, 0, 0, 0, 0, None) == -2  # D % 16

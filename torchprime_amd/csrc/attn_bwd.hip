@@ -1811,7 +1811,8 @@ namespace tp {
 int attn_bwd_f32(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
                  const int32_t* seg, void* dq, void* dk, void* dv, float* ws, int B, int Hq, int Hkv, int Sq, int Skv, int Dqk,
                  int Dv, const int64_t* dos, const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
-                 const int64_t* dqs, const int64_t* dks, const int64_t* dvs, float sm_scale, int causal, hipStream_t st);
+                 const int64_t* dqs, const int64_t* dks, const int64_t* dvs, float sm_scale, int causal, hipStream_t st,
+                 const MaskExt& mx);
 }  // namespace tp
 
 static int attn_bwd_impl(const void* dout, const void* q, const void* k, const void* v, const void* out,
@@ -1829,9 +1830,8 @@ static int attn_bwd_impl(const void* dout, const void* q, const void* k, const v
   TP_REQUIRE(!seg || Sq == Skv, TP_ERR_BAD_ARG, "tp_attn_bwd: segment ids need Sq == Skv (got %d, %d)", Sq, Skv);
   TP_REQUIRE(sm_scale > 0.f, TP_ERR_BAD_ARG, "tp_attn_bwd: sm_scale must be positive");
   if (dtype == TP_F32) {
-    TP_REQUIRE(!mx.on, TP_ERR_UNSUPPORTED, "tp_attn_bwd_masked: windows, soft cap and query positions need 16-bit tensors");
     return attn_bwd_f32(dout, q, k, v, out, lse, seg, dq, dk, dv, ws, B, Hq, Hkv, Sq, Skv, Dqk, Dv, do_strides, q_strides, k_strides,
-                        v_strides, o_strides, dq_strides, dk_strides, dv_strides, sm_scale, causal, (hipStream_t)stream);
+                        v_strides, o_strides, dq_strides, dk_strides, dv_strides, sm_scale, causal, (hipStream_t)stream, mx);
   }
   TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F16, TP_ERR_UNSUPPORTED, "tp_attn_bwd: dtype %d (bf16, fp16 and fp32 only)", dtype);
   TP_REQUIRE((int64_t)(B + 8) * Hq * ((Sq + 127) / 128 + (Skv + 127) / 128) < (1ll << 31), TP_ERR_UNSUPPORTED, "tp_attn_bwd: too many workgroups");

@@ -34,6 +34,8 @@ struct BwdArgs32 {
   int64_t qs[3], ks[3], vs[3], os[3], dos[3], dqs[3], dks[3], dvs[3];
   float scale_log2, sm_scale;
   int causal;
+  MaskExt mx;   // as in the forward
+  float cap2;
 };
 
 // delta[b, h, q] = sum_d dO[q][d] * O[q][d]
@@ -106,6 +108,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(const BwdArgs32 a)
 #pragma unroll
     for (int v = 0; v < 16; v++) dqacc[d][v] = 0.f;
 
+  const int qp = a.mx.on ? (a.mx.qpos ? a.mx.qpos[qrow_c] : qrow_c) : 0;
+  const int band_lo = a.mx.on ? qp - a.mx.lo_off : -BAND_INF, band_hi = a.mx.on ? qp + a.mx.hi_off : BAND_INF;
   const int kv_end = a.causal ? min(Skv, q0 + BM) : Skv;
   const int ntiles = (kv_end + BN - 1) / BN;
   for (int t = 0; t < ntiles; t++) {
@@ -135,9 +139,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(const BwdArgs32 a)
 #pragma unroll
     for (int v = 0; v < 16; v++) {
       const int kvl = 8 * (v / 4) + 4 * g + (v % 4), kv = kv0 + kvl;
-      const bool ok = kv < Skv && (!a.causal || kv <= qrow) && (!segb || ssm[kvl] == segq);
-      const float p = ok ? exp2f(s[v] - lse2) : 0.f;
-      s[v] = p * (dp[v] - delta);
+      const bool ok = kv < Skv && (!a.causal || kv <= qrow) && (!segb || ssm[kvl] == segq) && kv >= band_lo && kv <= band_hi;
+      float sv = s[v], fac = 1.f;
+      if (a.cap2 != 0.f) {
+        const float th = tanhf(sv / a.cap2);
+        sv = a.cap2 * th;
+        fac = 1.f - th * th;  // derivative of the capped score with respect to the raw one
+      }
+      const float p = ok ? exp2f(sv - lse2) : 0.f;
+      s[v] = p * (dp[v] - delta) * fac;
     }
     // dQ^T += K^T dS^T
 #pragma unroll
@@ -166,7 +176,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_f32_kernel(const BwdArgs32 
   __shared__ __align__(16) float qsm[BMQ * STRIDE];
   __shared__ __align__(16) float dosm[BMQ * STRIDE];
   __shared__ float lsm[BMQ], dsm[BMQ];
-  __shared__ int ssm[BMQ];
+  __shared__ int ssm[BMQ], psm[BMQ];  // segment ids and key-order positions of the tile's query rows
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, ln = lane & 31;
   const int n_kt = (a.Skv + BNK - 1) / BNK;
   const int kt = blockIdx.x % n_kt, bg = blockIdx.x / n_kt;
@@ -212,6 +222,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_f32_kernel(const BwdArgs32 
         lsm[tid] = (lraw == -INFINITY) ? INFINITY : lraw * LOG2E;
         dsm[tid] = a.delta[ro + qr];
         ssm[tid] = segb ? segb[qr] : 0;
+        psm[tid] = a.mx.qpos ? a.mx.qpos[qr] : qr;
       }
       __syncthreads();
       if ((a.causal && qi0 + BMQ - 1 < wkv0) || wkv0 >= Skv) continue;  // (uniform per wave)
@@ -234,10 +245,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_f32_kernel(const BwdArgs32 
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         const int r = 8 * (v / 4) + 4 * g + (v % 4), qrow = qi0 + r;
-        const bool ok = qrow < Sq && kvcol < Skv && (!a.causal || kvcol <= qrow) && (!segb || ssm[r] == segk);
-        const float p = ok ? exp2f(s[v] - lsm[r]) : 0.f;
+        bool ok = qrow < Sq && kvcol < Skv && (!a.causal || kvcol <= qrow) && (!segb || ssm[r] == segk);
+        if (a.mx.on) ok = ok && kvcol >= psm[r] - a.mx.lo_off && kvcol <= psm[r] + a.mx.hi_off;
+        float sv = s[v], fac = 1.f;
+        if (a.cap2 != 0.f) {
+          const float th = tanhf(sv / a.cap2);
+          sv = a.cap2 * th;
+          fac = 1.f - th * th;
+        }
+        const float p = ok ? exp2f(sv - lsm[r]) : 0.f;
         s[v] = p;
-        dp[v] = p * (dp[v] - dsm[r]);
+        dp[v] = p * (dp[v] - dsm[r]) * fac;
       }
       // dV^T += dO^T P,  dK^T += Q^T dS
 #pragma unroll
@@ -284,7 +302,8 @@ static int launch_bwd_f32(const BwdArgs32& a, hipStream_t st) {
 int attn_bwd_f32(const void* dout, const void* q, const void* k, const void* v, const void* out, const float* lse,
                  const int32_t* seg, void* dq, void* dk, void* dv, float* ws, int B, int Hq, int Hkv, int Sq, int Skv, int Dqk,
                  int Dv, const int64_t* dos, const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
-                 const int64_t* dqs, const int64_t* dks, const int64_t* dvs, float sm_scale, int causal, hipStream_t st) {
+                 const int64_t* dqs, const int64_t* dks, const int64_t* dvs, float sm_scale, int causal, hipStream_t st,
+                 const MaskExt& mx) {
   TP_REQUIRE(Dqk == Dv && (Dqk == 64 || Dqk == 128), TP_ERR_UNSUPPORTED,
              "tp_attn_bwd: fp32 attention is built for head dims 64 and 128 (got qk=%d, v=%d)", Dqk, Dv);
   BwdArgs32 a;
@@ -302,7 +321,9 @@ int attn_bwd_f32(const void* dout, const void* q, const void* k, const void* v, 
              "tp_attn_bwd: too many workgroups");
   a.scale_log2 = sm_scale * LOG2E;
   a.sm_scale = sm_scale;
-  a.causal = causal;
+  a.causal = mx.on ? 0 : causal;
+  a.mx = mx;
+  a.cap2 = mx.cap_in != 0.f ? mx.cap_out * sm_scale * LOG2E : 0.f;
   return Dqk == 64 ? launch_bwd_f32<64>(a, st) : launch_bwd_f32<128>(a, st);
 }
 

@@ -590,7 +590,7 @@ static int dispatch_fwd(const FwdArgs& a, int B, int causal, hipStream_t st) {
 // fp32 operands: attn_fwd_f32.hip
 int attn_fwd_f32(const void* q, const void* k, const void* v, const int32_t* seg, void* out, float* lse, int B, int Hq, int Hkv,
                  int Sq, int Skv, int Dqk, int Dv, const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
-                 float sm_scale, int causal, hipStream_t st);
+                 float sm_scale, int causal, hipStream_t st, const MaskExt& mx);
 
 }  // namespace tp
 
@@ -606,10 +606,9 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, const int3
   TP_REQUIRE(Hq % Hkv == 0, TP_ERR_BAD_ARG, "tp_attn_fwd: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
   TP_REQUIRE(!seg || Sq == Skv, TP_ERR_BAD_ARG, "tp_attn_fwd: segment ids need Sq == Skv (got %d, %d)", Sq, Skv);
   TP_REQUIRE(sm_scale > 0.f, TP_ERR_BAD_ARG, "tp_attn_fwd: sm_scale must be positive");
-  TP_REQUIRE(!mx.on || dtype != TP_F32, TP_ERR_UNSUPPORTED, "tp_attn_fwd_masked: windows, soft cap and query positions need 16-bit tensors");
   if (dtype == TP_F32)
     return attn_fwd_f32(q, k, v, seg, out, lse, B, Hq, Hkv, Sq, Skv, Dqk, Dv, q_strides, k_strides, v_strides, o_strides, sm_scale,
-                        causal, (hipStream_t)stream);
+                        causal, (hipStream_t)stream, mx);
   TP_REQUIRE(dtype == TP_BF16 || dtype == TP_F16, TP_ERR_UNSUPPORTED, "tp_attn_fwd: dtype %d (bf16, fp16 and fp32 only)", dtype);
   TP_REQUIRE((int64_t)(B + 8) * Hq * ((Sq + 127) / 128) < (1ll << 31), TP_ERR_UNSUPPORTED, "tp_attn_fwd: too many workgroups");
   FwdArgs a;

@@ -29,6 +29,8 @@ struct FwdArgs32 {
   int64_t qs[3], ks[3], vs[3], os[3];
   float scale_log2;
   int causal;
+  MaskExt mx;   // window / query positions / causal offset as a band of key positions per query row; soft cap
+  float cap2;   // the soft cap in the scores' log2 units (0: none)
 };
 
 typedef float f32x1 __attribute__((ext_vector_type(1)));
@@ -55,6 +57,10 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(const FwdArgs32 a) {
   const float* vb = a.v + b * a.vs[0] + hk * a.vs[1];
   const int32_t* segb = a.seg ? a.seg + (int64_t)b * Skv : nullptr;
   const int segq = segb ? segb[min(qrow, Sq - 1)] : 0;
+  // mask extensions: this lane's query row may see key positions qp - lo_off .. qp + hi_off (causality is part of
+  // the band then, and a.causal is off)
+  const int qp = a.mx.on ? (a.mx.qpos ? a.mx.qpos[min(qrow, Sq - 1)] : qrow) : 0;
+  const int band_lo = a.mx.on ? qp - a.mx.lo_off : -BAND_INF, band_hi = a.mx.on ? qp + a.mx.hi_off : BAND_INF;
 
   // Q^T fragments: lane (query column ln, group g) holds Q[q][g*HD + s] for s = 0..HD-1, pre-multiplied by the
   // scale in log2 units (an fp32 product: no precision is lost that the fp32 reference keeps)
@@ -112,7 +118,8 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(const FwdArgs32 a) {
     for (int v = 0; v < 16; v++) {
       const int kvl = 8 * (v / 4) + 4 * g + (v % 4);
       const int kv = kv0 + kvl;
-      const bool ok = kv < Skv && (!a.causal || kv <= qrow) && (!segb || ssm[kvl] == segq);
+      const bool ok = kv < Skv && (!a.causal || kv <= qrow) && (!segb || ssm[kvl] == segq) && kv >= band_lo && kv <= band_hi;
+      if (a.cap2 != 0.f) s[v] = a.cap2 * tanhf(s[v] / a.cap2);  // cap * tanh(score / cap), in log2 units
       s[v] = ok ? s[v] : -INFINITY;
       mx = fmaxf(mx, s[v]);
     }
@@ -160,7 +167,7 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(const FwdArgs32 a) {
 // called by tp_attn_fwd for TP_F32 inputs (arguments already validated there)
 int attn_fwd_f32(const void* q, const void* k, const void* v, const int32_t* seg, void* out, float* lse, int B, int Hq, int Hkv,
                  int Sq, int Skv, int Dqk, int Dv, const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
-                 float sm_scale, int causal, hipStream_t st) {
+                 float sm_scale, int causal, hipStream_t st, const MaskExt& mx) {
   TP_REQUIRE(Dqk == Dv && (Dqk == 64 || Dqk == 128), TP_ERR_UNSUPPORTED,
              "tp_attn_fwd: fp32 attention is built for head dims 64 and 128 (got qk=%d, v=%d)", Dqk, Dv);
   FwdArgs32 a;
@@ -173,7 +180,9 @@ int attn_fwd_f32(const void* q, const void* k, const void* v, const int32_t* seg
   }
   TP_REQUIRE(ok, TP_ERR_BAD_ARG, "tp_attn_fwd: fp32 pointers and strides must keep rows 16-byte aligned");
   a.scale_log2 = sm_scale * LOG2E;
-  a.causal = causal;
+  a.causal = mx.on ? 0 : causal;
+  a.mx = mx;
+  a.cap2 = mx.cap_in != 0.f ? mx.cap_out * sm_scale * LOG2E : 0.f;
   const int64_t blocks = (int64_t)B * Hq * ((Sq + 127) / 128);
   TP_REQUIRE(blocks < (1ll << 31), TP_ERR_UNSUPPORTED, "tp_attn_fwd: too many workgroups");
   if (Dqk == 64) attn_fwd_f32_kernel<64><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(a);

@@ -426,8 +426,6 @@ def attn_bwd_masked(
   sm_scale: float, causal: bool, causal_offset: int, window_left: int, window_right: int, soft_cap: float,
 ) -> tuple[Tensor, Tensor, Tensor]:  # fmt: skip
   dev = _lib.require_gpu(dout, q, k, v, out, lse, seg, qpos)
-  if q.dtype == torch.float32:
-    raise NotImplementedError("windows, soft cap and query positions are built for bfloat16 and float16 tensors")
   B, Hq, Hkv, Sq, Skv, Dqk, Dv = _check_attn(q, k, v, seg)
   q, k, v, out, dout = _prep_heads(q), _prep_heads(k), _prep_heads(v), _prep_heads(out), _prep_heads(dout)
   lse = lse.contiguous()
