@@ -215,3 +215,16 @@ def test_rotary_frequencies_stay_fp32_under_a_dtype_cast():
   assert holder[0].inv_freq.dtype == torch.float32 and torch.equal(holder[0].inv_freq, before)
   assert "inv_freq" not in rot.state_dict()
 
+
+def test_bench_refuses_more_than_one_gpu_and_needs_a_gpu():
+  """bench.py measures the one-GPU hot path: --gpus above 1 exits with a message that says so, and without a GPU the
+  default run stops before any work (no CPU fallback is ever timed in the product's place)."""
+  import subprocess
+  import sys
+  root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+  r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+  assert r.returncode != 0 and "one-GPU" in r.stderr
+  if not torch.cuda.is_available():
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py")], capture_output=True, text=True, timeout=300)
+    assert r.returncode != 0 and "needs a GPU" in r.stderr and "metric" not in r.stdout
+
