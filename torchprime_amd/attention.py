@@ -11,6 +11,7 @@ on a single GPU: they are accepted and ignored.
 from __future__ import annotations
 
 import math
+import weakref
 from typing import Any
 
 import torch
@@ -41,20 +42,25 @@ def _is_causal_additive_mask(mask: torch.Tensor, q_len: int, kv_len: int) -> boo
   return bool(ok.all())
 
 
-# Verdicts of the check above, keyed on the mask's storage, shape and version.  A model builds its mask once per
-# forward and hands the same tensor to every layer, so the (S x S) compare and its host sync run once per mask
-# rather than once per layer; ``kernel_config={"assume_causal_mask": True}`` skips the check altogether.
+# Verdicts of the check above, kept per mask tensor object (a weak reference and the tensor's version counter).  A
+# model builds its mask once per forward and hands the same tensor to every layer, so the (S x S) compare and its
+# host sync run once per mask rather than once per layer.  The key is the object, never its address: a mask built
+# for the next forward is a new tensor that the caching allocator may well place where the last one was.
+# ``kernel_config={"assume_causal_mask": True}`` skips the check altogether.
 _MASK_VERDICTS: dict = {}
 
 
 def _causal_mask_verdict(mask: torch.Tensor, q_len: int, kv_len: int) -> bool:
-  key = (mask.data_ptr(), tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask._version, q_len, kv_len)
-  hit = _MASK_VERDICTS.get(key)
-  if hit is None:
-    if len(_MASK_VERDICTS) > 16:
-      _MASK_VERDICTS.clear()
-    hit = _MASK_VERDICTS[key] = _is_causal_additive_mask(mask, q_len, kv_len)
-  return hit
+  ident = id(mask)
+  key = (mask._version, tuple(mask.shape), q_len, kv_len)
+  entry = _MASK_VERDICTS.get(ident)
+  if entry is not None and entry[0]() is mask and entry[1] == key:
+    return entry[2]
+  verdict = _is_causal_additive_mask(mask, q_len, kv_len)
+  # the entry leaves with the tensor (its id may be reused afterwards, hence also the identity check above)
+  ref = weakref.ref(mask, lambda _r, ident=ident: _MASK_VERDICTS.pop(ident, None))
+  _MASK_VERDICTS[ident] = (ref, key, verdict)
+  return verdict
 
 
 class AttentionModule(nn.Module):

@@ -314,13 +314,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   constexpr int BNK = 128;  // kv rows per workgroup, 32 per wave
   constexpr int KS_QK = DQK / 16, KS_DV = DV / 16;
   constexpr int DKB = DQK / 32, DVB = DV / 32;
-  typedef DmaTile<DQK> QT;
-  typedef DmaTile<DV> OT;
+  // PIPE: equal head dims up to 128.  Three row-major buffers, no transposed copies: the operands of the two
+  // accumulating products are read from the row-major tiles with transposing LDS reads.
+  constexpr bool PIPE = NBUF == 3 && DQK == DV && DQK <= 128;
+  static_assert(PIPE || NBUF == 1, "three buffers (pipelined path) or one");
+  typedef DmaTile<DQK, PIPE> QT;
+  typedef DmaTile<DV, PIPE> OT;
   constexpr int Q_BYTES = QT::BYTES, DO_BYTES = OT::BYTES;
-  constexpr int QTR_BYTES = DQK * TrTile64::ROW_BYTES, DOTR_BYTES = DV * TrTile64::ROW_BYTES;
+  constexpr int QTR_BYTES = PIPE ? 0 : DQK * TrTile64::ROW_BYTES, DOTR_BYTES = PIPE ? 0 : DV * TrTile64::ROW_BYTES;
   constexpr int ROW_BYTES = BMQ * 4 * 4;  // lse (log2 units), delta, segment id per query row (+1 unused): 3 slots
   constexpr int BUF_BYTES = Q_BYTES + DO_BYTES + QTR_BYTES + DOTR_BYTES;
-  constexpr bool PIPE = NBUF == 2 && DQK == DV && DQK <= 128;
   // LDS layout: the NBUF copies of each kind of tile lie side by side (Q.. dO.. Q^T.. dO^T.., then the row
   // vectors), so that with the buffer index a constant every fragment address is a loop-invariant per-lane
   // offset plus an immediate
@@ -412,7 +415,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     nact = cnt;
     __syncthreads();
     for (int i = tid; i < nact; i += 256) {
-      const int t = active[i];
+      const int t = active[nact - 1 - i];  // visiting order: last query tile first (see qtile_of)
       *(i32x4*)(ctl + 4 * i) = i32x4{qt_first + t, qmin[t], qmax[t], t};
     }
     __syncthreads();
@@ -429,7 +432,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   const unsigned q_tile_bytes = (unsigned)(BMQ * a.qs[2] * 2), do_tile_bytes = (unsigned)(BMQ * a.dos[2] * 2);
   const float* lse2 = a.delta + (int64_t)a.B * a.Hq * Sq;  // second half of the workspace (delta kernel)
   unsigned char* const rows_base = smem + NBUF * BUF_BYTES;
-  auto qtile_of = [&](int idx) { return SEG ? ctl[4 * idx] : qt_first + idx; };
+  // Query tiles are visited from the last one down.  The workgroups of a (batch, kv head) run side by side on one XCD
+  // and all stream the same Q / dO tiles; each needs the tiles from its own kv rows on, so counting up they would start
+  // at different tiles and never meet in the L2 (every tile fetched from memory once per workgroup); counting down
+  // they start together at the last tile and stay within an L2's reach of each other.
+  auto qtile_of = [&](int idx) { return SEG ? ctl[4 * idx] : nqt_all - 1 - idx; };
   auto issue_tile = [&](int hl, int idx, int buf, int rslot) {
     const int hq = hk * a.n_rep + hl;
     const int qt = qtile_of(idx);
@@ -492,40 +499,58 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     const int* e = ctl + 4 * idx;
     return tile_mode_of(SEG ? e[1] : 0, SEG ? e[2] : 0, SEG ? e[3] : 0, qi0);
   };
-  // iteration -> (query head of the group, query tile): heads outer, tiles inner, no division in the loop
+  // iteration -> (query head of the group, query tile): heads outer, tiles inner, no division in the loop.  (Tiles
+  // outer would keep the group's workgroups on the same tile for the whole launch and cut the fetches from memory to
+  // 1.8 GB at the benchmark's shape, against 6.5 GB this way - and ran 4 % slower: 32 CUs asking one L2 for the same
+  // lines at the same time, and the descriptors rebuilt every tile.)
   auto advance = [&](int& hl, int& idx) {
     if (++idx == nact) { idx = 0; hl++; }
   };
 
   if constexpr (PIPE) {
-    // Software pipeline over query tiles t, two full buffers (row-major + transposed) and three row-vector
-    // slots.  Tile t+1's loads are issued in the middle of tile t-1 and have a whole tile body to land;
-    // its transposed copies are made under the second half of tile t's MFMAs:
-    //   part 1 (S, dP: row-major tiles of buffer t&1)
-    //   wait for this wave's share of tile t+1, barrier      -> buffer t&1's row-major tiles are free,
-    //   issue the loads of tile t+2 into them                   tile t+1 has landed for everybody
-    //   part 2 (dV, dK: transposed tiles of buffer t&1), interleaved with transposing tile t+1
-    //   barrier
+    // Software pipeline over query tiles t, three row-major buffers and three row-vector slots (tile t lives in
+    // buffer and slot t % 3), one barrier per tile:
+    //   part 1 (S, dP: fragment reads of buffer t % 3)
+    //   wait for this wave's share of tile t+1 (issued a whole tile earlier), barrier
+    //                                  -> tile t+1 has landed for everybody, everybody is done with tile t-1
+    //   part 2 (dV, dK: transposing reads of buffer t % 3), with the loads of tile t+2 issued between its MFMAs
+    //   into the buffer tile t-1 used
     int c_hl = 0, c_idx = 0, n_hl = 0, n_idx = 0;  // tile being computed, tile whose loads are issued next
-    TransposeSteps<DQK> trq;
-    TransposeSteps<DV> tro;
-    // offsets into the transposed tiles carry TR_BIAS in their registers (an opaque value: the compiler would
-    // otherwise fold it back into constants too large for an instruction offset and add it at every use)
-    constexpr int TR_BIAS = QTR_AT;
-    unsigned tr_bias = (unsigned)TR_BIAS;
-    asm volatile("" : "+v"(tr_bias));
-    trq.init(tid, tr_bias);
-    tro.init(tid, tr_bias);
-    unsigned tb[4];
+    // Per-lane LDS byte addresses of the operands inside a tile (base of the workgroup's LDS included), each an
+    // opaque register: every read below is such a register plus an immediate.  (Formed from the `smem` symbol, the
+    // same addresses cost an add per read whenever the constant part happens to be zero, and the compiler
+    // recomputes what it could have kept.)  Addresses into the dO tiles carry O_BIAS: constants there would
+    // otherwise exceed the reach of an instruction offset.
+    //   aq / ao   fragment reads of the row-major tiles (S, dP): row ln, chunk 2 ks + g
+    //   trq / tro transposing reads (dK, dV): head-dim block d (32 columns), half h2 (rows +8); the query block and
+    //             the k-step are immediates (multiples of 16 rows leave the swizzle alone)
+    constexpr int O_BIAS = DO_AT;
+    const unsigned lb = (unsigned)(size_t)smem;
+    unsigned aq[KS_QK], ao[KS_DV], trq[DKB][2], tro[DVB][2];
 #pragma unroll
-    for (int m = 0; m < 4; m++) tb[m] = ta[m] + tr_bias;
+    for (int ks = 0; ks < KS_QK; ks++) { aq[ks] = faq[ks] + lb; asm volatile("" : "+v"(aq[ks])); }
+#pragma unroll
+    for (int ks = 0; ks < KS_DV; ks++) { ao[ks] = fao[ks] + lb + (unsigned)O_BIAS; asm volatile("" : "+v"(ao[ks])); }
+#pragma unroll
+    for (int d = 0; d < DKB; d++)
+#pragma unroll
+      for (int h2 = 0; h2 < 2; h2++) {
+        trq[d][h2] = (unsigned)QT::tr_off(8 * h2 + 4 * g, 2 * d + ((lane >> 4) & 1), lane & 15) + lb;
+        asm volatile("" : "+v"(trq[d][h2]));
+        tro[d][h2] = trq[d][h2] + (unsigned)O_BIAS;
+        asm volatile("" : "+v"(tro[d][h2]));
+      }
+    auto ld16 = [](unsigned addr) { return *(const __attribute__((address_space(3))) v8*)addr; };
+    auto ldtr = [](unsigned a0, unsigned a1) {
+      return tr_read8<v8>((const __attribute__((address_space(3))) unsigned char*)a0, (const __attribute__((address_space(3))) unsigned char*)a1);
+    };
     if (n_iter > 0) { issue_tile(n_hl, n_idx, 0, 0); advance(n_hl, n_idx); }
     if (n_iter > 1) { issue_tile(n_hl, n_idx, 1, 1); advance(n_hl, n_idx); }
     // the control entry of the tile being computed and the query tile whose loads are issued next, as scalars; their
     // successors are read at the top of a tile and taken over at its end
     auto entry = [&](int idx) {
       if constexpr (SEG) return *(const i32x4*)(ctl + 4 * min(idx, max(nact - 1, 0)));
-      else return i32x4{qt_first + idx, 0, 0, 0};
+      else return i32x4{nqt_all - 1 - idx, 0, 0, 0};
     };
     auto scalar4 = [&](i32x4 v) {
       return i32x4{__builtin_amdgcn_readfirstlane(v[0]), __builtin_amdgcn_readfirstlane(v[1]),
@@ -536,34 +561,23 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     // all earlier loads (the K/V fragments, the first tiles) have landed
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    if (n_iter > 0) {
-      trq.read(smem + Q_AT);
-      tro.read(smem + DO_AT);
-      static_for<0, 8>([&](auto J) {
-        trq.write(smem + (QTR_AT - TR_BIAS), J);
-        tro.write(smem + (DOTR_AT - TR_BIAS), J);
-      });
-    }
-    __syncthreads();
-
     // fragment ring: slot i's LDS fragment is requested AHEAD slots earlier and kept in fr[i % NF]; the
     // first AHEAD fragments of a tile are requested at the end of the tile before it (its row-major
     // tiles are complete by then), so that the LDS round trip and the scalar bookkeeping at the top of
     // the loop overlap
-    constexpr int AHEAD = KS_QK >= 8 ? 7 : 3, NF = AHEAD + 1;
+    constexpr int AHEAD = KS_QK >= 8 ? 5 : 3, NF = AHEAD + 1;
     v8 fr[NF];
     static_for<0, AHEAD>([&](auto I) {
       constexpr int i = decltype(I)::value;
       static_assert(AHEAD <= KS_QK, "the carried fragments all belong to S of the first query block");
-      fr[i % NF] = *(const v8*)(smem + Q_AT + faq[i]);
+      fr[i % NF] = ld16(aq[i] + Q_AT);
     });
     struct { u32x4 rq, ro, rr; unsigned offq, offo, offr; } nx;
     const unsigned lds_base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)smem);
     const unsigned wave_q = __builtin_amdgcn_readfirstlane((unsigned)(wave * QT::PER_WAVE * 1024));
     const unsigned wave_o = __builtin_amdgcn_readfirstlane((unsigned)(wave * OT::PER_WAVE * 1024));
     const unsigned wave_r = __builtin_amdgcn_readfirstlane((unsigned)(wave * BMQ * 4));
-    int rslot = 0;
-    // one query tile; the buffer index is a constant (the loop below alternates two copies of this)
+    // one query tile; the buffer index is a constant (the loop below rotates three copies of this)
     auto iteration = [&](auto BUFc, const int it) {
       constexpr int buf = decltype(BUFc)::value;
       const int qi0 = cur[0] * BMQ;
@@ -575,24 +589,18 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       if (issue_next) advance(n_hl2, n_idx2);
       const i32x4 cur_next = entry(c_idx2);
       const int nq_next = entry(n_idx2)[0];
-      const unsigned char* ql = smem + Q_AT + buf * Q_BYTES;
-      const unsigned char* dol = smem + DO_AT + buf * DO_BYTES;
-      const unsigned char* qtl = smem + (QTR_AT + buf * QTR_BYTES - TR_BIAS);     // + tb[]
-      const unsigned char* dotl = smem + (DOTR_AT + buf * DOTR_BYTES - TR_BIAS);  // + tb[]
-      // tile t+1 (being transposed, then read first in the next iteration) lives in the other buffer
-      unsigned char* const nxq = smem + Q_AT + (buf ^ 1) * Q_BYTES;
-      unsigned char* const nxdo = smem + DO_AT + (buf ^ 1) * DO_BYTES;
-      unsigned char* const nxqt = smem + (QTR_AT + (buf ^ 1) * QTR_BYTES - TR_BIAS);
-      unsigned char* const nxdot = smem + (DOTR_AT + (buf ^ 1) * DOTR_BYTES - TR_BIAS);
-      const float* lsel = (const float*)(rows_base + rslot * ROW_BYTES);
+      constexpr int buf1 = (buf + 1) % 3, buf2 = (buf + 2) % 3;  // tile t+1 (read first in the next iteration), tile t+2
+      constexpr unsigned ql = Q_AT + buf * Q_BYTES;                // + aq[] / trq[]
+      constexpr unsigned dol = DO_AT + buf * DO_BYTES - O_BIAS;    // + ao[] / tro[]
+      constexpr unsigned nxq = Q_AT + buf1 * Q_BYTES;
+      const float* lsel = (const float*)(rows_base + buf * ROW_BYTES);
       const float* deltal = lsel + BMQ;
       const int* segl = (const int*)(deltal + BMQ);
       const int* posl = segl + BMQ;  // query positions of the tile's rows (mask extensions)
-      const int rnext = rslot >= 1 ? rslot - 1 : 2;  // (it + 2) % 3, the slot tile t-1 used
       // LDS destinations of this wave's loads of tile t+2 (scalar byte addresses)
-      const unsigned dma_q = lds_base + (unsigned)(Q_AT + buf * Q_BYTES) + wave_q;
-      const unsigned dma_o = lds_base + (unsigned)(DO_AT + buf * DO_BYTES) + wave_o;
-      const unsigned dma_r = lds_base + (unsigned)(NBUF * BUF_BYTES + rnext * ROW_BYTES) + wave_r;
+      const unsigned dma_q = lds_base + (unsigned)(Q_AT + buf2 * Q_BYTES) + wave_q;
+      const unsigned dma_o = lds_base + (unsigned)(DO_AT + buf2 * DO_BYTES) + wave_o;
+      const unsigned dma_r = lds_base + (unsigned)(NBUF * BUF_BYTES + buf2 * ROW_BYTES) + wave_r;
       // descriptors of tile t+2's loads (wave-uniform), issued piecewise in part 2.  The bases change with
       // the query head only; they are rebuilt when a new head starts (and when the tiles run out: size 0).
       if (it == 0 || n_idx == 0 || !issue_next) {
@@ -636,9 +644,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         static_assert(VL == 2 * K && VP0 + VL <= C0 && VS0 + VL <= C0 + CL && VP1 + VL <= C0 + 2 * CL &&
                           VS1 + VL <= C0 + 3 * CL,
                       "operands not ready");
-        // transposing the next tile: reads of a tile in one slot, then WPS column pairs per slot
-        constexpr int WPS = (NS - C0 >= 24) ? 1 : 2, TQ0 = C0, TO0 = TQ0 + 2 + 8 / WPS;
-        static_assert(TO0 + 2 + 8 / WPS <= NS, "second half too short for the transposition");
         constexpr int N_DMA = QT::PER_WAVE + OT::PER_WAVE + 1, DMA_EVERY = (NS - C0) / N_DMA;
         static_assert(DMA_EVERY >= 1, "second half too short for the loads");
         const int kvcol = wkv0 + ln;
@@ -681,12 +686,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
           constexpr int i = decltype(I)::value;
           if constexpr (i < C0) {
             constexpr int qb = (i / K) % 2, ks = i % K;
-            if constexpr (i < 2 * K) return *(const v8*)(ql + faq[ks] + qb * 32 * QT::ROWB);
-            else return *(const v8*)(dol + fao[ks] + qb * 32 * OT::ROWB);
+            if constexpr (i < 2 * K) return ld16(aq[ks] + (ql + qb * 32 * QT::ROWB));
+            else return ld16(ao[ks] + (dol + qb * 32 * OT::ROWB));
           } else {
+            // operand of an accumulating product: rows = head-dim block d, contraction over query rows
+            // 32 qb + 16 hh + {4g..4g+3, 8+4g..8+4g+3} (the order in which P / dS hold them), read transposed
             constexpr int ph = (i - C0) / CL, qb = ph / 2, j = (i - C0) % CL, hh = j / DVB, d = j % DVB;
-            const unsigned char* base = (ph % 2 == 0) ? dotl : qtl;
-            return *(const v8*)(base + tb[(2 * qb + hh) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
+            constexpr int rows = (32 * qb + 16 * hh) * QT::ROWB;
+            if constexpr (ph % 2 == 0) return ldtr(tro[d][0] + (dol + rows), tro[d][1] + (dol + rows));
+            else return ldtr(trq[d][0] + (ql + rows), trq[d][1] + (ql + rows));
           }
         };
         auto mma = [&](auto I, const v8& f) {
@@ -772,20 +780,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
             }
           }
         };
-        // transposition of tile t+1 (buffer bn), one step per slot from slot C0 on
-        auto transpose_step = [&](auto I) {
-          constexpr int i = decltype(I)::value;
-          if constexpr (i == TQ0) trq.read(nxq);
-          if constexpr (i == TO0) tro.read(nxdo);
-          if constexpr (i >= TQ0 + 2 && i < TQ0 + 2 + 8 / WPS)
-            static_for<0, WPS>([&](auto W) {
-              trq.write(nxqt, std::integral_constant<int, (i - TQ0 - 2) * WPS + decltype(W)::value>{});
-            });
-          if constexpr (i >= TO0 + 2 && i < TO0 + 2 + 8 / WPS)
-            static_for<0, WPS>([&](auto W) {
-              tro.write(nxdot, std::integral_constant<int, (i - TO0 - 2) * WPS + decltype(W)::value>{});
-            });
-        };
         typedef std::integral_constant<int, 0> I0;
         typedef std::integral_constant<int, 1> I1;
         static_for<0, NS>([&](auto I) {
@@ -807,17 +801,20 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
             else dma_dword_at(nx.rr, nx.offr, dma_r, lane);
           }
           if constexpr (COMPUTE) {
-            if constexpr (i == 0) {
-#pragma unroll
-              for (int vq = 0; vq < 4; vq++) nl0[vq] = *(const f32x4*)(lsel + 8 * vq + 4 * g);
-            }
-            if constexpr (i == K) {
-#pragma unroll
-              for (int vq = 0; vq < 4; vq++) nl1[vq] = *(const f32x4*)(lsel + 32 + 8 * vq + 4 * g);
+            // row vectors, a quad of rows at a time: -LSE of query block qb LEAD slots before the exponentials of that
+            // quad (VP0 / VP1 + QS vq), -delta two slots before the first dP MFMA of the block (2K, 3K)
+            constexpr int QS = 4 / EPS, LEAD = 3;
+            static_for<0, 4>([&](auto VQ) {
+              constexpr int vq = decltype(VQ)::value;
+              constexpr int r0 = VP0 + QS * vq - LEAD, r1 = VP1 + QS * vq - LEAD;
+              if constexpr (i == (r0 < 0 ? 0 : r0)) nl0[vq] = *(const f32x4*)(lsel + 8 * vq + 4 * g);
+              if constexpr (i == (r1 < 0 ? 0 : r1)) nl1[vq] = *(const f32x4*)(lsel + 32 + 8 * vq + 4 * g);
+            });
+            if constexpr (i == 2 * K - 2) {
 #pragma unroll
               for (int vq = 0; vq < 4; vq++) nd0[vq] = *(const f32x4*)(deltal + 8 * vq + 4 * g);
             }
-            if constexpr (i == 2 * K) {
+            if constexpr (i == 3 * K - 2) {
 #pragma unroll
               for (int vq = 0; vq < 4; vq++) nd1[vq] = *(const f32x4*)(deltal + 32 + 8 * vq + 4 * g);
             }
@@ -828,27 +825,25 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
             valu(I, std::integral_constant<int, VS0>{}, I0{}, std::false_type{});
             valu(I, std::integral_constant<int, VS1>{}, I1{}, std::false_type{});
           }
-          transpose_step(I);
           __builtin_amdgcn_sched_barrier(0);
         });
         static_for<0, AHEAD>([&](auto I) {
           constexpr int i = decltype(I)::value;
-          fr[i % NF] = *(const v8*)(nxq + faq[i]);
+          fr[i % NF] = ld16(aq[i] + nxq);
         });
       };
       if (mode == 1) body(std::integral_constant<int, 1>{});
       else if (mode == 2) body(std::integral_constant<int, 2>{});
       else body(std::integral_constant<int, 0>{});
-      __syncthreads();
       n_hl = n_hl2; n_idx = n_idx2;
       c_hl = c_hl2; c_idx = c_idx2;
       cur = scalar4(cur_next);
       nq_cur = __builtin_amdgcn_readfirstlane(nq_next);
-      rslot = rslot == 2 ? 0 : rslot + 1;
     };
-    for (int it = 0; it < n_iter; it += 2) {
+    for (int it = 0; it < n_iter; it += 3) {
       iteration(std::integral_constant<int, 0>{}, it);
       if (it + 1 < n_iter) iteration(std::integral_constant<int, 1>{}, it + 1);
+      if (it + 2 < n_iter) iteration(std::integral_constant<int, 2>{}, it + 2);
     }
   } else {
     // Wide heads: one buffer of each kind; both query blocks go through each step together.  Per tile:
@@ -1071,7 +1066,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   // The accumulating MFMAs are opaque assembly (mfma32_acc): the compiler does not know that dkacc / dvacc come
   // out of a 16-pass matrix instruction and inserts no wait states before reading them.  Make the distance
   // explicit (the longest MFMA-write -> VALU-read hazard is 18 wait states).
-  asm volatile("s_nop 15\n\ts_nop 3" ::: "memory");
+  // (the accumulators are operands of the statement, so that no read of them can be scheduled ahead of it)
+  static_assert(DKB <= 6 && DVB <= 4, "operand lists below");
+  asm volatile("s_nop 15\n\ts_nop 3" : "+a"(dkacc[0]), "+a"(dkacc[1]), "+a"(dvacc[0]), "+a"(dvacc[1]) :: "memory");
+  if constexpr (DKB > 2) asm volatile("" : "+a"(dkacc[2]), "+a"(dkacc[3]));
+  if constexpr (DKB > 4) asm volatile("" : "+a"(dkacc[4]), "+a"(dkacc[5]));
+  if constexpr (DVB > 2) asm volatile("" : "+a"(dvacc[2]), "+a"(dvacc[3]));
   // ---- epilogue: lane = kv row, 4 consecutive head-dim values per store
   const int row = wkv0 + ln;
   if (row < Skv) {
@@ -1711,9 +1711,11 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
   // dK, dV
   {
     constexpr int BMQ = 64, BNK = 128;
-    constexpr int BUF = DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES + (DQK + DV) * TrTile64::ROW_BYTES;
+    // equal head dims up to 128: three row-major buffers (pipelined path); wide heads: one buffer with transposed copies
+    constexpr bool PIPE = DQK == DV && DQK <= 128;
+    constexpr int NBUF = PIPE ? 3 : 1;
+    constexpr int BUF = DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES + (PIPE ? 0 : (DQK + DV) * TrTile64::ROW_BYTES);
     constexpr int ROWS = 3 * BMQ * 16;
-    constexpr int NBUF = (2 * BUF + ROWS + 4096 <= 160 * 1024) ? 2 : 1;
     const int nqt = (a.Sq + BMQ - 1) / BMQ;
     const size_t smem = (size_t)NBUF * BUF + ROWS + (SEG ? (size_t)(6 * nqt + 8 + 4) * 4 : 0);
     TP_REQUIRE(smem <= 160 * 1024 && (size_t)3 * nqt * 4 <= (size_t)NBUF * BUF, TP_ERR_UNSUPPORTED,
@@ -1782,8 +1784,10 @@ int bwd_by_dims_f16(const BwdArgs& a, int Dqk, int Dv, int causal, hipStream_t s
 template <typename T>
 static int bwd_by_dims(const BwdArgs& a, int Dqk, int Dv, int causal, hipStream_t st, void* const* ev) {
   if (Dqk == 128 && Dv == 128) return dispatch_bwd<T, 128, 128>(a, causal, st, ev);
+#ifndef TP_ONLY_HEAD_DIM_128  // (a build option for quick timing builds of the head dim the benchmark runs)
   if (Dqk == 64 && Dv == 64) return dispatch_bwd<T, 64, 64>(a, causal, st, ev);
   if (Dqk == 192 && Dv == 128) return dispatch_bwd<T, 192, 128>(a, causal, st, ev);
+#endif
   return TP_DIMS_NOT_BUILT;
 }
 #if TP_BWD_F16

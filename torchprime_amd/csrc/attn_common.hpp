@@ -272,16 +272,31 @@ __device__ __forceinline__ u32x2 transpose_col(const u32x4 (&r)[4], int j) {
 // the lane, which global chunk it carries is free.  A tile of 64 rows x D 16-bit elements is stored
 // densely (row r at r * D*2) with the 16-byte chunks of a row XOR-swizzled by the row, so that the MFMA
 // fragment reads (lanes = consecutive rows, same logical chunk) fall into different banks.
-template <int D>
+// ROT picks the swizzle that also serves transposing reads (ds_read_b64_tr_b16) of the same tile: such a read
+// takes, per 32 lanes, a patch of 4 rows x 64 bytes, so the four rows of a quad must differ in the bits that select
+// the 64-byte quarter of the 256-byte bank line; the row's low bits go to the swizzle's high bits for that.  Both
+// swizzles are a permutation of the chunk positions over any 16 consecutive rows (fragment reads stay conflict free).
+template <int D, bool ROT = false>
 struct DmaTile {
   static constexpr int CPR = D / 8;              // 16-byte chunks per row
   static constexpr int ROWB = D * 2;             // bytes per row
   static constexpr int BYTES = 64 * ROWB;
   static constexpr int PER_WAVE = CPR / 4;       // load instructions per wave for one tile (4 waves)
   static_assert(CPR % 8 == 0, "head dim must be a multiple of 64");
-  static __device__ __forceinline__ int swz(int row) { return (CPR % 16 == 0) ? (row & 15) : ((row >> 1) & 7); }
+  static __device__ __forceinline__ int swz(int row) {
+    if constexpr (ROT) return (CPR % 16 == 0) ? (((row & 3) << 2) | ((row >> 2) & 3)) : ((((row >> 1) & 1) << 2) | ((row >> 2) & 3));
+    else return (CPR % 16 == 0) ? (row & 15) : ((row >> 1) & 7);
+  }
   // byte offset of logical chunk c of a row
   static __device__ __forceinline__ int off(int row, int c) { return row * ROWB + ((c ^ swz(row)) << 4); }
+  // Transposing read of the patch rows r0..r0+3 (r0 a multiple of 4) x columns 16 cb..16 cb + 15 by a group of 16
+  // lanes: lane 4 e + m of the group supplies the address of (row r0 + e, columns 16 cb + 4 m ..+3), and receives
+  // the four values (rows r0..r0+3) of column 16 cb + its own index in the group.  Byte offset inside the tile:
+  static __device__ __forceinline__ int tr_off(int r0, int cb, int lane16) {
+    static_assert(ROT || D == 0, "transposing reads need the rotated swizzle");
+    const int row = r0 + (lane16 >> 2), col = 16 * cb + 4 * (lane16 & 3);
+    return row * ROWB + (((col >> 3) ^ swz(row)) << 4) + (col & 7) * 2;
+  }
 
   unsigned vo[PER_WAVE];  // global byte offset (inside a tile) of the chunk this lane carries, per instruction
 
@@ -321,6 +336,17 @@ struct DmaTile {
     static_assert(PER_WAVE <= 6, "head dim above 192");
   }
 };
+// two transposing reads -> one 16-byte MFMA operand: values 0..3 from the first address, 4..7 from the second
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) unsigned char lds_byte;
+template <typename V8>
+__device__ __forceinline__ V8 tr_read8(const lds_byte* p0, const lds_byte* p1) {
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p0);
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p1);
+  const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(V8, v);
+}
 // buffer resource words for the assembly loads: base, stride 0, size in bytes, raw-buffer flags
 __device__ __forceinline__ u32x4 make_rsrc_words(const void* base, unsigned bytes) {
   const unsigned long long p = (unsigned long long)base;

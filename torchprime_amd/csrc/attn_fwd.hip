@@ -54,9 +54,10 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   constexpr int BM = 128;             // q rows per workgroup, 32 per wave
   constexpr int KSTEPS = DQK / 16;    // MFMA k-steps over the qk head dim
   constexpr int DVB = DV / 32;        // 32-column blocks of the v head dim
-  typedef DmaTile<DQK> KD;
+  typedef DmaTile<DQK, true> KD;
+  typedef DmaTile<DV, true> VD;  // row-major like K; its transposed operand comes out of transposing LDS reads
   constexpr int K_BYTES = KD::BYTES;
-  constexpr int V_BYTES = DV * TrTile64::ROW_BYTES;
+  constexpr int V_BYTES = VD::BYTES;
   constexpr int SEG_BYTES = SEG ? BN * 4 : 0;
   constexpr int BUF_BYTES = K_BYTES + V_BYTES + SEG_BYTES;
   // LDS layout: the two K tiles, then the two V^T tiles, then the two segment-id rows: with the buffer index a
@@ -67,9 +68,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   constexpr int K_AT = 0, K_STEP = STATIC_BUF ? K_BYTES : BUF_BYTES;
   constexpr int V_AT = STATIC_BUF ? 2 * K_BYTES : K_BYTES, V_STEP = STATIC_BUF ? V_BYTES : BUF_BYTES;
   constexpr int SEG_AT = STATIC_BUF ? 2 * (K_BYTES + V_BYTES) : K_BYTES + V_BYTES, SEG_STEP = STATIC_BUF ? SEG_BYTES : BUF_BYTES;
-  constexpr int K_ITEMS = KD::PER_WAVE;             // LDS-writing K loads per wave and tile
-  constexpr int V_TOT = (DV / 8) * (BN / 4);        // 4x8 blocks of the V tile
-  constexpr int V_ITEMS = (V_TOT + 255) / 256;
+  constexpr int K_ITEMS = KD::PER_WAVE, V_ITEMS = VD::PER_WAVE;  // LDS-writing loads per wave and tile
 
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -164,73 +163,37 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
     __syncthreads();
   }
 
-  // ---- global -> register staging of one K/V tile (buffer loads, rows past Skv read as zero)
-  // V row quads are dealt to threads so that the 32 lanes whose transposed 8-byte stores are served
-  // together fall into 32 different bank pairs
-  auto v_quad = [](int rqi) { return (rqi & ~3) | ((rqi & 1) << 1) | ((rqi >> 1) & 1); };
-  const rsrc_t vrs = make_rsrc(vb, span_bytes(Skv, a.vs[2], DV));
+  // ---- K and V tiles travel from memory into LDS by loads that write LDS themselves (rows past Skv arrive as zeros)
   const unsigned k_tile_bytes = (unsigned)(BN * a.ks[2] * 2), v_tile_bytes = (unsigned)(BN * a.vs[2] * 2);
-  unsigned vvo[V_ITEMS][4];
   KD kdma;
+  VD vdma;
   kdma.init(a.ks[2], wave, lane);
+  vdma.init(a.vs[2], wave, lane);
   const u32x4 krw = make_rsrc_words(kb, span_bytes(Skv, a.ks[2], DQK));
-#pragma unroll
-  for (int i = 0; i < V_ITEMS; i++) {
-    const int item = tid + 256 * i;
-    const int c8 = item % (DV / 8), rq = v_quad(item / (DV / 8));
-#pragma unroll
-    for (int ii = 0; ii < 4; ii++) vvo[i][ii] = (unsigned)(((4 * rq + ii) * a.vs[2] + c8 * 8) * 2);
-  }
-  u32x4 vreg[V_ITEMS][4];
+  const u32x4 vrw = make_rsrc_words(vb, span_bytes(Skv, a.vs[2], DV));
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const unsigned lds_base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)smem);
+  // this wave's first LDS destinations in buffer 0 (scalar byte addresses)
+  const unsigned kdst0 = lds_base + (unsigned)K_AT + (unsigned)(wave_s * K_ITEMS * 1024);
+  const unsigned vdst0 = lds_base + (unsigned)V_AT + (unsigned)(wave_s * V_ITEMS * 1024);
   int sreg = 0;
-  // the K tile goes straight into buffer `kbuf`, which nobody reads before the next barrier
-  auto load_tile = [&](int t, int kbuf) {
-    const unsigned kso = (unsigned)t * k_tile_bytes, vso = (unsigned)t * v_tile_bytes;
-    kdma.issue(krw, kso, smem + K_AT + kbuf * K_STEP, wave);
-#pragma unroll
-    for (int i = 0; i < V_ITEMS; i++) {
-      if (tid + 256 * i < V_TOT) {
-#pragma unroll
-        for (int ii = 0; ii < 4; ii++) vreg[i][ii] = buf_load16(vrs, vvo[i][ii], vso);
-      }
-    }
-    if (has_seg && tid < BN) sreg = segb[min(t * BN + tid, Skv - 1)];
-  };
-  // the same loads one at a time (piece P of K_ITEMS + 4 V_ITEMS), for issuing between MFMAs
+  // piece P of the K_ITEMS + V_ITEMS loads of tile t into buffer kbuf, for issuing between MFMAs
   auto load_piece = [&](auto Pc, int t, int kbuf) {
     constexpr int p = decltype(Pc)::value;
-    if constexpr (p < K_ITEMS) {
-      kdma.template issue_one<p>(krw, __builtin_amdgcn_readfirstlane((unsigned)t * k_tile_bytes), smem + K_AT + kbuf * K_STEP, wave);
-    } else {
-      constexpr int i = (p - K_ITEMS) / 4, ii = (p - K_ITEMS) % 4;
-      if (tid + 256 * i < V_TOT) vreg[i][ii] = buf_load16(vrs, vvo[i][ii], (unsigned)t * v_tile_bytes);
-    }
+    if constexpr (p < K_ITEMS)
+      kdma.template issue_one_at<p>(krw, __builtin_amdgcn_readfirstlane((unsigned)t * k_tile_bytes), kdst0 + (unsigned)(kbuf * K_STEP));
+    else
+      vdma.template issue_one_at<p - K_ITEMS>(vrw, __builtin_amdgcn_readfirstlane((unsigned)t * v_tile_bytes), vdst0 + (unsigned)(kbuf * V_STEP));
   };
+  // the whole tile at once (nobody reads buffer kbuf before the next barrier)
+  auto load_tile = [&](int t, int kbuf) {
+    static_for<0, K_ITEMS + V_ITEMS>([&](auto P) { load_piece(P, t, kbuf); });
+    if (has_seg && tid < BN) sreg = segb[min(t * BN + tid, Skv - 1)];
+  };
+  // what is left to do before the barrier that hands buffer `buf` over: the id row, and the wait for this wave's
+  // loads (they are outside the compiler's bookkeeping)
   auto store_tile = [&](int buf) {
-    unsigned char* kl = smem + K_AT + buf * K_STEP;
-    unsigned char* vl = kl + (V_AT - K_AT) + buf * (V_STEP - K_STEP);
-#pragma unroll
-    for (int i = 0; i < V_ITEMS; i++) {
-      const int item = tid + 256 * i;
-      if (item < V_TOT) {
-        const int c8 = item % (DV / 8), rq = v_quad(item / (DV / 8));
-        // odd column chunks take their columns in the order 1,0,3,2,...: at every step half the lanes
-        // write even LDS rows and half odd ones
-        const int flip = c8 & 1;
-        const unsigned sel_even = flip ? 0x07060302u : 0x05040100u, sel_odd = flip ? 0x05040100u : 0x07060302u;
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-          const unsigned sel = (j & 1) ? sel_odd : sel_even;
-          const int w = j >> 1;
-          u32x2 o;
-          o.x = __builtin_amdgcn_perm(vreg[i][1][w], vreg[i][0][w], sel);
-          o.y = __builtin_amdgcn_perm(vreg[i][3][w], vreg[i][2][w], sel);
-          *(u32x2*)(vl + TrTile64::quad_off(c8 * 8 + (j ^ flip), rq)) = o;
-        }
-      }
-    }
     if (SEG && tid < BN) ((int*)(smem + SEG_AT + buf * SEG_STEP))[tid] = sreg;
-    // the LDS-writing K loads are outside the compiler's bookkeeping: they have landed before the barrier that follows
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
 
@@ -242,6 +205,9 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
     for (int v = 0; v < 16; v++) oacc[d][v] = 0.f;
   float m_run = -INFINITY;  // reference max of the row (stale by at most 8: lazy rescale)
   float m_use = 0.f;        // m_run, or 0 while the row has seen no allowed key
+  // (Row sums by the matrix unit - a block of ones beside V^T, two more MFMAs per 32 key rows instead of 32 additions
+  // per lane - were measured and dropped: they sum the 16-bit P, the LSE then carries P's rounding (up to 2^-9
+  // relative when one key dominates a row), and the backward, which rebuilds P from the LSE, inherits it.)
   float l_run = 0.f;
   const float c = a.scale_log2;
 
@@ -283,32 +249,40 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   // and the softmax arithmetic of one 32-row half is spread under the MFMAs that follow it:
   //   slots   S0 = K[0:32] Q^T | S1 = K[32:64] Q^T | O += V[0:32]^T P0 | O += V[32:64]^T P1
   //   VALU                     | max0, exp(S0)     | max1, exp(S1)     | (LDS store of the next tile after)
-  // per-lane offsets of the V^T fragments; they carry the start of the V^T region (an opaque value, or the
-  // compiler folds it back into constants beyond the reach of an instruction offset)
-  unsigned tb[4];
-  if constexpr (STATIC_BUF) {
-    unsigned v_at = (unsigned)V_AT;
-    asm volatile("" : "+v"(v_at));
-#pragma unroll
-    for (int m = 0; m < 4; m++) tb[m] = (unsigned)TrTile64::chunk_off(ln, m, g) + v_at;
-  }
-  // Per-lane offsets of the K fragments in the swizzled tile.  Row hf*32 + ln, chunk 2 ks + g lies at
-  // (hf*32 + ln) * ROWB + ((2 ks + g) ^ swz) * 16.  With 24 chunks per row the swizzle has three bits,
-  // (ln >> 1) & 7, so only the low three bits of the chunk depend on the lane: four offsets (ks & 3), the rest is an
-  // immediate.  With 16 chunks per row it has four bits (ln & 15): one offset per k-step.
+  // Per-lane LDS byte addresses of the operands in buffer 0 (the workgroup's LDS base included), each an opaque
+  // register: every fragment read is such a register plus an immediate (plus, where the buffer index is a run-time
+  // value, one add per tile).
+  //   kfo   K fragments: row ln (+32 for the second half), chunk 2 ks + g.  With 24 chunks per row the swizzle has
+  //         three bits, so only the low three bits of the chunk depend on the lane: four offsets (ks & 3), the rest
+  //         is an immediate; with 16 chunks per row it has four bits: one offset per k-step
+  //   vfo   transposing reads of V: v-dim block d (32 columns), rows 8 h2 + 4 g ..+3 of a group of 16 key rows
+  //         (the half of the tile and the k-step are immediates: multiples of 16 rows leave the swizzle alone);
+  //         they carry V_AT, which would not fit an instruction offset for the wide heads
+  const unsigned lds0 = (unsigned)(size_t)smem;
   constexpr bool KSWZ3 = KD::CPR % 16 != 0;
   constexpr int NKFO = KSWZ3 ? (KSTEPS < 4 ? KSTEPS : 4) : KSTEPS;
-  unsigned kfo[NKFO];
+  unsigned kfo[NKFO], vfo[DVB][2];
 #pragma unroll
-  for (int j = 0; j < NKFO; j++) kfo[j] = (unsigned)(ln * KD::ROWB + (((2 * j + g) ^ KD::swz(ln)) << 4));
+  for (int j = 0; j < NKFO; j++) {
+    kfo[j] = lds0 + (unsigned)K_AT + (unsigned)(ln * KD::ROWB + (((2 * j + g) ^ KD::swz(ln)) << 4));
+    asm volatile("" : "+v"(kfo[j]));
+  }
+#pragma unroll
+  for (int d = 0; d < DVB; d++)
+#pragma unroll
+    for (int h2 = 0; h2 < 2; h2++) {
+      vfo[d][h2] = lds0 + (unsigned)V_AT + (unsigned)VD::tr_off(8 * h2 + 4 * g, 2 * d + ((lane >> 4) & 1), lane & 15);
+      asm volatile("" : "+v"(vfo[d][h2]));
+    }
+  auto ld16 = [](unsigned addr) { return *(const __attribute__((address_space(3))) v8*)addr; };
+  auto ldtr = [](unsigned a0, unsigned a1) { return tr_read8<v8>((const lds_byte*)a0, (const lds_byte*)a1); };
   auto tile_body = [&](auto masked_c, auto BUFc, int buf_rt, int t, bool has_next, int t_next) {
     constexpr bool MASKED = decltype(masked_c)::value;
     // the buffer index: a constant, or (-1) the run-time one
     const int buf = decltype(BUFc)::value >= 0 ? decltype(BUFc)::value : buf_rt;
     const int kv0 = t * BN;
-    const unsigned char* kl = smem + K_AT + buf * K_STEP;
-    const unsigned char* vl = smem + buf * V_BYTES;  // + tb[]
-    const int* sl = (const int*)(kl + (SEG_AT - K_AT) + buf * (SEG_STEP - K_STEP));
+    const unsigned kl = (unsigned)(buf * K_STEP), vl = (unsigned)(buf * V_STEP);  // + kfo[] / vfo[]
+    const int* sl = (const int*)(smem + SEG_AT + buf * SEG_STEP);
     // Masked tiles: which of the tile's 64 kv rows this lane's query row may see, one bit per row, built once per
     // tile (bounds, causality and the band of the mask extensions are a bit range; the rows of each id present among
     // the wave's query rows come from a ballot over the tile's id vector).  An element then costs a bit-field
@@ -351,7 +325,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
         s[v] = __uint_as_float((__float_as_uint(x) & keep) | (0xff800000u & ~keep));
       }
     };
-    constexpr int S1 = KSTEPS, PV0 = 2 * KSTEPS, PV1 = PV0 + 2 * DVB, NS = PV1 + 2 * DVB;
+    constexpr int PVB = DVB, S1 = KSTEPS, PV0 = 2 * KSTEPS, PV1 = PV0 + 2 * PVB, NS = PV1 + 2 * PVB;
     constexpr int AHEAD = (STATIC_BUF && DQK <= 128) ? 5 : 3, NF = AHEAD + 1;  // (the plain causal kernel up to head dim 128 has registers left for a deeper ring; seven slots gain nothing)
     v8 fr[NF];
     f32x16 s[2];
@@ -362,13 +336,15 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
       constexpr int i = decltype(I)::value;
       if constexpr (i < PV0) {
         constexpr int hf = i / KSTEPS, ks = i % KSTEPS;
-        return *(const v8*)(kl + kfo[KSWZ3 ? (ks & 3) : ks] + hf * 32 * KD::ROWB + (KSWZ3 ? 128 * (ks >> 2) : 0));
+        return ld16(kfo[KSWZ3 ? (ks & 3) : ks] + (kl + (unsigned)(hf * 32 * KD::ROWB + (KSWZ3 ? 128 * (ks >> 2) : 0))));
       } else {
-        constexpr int hf = (i - PV0) / (2 * DVB), j = (i - PV0) % (2 * DVB), kk = j / DVB, d = j % DVB;
-        if constexpr (STATIC_BUF) return *(const v8*)(vl + tb[(2 * hf + kk) ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
-        else return *(const v8*)(kl + (V_AT - K_AT) + TrTile64::chunk_off(d * 32 + ln, 2 * hf + kk, g));
+        // V^T block d, contraction over key rows 32 hf + 16 kk + {4g..4g+3, 8+4g..8+4g+3}: the order in which P holds them
+        constexpr int hf = (i - PV0) / (2 * PVB), j = (i - PV0) % (2 * PVB), kk = j / PVB, d = j % PVB;
+        constexpr unsigned rows = (unsigned)((32 * hf + 16 * kk) * VD::ROWB);
+        return ldtr(vfo[d][0] + (vl + rows), vfo[d][1] + (vl + rows));
       }
     };
+
     auto mma = [&](auto I, const v8& f) {
       constexpr int i = decltype(I)::value;
       const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -376,7 +352,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
         constexpr int hf = i / KSTEPS, ks = i % KSTEPS;
         s[hf] = MT<T>::mfma32(f, qf[ks], ks == 0 ? zero : s[hf]);
       } else {
-        constexpr int hf = (i - PV0) / (2 * DVB), j = (i - PV0) % (2 * DVB), kk = j / DVB, d = j % DVB;
+        constexpr int hf = (i - PV0) / (2 * PVB), j = (i - PV0) % (2 * PVB), kk = j / PVB, d = j % PVB;
         oacc[d] = MT<T>::mfma32(f, pf[hf][kk], oacc[d]);
       }
     };
@@ -412,7 +388,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
       if constexpr (i + AHEAD < NS) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
       mma(I, fr[i % NF]);
       // the next tile's loads, one per slot (past the last tile they re-read the last one: no branch here)
-      if constexpr (i < K_ITEMS + 4 * V_ITEMS) load_piece(I, t_next, buf ^ 1);
+      if constexpr (i < K_ITEMS + V_ITEMS) load_piece(I, t_next, buf ^ 1);
       if constexpr (i == 0) {
         if (has_seg && tid < BN) sreg = segb[min(t_next * BN + tid, Skv - 1)];
       }
@@ -432,7 +408,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
         moved1 = row_max_update(s[1], alpha1);
       }
       exp_part(I, I0{}, std::integral_constant<int, S1 + 1>{}, std::integral_constant<int, KSTEPS - 1>{});
-      exp_part(I, I1{}, std::integral_constant<int, PV0 + 1>{}, std::integral_constant<int, 2 * DVB - 1>{});
+      exp_part(I, I1{}, std::integral_constant<int, PV0 + 1>{}, std::integral_constant<int, 2 * PVB - 1>{});
       if constexpr (i == PV1 - 1) {
         if (moved1) rescale_o(alpha1);
       }
@@ -557,7 +533,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
 template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
 static int launch_fwd(const FwdArgs& a, int B, hipStream_t st) {
   constexpr int BN = 64, BM = 128;
-  constexpr int BUF = DmaTile<DQK>::BYTES + DV * TrTile64::ROW_BYTES + (SEG ? BN * 4 : 0);
+  constexpr int BUF = DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES + (SEG ? BN * 4 : 0);
   const int ntiles_max = (a.Skv + BN - 1) / BN;
   const size_t smem = 2 * (size_t)BUF + (SEG ? (size_t)(3 * ntiles_max + 16) * 4 : 0);
   TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_fwd: Skv=%d needs %zu bytes of LDS (max 163840)", a.Skv, smem);

@@ -11,6 +11,7 @@ Every op is GPU-only: CPU tensors raise, nothing falls back to torch math.
 from __future__ import annotations
 
 import math
+import weakref
 
 import torch
 from torch import Tensor
@@ -159,25 +160,25 @@ def _(inv_freq, position_ids, attention_scaling, dtype):
   return c, torch.empty_like(c)
 
 
-# verdicts of the position range check, keyed on the tensor's storage, shape and version: a model hands the same
-# position_ids tensor to every layer (and to the backward of each), so the device reduction and its host sync run
-# once per tensor, not once per call
+# verdicts of the position range check, kept per tensor object (weak reference + version counter, never the address:
+# the allocator reuses addresses): a model hands the same position_ids tensor to every layer (and to the backward of
+# each), so the device reduction and its host sync run once per tensor, not once per call
 _POS_OK: dict = {}
 
 
 def _check_positions(pos: Tensor, rows: int) -> None:
   """``cos[position_ids]`` raises IndexError for ids outside the table (model/mixtral/model.py:136-137); so does this."""
-  key = (pos.data_ptr(), tuple(pos.shape), pos._version, rows)
-  if key in _POS_OK:
+  ident = id(pos)
+  key = (pos._version, tuple(pos.shape), rows)
+  entry = _POS_OK.get(ident)
+  if entry is not None and entry[0]() is pos and entry[1] == key:
     return
   lo, hi = (int(v) for v in torch.stack((pos.min(), pos.max())).tolist()) if pos.numel() else (0, 0)
   if lo < -rows or hi >= rows:
     raise IndexError(f"position id {hi if hi >= rows else lo} is out of bounds for a rotary table of {rows} rows")
   if lo < 0:
     raise NotImplementedError("negative position ids (indexing the table from its end) are not supported")
-  if len(_POS_OK) > 64:
-    _POS_OK.clear()
-  _POS_OK[key] = True
+  _POS_OK[ident] = (weakref.ref(pos, lambda _r, ident=ident: _POS_OK.pop(ident, None)), key)
 
 
 def _rope_launch(q, k, cos, sin, pos, interleaved: int, backward: bool):
