@@ -225,6 +225,26 @@ def bench_norm_rope(dev, iters=20):
   res["rmsnorm_bwd"] = {"ms": round(ms, 4), "GBps": round(3 * n * 2 / ms / 1e6, 1)}
   del y, dy, dx, ws
 
+  # The DeepSeek-V3 configuration's own norms: RMSNorm on the q / kv latents (hidden 1536 / 512,
+  # model/deepseek_v3/model.py:373,383).  At that configuration's B=1, S=4096 a tensor is 12.6 / 4.2 MB and a launch
+  # lasts a few microseconds ("c5" entries: what a layer sees, bound by launch latency); the same kernels over
+  # 128 Mi elements ("128Mi" entries) show what they stream.
+  for hid in (1536, 512):
+    for tag, r5 in (("c5", 4096), ("128Mi", (128 << 20) // hid)):
+      x5 = torch.randn((r5, hid), generator=None, device=dev, dtype=torch.bfloat16)
+      g5 = torch.randn((r5, hid), generator=None, device=dev, dtype=torch.bfloat16)
+      w5 = torch.ones((hid,), dtype=torch.bfloat16, device=dev)
+      y5, dx5, dw5 = torch.empty_like(x5), torch.empty_like(x5), torch.empty_like(w5)
+      rs5 = torch.empty((r5,), dtype=torch.float32, device=dev)
+      ws5 = torch.empty((_lib.load().tp_rmsnorm_bwd_workspace_bytes(r5, hid),), dtype=torch.uint8, device=dev)
+      ms = timed(lambda: _lib.call("tp_rmsnorm_fwd", x5.data_ptr(), w5.data_ptr(), y5.data_ptr(), rs5.data_ptr(), r5, hid,
+                                   hid, hid, 1e-6, bf, bf, st))  # fmt: skip
+      res[f"rmsnorm_fwd_h{hid}_{tag}"] = {"ms": round(ms, 4), "GBps": round(2 * r5 * hid * 2 / ms / 1e6, 1)}
+      ms = timed(lambda: _lib.call("tp_rmsnorm_bwd", g5.data_ptr(), x5.data_ptr(), w5.data_ptr(), rs5.data_ptr(),
+                                   dx5.data_ptr(), dw5.data_ptr(), ws5.data_ptr(), r5, hid, hid, hid, hid, bf, bf, st))  # fmt: skip
+      res[f"rmsnorm_bwd_h{hid}_{tag}"] = {"ms": round(ms, 4), "GBps": round(3 * r5 * hid * 2 / ms / 1e6, 1)}
+      del x5, g5, y5, dx5, ws5
+
   Hq, Hkv, D = 32, 8, 128
   q = torch.randn((B, S, Hq, D), generator=g).to(torch.bfloat16).to(dev).transpose(1, 2)
   k = torch.randn((B, S, Hkv, D), generator=g).to(torch.bfloat16).to(dev).transpose(1, 2)
@@ -244,6 +264,22 @@ def bench_norm_rope(dev, iters=20):
                                qo.data_ptr(), ko.data_ptr(), B, Hq, Hkv, S, D, _lib.strides3(q), _lib.strides3(k),
                                _lib.strides3(qo), _lib.strides3(ko), 0, D, 0, 0, 2, 0, bf, st))  # fmt: skip
   res["rope_llama4_pairs_fwd"] = {"ms": round(ms, 4), "GBps": round(nb / ms / 1e6, 1)}
+  # The DeepSeek-V3 configuration's rotary: interleaved pairs on the 64 rotated dims of q (1, 128, 4096, 64) and of
+  # the shared key (1, 1, 4096, 64); model/deepseek_v3/model.py:84-103
+  H5, S5, D5 = 128, 4096, 64
+  q5 = torch.randn((1, S5, H5, D5), generator=None, device=dev, dtype=torch.bfloat16).transpose(1, 2)
+  k5 = torch.randn((1, S5, 1, D5), generator=None, device=dev, dtype=torch.bfloat16).transpose(1, 2)
+  qo5, ko5 = torch.empty_like(q5), torch.empty_like(k5)
+  inv5 = tpa.default_rope_frequencies(D5, 10000.0).to(dev)
+  cos5, sin5 = tpa.ops.rope_table(inv5, torch.arange(S5, device=dev)[None].float(), 1.0, torch.bfloat16)
+  cos5, sin5 = cos5.reshape(S5, D5), sin5.reshape(S5, D5)
+  nb5 = 2 * (q5.numel() + k5.numel()) * 2
+  for name, backward in (("rope_interleaved_c5_fwd", 0), ("rope_interleaved_c5_bwd", 1)):
+    ms = timed(lambda: _lib.call("tp_rope_apply", q5.data_ptr(), k5.data_ptr(), cos5.data_ptr(), sin5.data_ptr(), None,
+                                 qo5.data_ptr(), ko5.data_ptr(), 1, H5, 1, S5, D5, _lib.strides3(q5), _lib.strides3(k5),
+                                 _lib.strides3(qo5), _lib.strides3(ko5), 0, D5, 0, 0, 1, backward, bf, st))  # fmt: skip
+    res[name] = {"ms": round(ms, 4), "GBps": round(nb5 / ms / 1e6, 1)}
+  del q5, k5, qo5, ko5
   # Llama-4 qk L2 norm over the head dim of q: rows = B * S * Hq of 128
   qrows = B * S * Hq
   rstd_q = torch.empty((qrows,), dtype=torch.float32, device=dev)

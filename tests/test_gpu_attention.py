@@ -47,6 +47,29 @@ def _check(B, Hq, Hkv, S, Dqk, Dv, dtype, causal, seg=None, layout="bshd", seed=
   return out
 
 
+def _check_against_eager_16_bit(B, Hq, Hkv, S, Dqk, Dv, dtype, causal, seg=None, seed=0, std=1.0, v_std=None):
+  """For inputs outside what the stated bound is meant for (scores far larger than N(0,1) inputs give, or a softmax
+  so sharp that a single rounding of dS decides an element): the yardstick is the same formula evaluated eagerly in
+  the tensors' 16-bit dtype on the CPU, the reference's own arithmetic.  Every gradient must be within 1.25 times that
+  evaluation's error against fp64, in max-abs and in relative-L2 (which also stays under 1e-2); the forward output is
+  held to the usual bound."""
+  q = heads_view(B, Hq, S, Dqk, seed + 1, dtype, std)
+  k = heads_view(B, Hkv, S, Dqk, seed + 2, dtype, std)
+  v = heads_view(B, Hkv, S, Dv, seed + 3, dtype, std if v_std is None else v_std)
+  do = heads_view(B, Hq, S, Dv, seed + 4, dtype, 1.0)
+  sm_scale = 1.0 / math.sqrt(Dv)
+  out, _, dq, dk, dv = _run(q, k, v, do, seg, causal, sm_scale)
+  ref = orc.attention_grads_ref(q, k, v, do, seg, causal, sm_scale, torch.float64)
+  eager = orc.attention_grads_ref(q, k, v, do, seg, causal, sm_scale, dtype)
+  assert_close(out, ref[0], "out")
+  for name, got, e16, r64 in zip(("dq", "dk", "dv"), (dq, dk, dv), eager[1:], ref[1:]):
+    err_gpu, err_16 = (got.double().cpu() - r64).abs(), (e16.double() - r64).abs()
+    assert torch.isfinite(got.float()).all(), name
+    assert err_gpu.max().item() <= 1.25 * err_16.max().item(), (name, err_gpu.max().item(), err_16.max().item())
+    rl_gpu, rl_16 = (err_gpu.norm() / r64.norm()).item(), (err_16.norm() / r64.norm()).item()
+    assert rl_gpu <= 1e-2 and rl_gpu <= 1.25 * rl_16 + 1e-3, (name, rl_gpu, rl_16)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize(
   "B,Hq,Hkv,S,Dqk,Dv",
@@ -64,12 +87,8 @@ def test_causal_fwd_bwd(dtype, B, Hq, Hkv, S, Dqk, Dv):
   _check(B, Hq, Hkv, S, Dqk, Dv, dtype, True)
 
 
-@pytest.mark.parametrize("seed", range(12))
-def test_randomised_shapes_and_segment_layouts(seed):
-  """Seeded random draws over what the kernels branch on: length (around tile edges too), GQA ratio, head dims, dtype,
-  causality, and the id layout (none, packed documents, short documents of a few rows, unsorted ids with repeats):
-  masked tiles are resolved through per-tile bit masks and per-workgroup tile lists, whose corner cases are lengths
-  and document boundaries that fall on or next to tile and wave boundaries."""
+def _random_draw(seed):
+  """One seeded draw over what the kernels branch on (see test_randomised_shapes_and_segment_layouts)."""
   rng = random.Random(1000 + seed)
   Dqk, Dv = rng.choice([(64, 64), (128, 128), (128, 128), (192, 128)])
   Hkv = rng.choice([1, 2])
@@ -88,7 +107,30 @@ def test_randomised_shapes_and_segment_layouts(seed):
   else:
     g = torch.Generator().manual_seed(seed)
     seg = torch.randint(-3, 4, (B, S), generator=g, dtype=torch.int32)
-  _check(B, Hq, Hkv, S, Dqk, Dv, dtype, causal, seg=seg, seed=10 * seed)
+  return dict(B=B, Hq=Hq, Hkv=Hkv, S=S, Dqk=Dqk, Dv=Dv, dtype=dtype, causal=causal, seg=seg, seed=10 * seed)
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_randomised_shapes_and_segment_layouts(seed):
+  """Seeded random draws over what the kernels branch on: length (around tile edges too), GQA ratio, head dims, dtype,
+  causality, and the id layout (none, packed documents, short documents of a few rows, unsorted ids with repeats):
+  masked tiles are resolved through per-tile bit masks and per-workgroup tile lists, whose corner cases are lengths
+  and document boundaries that fall on or next to tile and wave boundaries."""
+  d = _random_draw(seed)
+  _check(d["B"], d["Hq"], d["Hkv"], d["S"], d["Dqk"], d["Dv"], d["dtype"], d["causal"], seg=d["seg"], seed=d["seed"])
+
+
+def test_sharp_softmax_draw_against_the_eager_16_bit_evaluation():
+  """The one draw of 248 further seeds of the sweep above that leaves the per-element bound (seed 144: 192/128 heads,
+  65 rows, seven interleaved ids, bf16; one element of dq 7e-4 over ``2e-2 + 2^-7 |ref|``).  With a handful of allowed
+  keys per row the softmax is sharp, dS is large, and its one rounding to 16 bits is what that element carries: no
+  16-bit evaluation does better there.  So this case is held to the yardstick that is independent of the bound's
+  constants: the same formula evaluated eagerly in bf16 on the CPU (the reference's own arithmetic).  Every gradient
+  must be within 1.25 times that evaluation's error against fp64, in max-abs and in relative-L2; the forward output
+  and the relative-L2 limit of 1e-2 hold as everywhere."""
+  d = _random_draw(144)
+  assert (d["Dqk"], d["Dv"], d["S"], d["dtype"]) == (192, 128, 65, torch.bfloat16) and d["seg"] is not None
+  _check_against_eager_16_bit(d["B"], d["Hq"], d["Hkv"], d["S"], d["Dqk"], d["Dv"], d["dtype"], d["causal"], seg=d["seg"], seed=d["seed"])
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,S,Skv,Dqk,Dv", [(1, 4, 2, 130, 130, 128, 128), (2, 2, 2, 64, 300, 64, 64), (1, 2, 1, 257, 100, 128, 128)])
@@ -101,11 +143,10 @@ def test_full_attention_fwd_bwd(B, Hq, Hkv, S, Skv, Dqk, Dv):
 def test_running_max_moves_often(seed):
   # large score spread: the row maximum keeps growing by more than the lazy-rescale threshold, in either
   # half of a KV tile, so the rescale paths (including the one deferred past the first half's P V) run
-  # (q and k are 2.5x / 3x the N(0,1) scale the tolerance is stated for: the scores, and with them the rounding
-  # errors of P and dS that dq = sm_scale dS K and dk = sm_scale dS^T Q multiply by the larger q / k values, grow
-  # with the square of that factor, and so does the absolute bound here; relative-L2 stays at 1e-2)
-  _check(1, 4, 2, 512, 128, 128, torch.bfloat16, True, seed=10 * seed, std=2.5, v_std=1.0, grad_abs=2e-2 * 2.5**2)
-  _check(1, 2, 2, 300, 64, 64, torch.bfloat16, False, seed=10 * seed + 5, std=3.0, v_std=1.0, grad_abs=2e-2 * 3.0**2)
+  # (q and k are 2.5x / 3x the N(0,1) scale the tolerance is stated for, so the gradients are held to the eager 16-bit
+  # evaluation of the same inputs instead of a bound scaled to fit)
+  _check_against_eager_16_bit(1, 4, 2, 512, 128, 128, torch.bfloat16, True, seed=10 * seed, std=2.5, v_std=1.0)
+  _check_against_eager_16_bit(1, 2, 2, 300, 64, 64, torch.bfloat16, False, seed=10 * seed + 5, std=3.0, v_std=1.0)
 
 
 def test_contiguous_bhsd_layout_and_scale():
@@ -221,6 +262,33 @@ def test_attention_module_matches_eager_branch(kernel):
   ref = orc.eager_attention(q.float(), k.float(), v.float(), mask)
   assert_close(out, ref, f"kernel={kernel}")
   assert m.partition_spec is None and out.transpose(1, 2).is_contiguous()
+
+
+def test_mask_verdict_is_not_reused_for_a_new_mask_at_the_same_address():
+  """A model rebuilds its additive mask every forward (model/llama/model.py:347-355).  The allocator hands the freed
+  mask's memory to the next one, so a verdict remembered by address would let a padded mask of the same shape pass as
+  the causal one; the verdict belongs to the tensor object."""
+  from torchprime_amd import attention as att
+
+  B, H, S, D = 1, 2, 96, 64
+  q, k, v = (heads_view(B, H, S, D, s, torch.bfloat16).to(DEV) for s in (1, 2, 3))
+  m = tpa.AttentionModule(_cfg(None, H, H))
+  causal = orc.causal_additive_mask(S).to(DEV)
+  m(q, k, v, causal)  # accepted, verdict remembered
+  m(q, k, v, causal)  # same tensor again: no second check needed
+  ptr, n_entries = causal.data_ptr(), len(att._MASK_VERDICTS)
+  assert n_entries >= 1
+  del causal
+  assert len(att._MASK_VERDICTS) == n_entries - 1  # the entry left with the tensor
+  hit = False
+  for _ in range(8):  # (the allocator normally reuses the block at once; a few tries in case it does not)
+    padded = orc.causal_additive_mask(S).to(DEV)
+    padded[..., : S // 4] = float("-inf")  # a padded batch: the first keys masked for every query
+    hit = hit or padded.data_ptr() == ptr
+    with pytest.raises(NotImplementedError):
+      m(q, k, v, padded)
+    del padded
+  assert hit, "the allocator never reused the freed mask's address: the test did not exercise the aliasing"
 
 
 def test_attention_module_scale_uses_v_head_dim():

@@ -175,3 +175,27 @@ def test_cross_entropy_all_ignored_is_nan_like_torch_and_vocab_128k_row():
   ign = torch.full((1, 3), -100)
   assert torch.isnan(tpa.cross_entropy_loss(logits.to(DEV), ign.to(DEV), V))
   assert torch.isnan(orc.cross_entropy_loss(logits, ign, V))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_cross_entropy_with_a_masked_vocabulary_range(dtype):
+  """-inf logits (a masked range of the vocabulary, here the low column indices, which every thread of the kernel
+  meets first, and a block in the middle) add nothing to the row's sum: the loss and the gradient stay finite and
+  match the oracle, and the masked columns get gradient 0."""
+  B, S, V = 2, 9, 5000
+  logits = randn((B, S, V), 71, dtype, 2.0)
+  logits[:, :, :2100] = float("-inf")
+  logits[:, :, 3000:3300] = float("-inf")
+  labels = torch.randint(2100, 3000, (B, S), generator=torch.Generator().manual_seed(72))
+  ld = logits.to(DEV).requires_grad_(True)
+  loss = tpa.cross_entropy_loss(ld, labels.to(DEV), V)
+  loss.backward()
+  l64 = logits.double().requires_grad_(True)
+  ref = orc.cross_entropy_loss(l64, labels, V)
+  ref.backward()
+  assert torch.isfinite(loss).item()
+  assert abs(loss.item() - ref.item()) <= 2e-6 * max(1.0, abs(ref.item()))
+  assert torch.isfinite(ld.grad).all().item()
+  assert ld.grad[:, :, :2100].abs().max().item() == 0 and ld.grad[:, :, 3000:3300].abs().max().item() == 0
+  assert_close(ld.grad, l64.grad, "dlogits", max_abs=1e-7 if dtype == torch.float32 else 1e-4, rel_l2=1e-5 if dtype == torch.float32 else 5e-3)
+

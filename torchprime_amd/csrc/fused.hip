@@ -194,8 +194,11 @@ __global__ __launch_bounds__(256) void xent_fwd_kernel(const T* __restrict__ log
       float mx = x[0];
 #pragma unroll
       for (int e = 1; e < E; e++) mx = fmaxf(mx, x[e]);
+      // (a vector of -inf logits - a masked range of the vocabulary - while the thread has seen nothing finite yet:
+      // m stays -inf, and exp(x - m) would be exp(NaN); such logits add nothing)
+      if (mx == -INFINITY) continue;
       if (mx > m) {
-        acc *= __expf(m - mx);
+        acc *= __expf(m - mx);  // (m = -inf the first time: acc is 0 and exp(-inf) = 0)
         m = mx;
       }
 #pragma unroll
@@ -204,6 +207,7 @@ __global__ __launch_bounds__(256) void xent_fwd_kernel(const T* __restrict__ log
   }
   for (int c = (vec ? nvec * E : 0) + threadIdx.x; c < V; c += 256) {
     const float x = Elem<T>::to_f(lr[c]);
+    if (x == -INFINITY) continue;
     if (x > m) {
       acc *= __expf(m - x);
       m = x;
