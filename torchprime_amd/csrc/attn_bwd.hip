@@ -1684,6 +1684,266 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------------
+// dQ, the plain kernels (no segment ids, no mask extensions; equal head dims up to 128)
+// ------------------------------------------------------------------------------------------------
+// Shaped like the forward: workgroup = 4 waves = 128 query rows of one (batch, head), two workgroups per CU (so two
+// waves per SIMD whose barriers are independent of each other); Q and dO fragments, LSE and delta stay in registers;
+// K and V tiles of 64 rows travel into LDS by loads that write LDS themselves (two buffers, one barrier per tile, no
+// staging registers, no second copy of K: the K^T operand of dQ^T += K^T dS^T comes out of transposing reads).
+// S^T = K Q^T and dP^T = V dO^T are computed transposed, so LSE and delta are per-lane scalars and dS^T, converted to
+// 16 bit, is the B operand of the accumulating product as it stands.  -delta joins dP through the matrix unit (one
+// more k-step per block: a column of ones on the V side, the lane's -delta split into two 16-bit values on the dO
+// side) instead of 32 additions per lane and tile: the kernels are bound by the instructions a SIMD can issue.
+// Per tile and 32-row half h of it:  S_h (KS MFMAs) | dP_h (KS + 1) | ... | dQ += K_h^T dS_h (2 DB), with P_h computed
+// under dP_h and dS_h under what follows.
+template <typename T, int D, bool CAUSAL>
+__global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs a) {
+  typedef typename MT<T>::v8 v8;
+  constexpr int BN = 64, BM = 128, KS = D / 16, DB = D / 32;
+  typedef DmaTile<D, true> KT;
+  constexpr int T_BYTES = KT::BYTES, K_AT = 0, V_AT = 2 * T_BYTES;
+  constexpr int NLOAD = KT::PER_WAVE;  // loads per wave, tile and tensor
+
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, ln = lane & 31;
+  const int n_qt = (a.Sq + BM - 1) / BM;
+  int tile, inner, group;
+  if (!xcd_map(n_qt, a.n_rep, a.B * a.Hkv, tile, inner, group)) return;
+  const int qt = n_qt - 1 - tile;  // the longest rows first
+  const int b = group / a.Hkv, hk = group - b * a.Hkv, h = hk * a.n_rep + inner;
+  const int q0 = qt * BM, wq0 = q0 + wave * 32;
+  const int Sq = a.Sq, Skv = a.Skv;
+  const int kv_end = CAUSAL ? min(Skv, q0 + BM) : Skv;
+  const int ntiles = (kv_end + BN - 1) / BN;
+
+  // ---- Q, dO fragments (B operands: lane = query column), per-lane LSE / -delta
+  const int qrow = wq0 + ln, qrow_c = min(qrow, Sq - 1);
+  v8 qf[KS], dof[KS];
+  {
+    const T* qp = (const T*)a.q + b * a.qs[0] + h * a.qs[1] + qrow_c * a.qs[2] + 8 * g;
+    const T* dp = (const T*)a.dout + b * a.dos[0] + h * a.dos[1] + qrow_c * a.dos[2] + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[ks] = *(const v8*)(qp + 16 * ks);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) dof[ks] = *(const v8*)(dp + 16 * ks);
+  }
+  const int64_t ro = ((int64_t)b * a.Hq + h) * Sq + qrow_c;
+  const float lraw = a.lse[ro];
+  const float nlse = (lraw == -INFINITY) ? -INFINITY : -lraw * LOG2E;  // (a row without keys: P = exp2(-inf) = 0)
+  const float ndelta = a.delta[ro];                                     // -rowsum(dO o O)
+  v8 ones_a, ndelta_b;
+  {
+    const float hi = (float)(T)ndelta, lo = ndelta - hi;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      ones_a[e] = (T)((g == 0 && e < 2) ? 1.0f : 0.0f);
+      ndelta_b[e] = (T)0.0f;
+    }
+    if (g == 0) { ndelta_b[0] = (T)hi; ndelta_b[1] = (T)lo; }
+    asm volatile("" : "+v"(ones_a), "+v"(ndelta_b));
+  }
+
+  // ---- loads
+  const unsigned k_tile_bytes = (unsigned)(BN * a.ks[2] * 2), v_tile_bytes = (unsigned)(BN * a.vs[2] * 2);
+  KT kdma, vdma;
+  kdma.init(a.ks[2], wave, lane);
+  vdma.init(a.vs[2], wave, lane);
+  const u32x4 krw = make_rsrc_words((const T*)a.k + b * a.ks[0] + hk * a.ks[1], span_bytes(Skv, a.ks[2], D));
+  const u32x4 vrw = make_rsrc_words((const T*)a.v + b * a.vs[0] + hk * a.vs[1], span_bytes(Skv, a.vs[2], D));
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const unsigned lds_base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)smem);
+  const unsigned kdst0 = lds_base + (unsigned)K_AT + (unsigned)(wave_s * NLOAD * 1024);
+  const unsigned vdst0 = lds_base + (unsigned)V_AT + (unsigned)(wave_s * NLOAD * 1024);
+  auto load_piece = [&](auto Pc, int t, int buf) {
+    constexpr int p = decltype(Pc)::value;
+    if constexpr (p < NLOAD)
+      kdma.template issue_one_at<p>(krw, __builtin_amdgcn_readfirstlane((unsigned)t * k_tile_bytes), kdst0 + (unsigned)(buf * T_BYTES));
+    else
+      vdma.template issue_one_at<p - NLOAD>(vrw, __builtin_amdgcn_readfirstlane((unsigned)t * v_tile_bytes), vdst0 + (unsigned)(buf * T_BYTES));
+  };
+
+  // ---- per-lane LDS addresses in buffer 0 (opaque registers; reads add immediates)
+  const unsigned lds0 = (unsigned)(size_t)smem;
+  constexpr bool SWZ3 = KT::CPR % 16 != 0;
+  constexpr int NFO = SWZ3 ? (KS < 4 ? KS : 4) : KS;
+  unsigned kfo[NFO], ktr[DB][2];
+#pragma unroll
+  for (int j = 0; j < NFO; j++) {
+    kfo[j] = lds0 + (unsigned)(ln * KT::ROWB + (((2 * j + g) ^ KT::swz(ln)) << 4));  // K; V lies V_AT further on
+    asm volatile("" : "+v"(kfo[j]));
+  }
+#pragma unroll
+  for (int d = 0; d < DB; d++)
+#pragma unroll
+    for (int h2 = 0; h2 < 2; h2++) {
+      ktr[d][h2] = lds0 + (unsigned)KT::tr_off(8 * h2 + 4 * g, 2 * d + ((lane >> 4) & 1), lane & 15);
+      asm volatile("" : "+v"(ktr[d][h2]));
+    }
+  auto ld16 = [](unsigned addr) { return *(const __attribute__((address_space(3))) v8*)addr; };
+  auto ldtr = [](unsigned a0, unsigned a1) { return tr_read8<v8>((const lds_byte*)a0, (const lds_byte*)a1); };
+
+  f32x16 dqacc[DB];
+#pragma unroll
+  for (int d = 0; d < DB; d++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) dqacc[d][v] = 0.f;
+  const float c = a.scale_log2;
+  const int wq_last = wq0 + 31;
+
+  // slots of a tile: S0 | dP0 | S1 | dP1 | dQ0 | dQ1
+  constexpr int KSD = KS + 1, A2 = 2 * DB;
+  constexpr int P_S0 = 0, P_D0 = KS, P_S1 = P_D0 + KSD, P_D1 = P_S1 + KS, P_Q0 = P_D1 + KSD, P_Q1 = P_Q0 + A2, NS = P_Q1 + A2;
+  constexpr int AHEAD = 4, NF = AHEAD + 1;
+
+  auto tile_body = [&](auto masked_c, auto BUFc, int t, int t_next) {
+    constexpr bool MASKED = decltype(masked_c)::value;
+    constexpr int buf = decltype(BUFc)::value;
+    constexpr unsigned kl = K_AT + buf * T_BYTES, vl = V_AT + buf * T_BYTES;
+    const int kv0 = t * BN;
+    // masked tiles: which of the tile's 64 kv rows this lane's query row may see, as bits (value v of a half: bit
+    // 8 (v / 4) + v % 4 after the shift by 4 g)
+    unsigned kbits[2] = {0u, 0u};
+    if (MASKED) {
+      int hi = min(Skv - kv0, BN);
+      if (CAUSAL) hi = min(hi, qrow - kv0 + 1);
+      if (qrow >= Sq) hi = 0;
+      unsigned long long m = hi > 0 ? (~0ull >> (64 - hi)) : 0ull;
+      kbits[0] = (unsigned)m >> (4 * g);
+      kbits[1] = (unsigned)(m >> 32) >> (4 * g);
+    }
+    v8 fr[NF];
+    f32x16 s[2], dp[2];
+    v8 df[2][2];
+    auto has_frag = [](int i) constexpr { return i != P_D0 && i != P_D1; };
+    auto frag = [&](auto I) -> v8 {
+      constexpr int i = decltype(I)::value;
+      auto rowfrag = [&](unsigned base, int hf, int ks) {
+        return ld16(kfo[SWZ3 ? (ks & 3) : ks] + (base + (unsigned)(hf * 32 * KT::ROWB + (SWZ3 ? 128 * (ks >> 2) : 0))));
+      };
+      if constexpr (i < P_D0) return rowfrag(kl, 0, i - P_S0);
+      else if constexpr (i < P_S1) return rowfrag(vl, 0, i - P_D0 - 1);
+      else if constexpr (i < P_D1) return rowfrag(kl, 1, i - P_S1);
+      else if constexpr (i < P_Q0) return rowfrag(vl, 1, i - P_D1 - 1);
+      else {
+        // K^T block d, contraction over kv rows 32 hf + 16 kk + {4g..4g+3, 8+4g..8+4g+3}: the order in which dS holds them
+        constexpr int hf = i >= P_Q1 ? 1 : 0, j = i - (hf ? P_Q1 : P_Q0), kk = j / DB, d = j % DB;
+        constexpr unsigned rows = (unsigned)((32 * hf + 16 * kk) * KT::ROWB);
+        return ldtr(ktr[d][0] + (kl + rows), ktr[d][1] + (kl + rows));
+      }
+    };
+    auto mma = [&](auto I, const v8& f) {
+      constexpr int i = decltype(I)::value;
+      const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if constexpr (i < P_D0) s[0] = MT<T>::mfma32(f, qf[i], i == 0 ? zero : s[0]);
+      else if constexpr (i == P_D0) dp[0] = MT<T>::mfma32(ones_a, ndelta_b, zero);
+      else if constexpr (i < P_S1) dp[0] = MT<T>::mfma32(f, dof[i - P_D0 - 1], dp[0]);
+      else if constexpr (i < P_D1) s[1] = MT<T>::mfma32(f, qf[i - P_S1], i == P_S1 ? zero : s[1]);
+      else if constexpr (i == P_D1) dp[1] = MT<T>::mfma32(ones_a, ndelta_b, zero);
+      else if constexpr (i < P_Q0) dp[1] = MT<T>::mfma32(f, dof[i - P_D1 - 1], dp[1]);
+      else {
+        constexpr int hf = i >= P_Q1 ? 1 : 0, j = i - (hf ? P_Q1 : P_Q0), kk = j / DB, d = j % DB;
+        dqacc[d] = MT<T>::mfma32(f, df[hf][kk], dqacc[d]);
+      }
+    };
+    // elements [k 16 / LEN, (k + 1) 16 / LEN) of half HF in slot START + k: P = exp2(s c - lse) (masked) ...
+    auto p_piece = [&](auto I, auto HFc, auto STARTc, auto LENc) {
+      constexpr int i = decltype(I)::value, hf = decltype(HFc)::value, st = decltype(STARTc)::value, len = decltype(LENc)::value;
+      if constexpr (i >= st && i < st + len) {
+        constexpr int k = i - st, lo = (k * 16 + len - 1) / len, hi = ((k + 1) * 16 + len - 1) / len;
+#pragma unroll
+        for (int v = lo; v < hi; v++) {
+          float pv = fast_exp2(__builtin_fmaf(s[hf][v], c, nlse));
+          if (MASKED) pv = __builtin_bit_cast(float, __builtin_bit_cast(int, pv) & __builtin_amdgcn_sbfe((int)kbits[hf], 8 * (v / 4) + (v % 4), 1));
+          asm volatile("" : "+v"(pv));  // keeps the computation in this slot
+          s[hf][v] = pv;
+        }
+      }
+    };
+    // ... and dS = P o (dP - delta), packed as soon as the eight values of an operand are there
+    auto ds_piece = [&](auto I, auto HFc, auto STARTc, auto LENc) {
+      constexpr int i = decltype(I)::value, hf = decltype(HFc)::value, st = decltype(STARTc)::value, len = decltype(LENc)::value;
+      if constexpr (i >= st && i < st + len) {
+        constexpr int k = i - st, lo = (k * 16 + len - 1) / len, hi = ((k + 1) * 16 + len - 1) / len;
+#pragma unroll
+        for (int v = lo; v < hi; v++) {
+          float dsv = s[hf][v] * dp[hf][v];
+          asm volatile("" : "+v"(dsv));
+          dp[hf][v] = dsv;
+        }
+        static_for<0, 2>([&](auto H) {
+          constexpr int hh = decltype(H)::value;
+          if constexpr (8 * hh + 8 > lo && 8 * hh + 8 <= hi) {
+            const f32x16& x = dp[hf];
+            df[hf][hh] = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4], x[8 * hh + 5],
+                                  x[8 * hh + 6], x[8 * hh + 7]);
+          }
+        });
+      }
+    };
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 1> I1;
+    static_for<0, AHEAD>([&](auto I) { fr[decltype(I)::value % NF] = frag(I); });
+    static_for<0, NS>([&](auto I) {
+      constexpr int i = decltype(I)::value;
+      if constexpr (i + AHEAD < NS && has_frag(i + AHEAD)) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
+      mma(I, fr[i % NF]);
+      // the next tile's loads, one per slot (past the last tile they re-read the last one: no branch here)
+      if constexpr (i < 2 * NLOAD) load_piece(I, t_next, buf ^ 1);
+      // P0 under dP0 (its S is complete from slot P_D0 on), dS0 under S1 (dP0 is complete from P_S1 on),
+      // P1 under dP1, dS1 under dQ0; each group ends before the MFMAs that need its operand
+      p_piece(I, I0{}, std::integral_constant<int, P_D0 + 1>{}, std::integral_constant<int, KSD - 1>{});
+      ds_piece(I, I0{}, std::integral_constant<int, P_S1 + 1>{}, std::integral_constant<int, KS - 1>{});
+      p_piece(I, I1{}, std::integral_constant<int, P_D1 + 1>{}, std::integral_constant<int, KSD - 1>{});
+      ds_piece(I, I1{}, std::integral_constant<int, P_Q0 + 1>{}, std::integral_constant<int, A2 - 1>{});
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next tile has landed
+  };
+
+  if (ntiles > 0) {
+    static_for<0, 2 * NLOAD>([&](auto P) { load_piece(P, 0, 0); });
+  }
+  __builtin_amdgcn_s_waitcnt(0);  // the fragments above and the first tile have landed (see the forward kernel)
+  __syncthreads();
+  auto iteration = [&](auto BUFc, int t) {
+    const int kv0 = t * BN;
+    const int t_next = t + 1 < ntiles ? t + 1 : t;
+    const bool skip = CAUSAL && kv0 > wq_last;
+    const bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0) || (wq0 + 32 > Sq);
+    if (skip) {
+      constexpr int buf = decltype(BUFc)::value;
+      if (t + 1 < ntiles) {
+        static_for<0, 2 * NLOAD>([&](auto P) { load_piece(P, t_next, buf ^ 1); });
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+    } else if (need_mask) {
+      tile_body(std::true_type{}, BUFc, t, t_next);
+    } else {
+      tile_body(std::false_type{}, BUFc, t, t_next);
+    }
+    __syncthreads();
+  };
+  for (int t = 0; t < ntiles; t += 2) {
+    iteration(std::integral_constant<int, 0>{}, t);
+    if (t + 1 < ntiles) iteration(std::integral_constant<int, 1>{}, t + 1);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-writing load outlives the workgroup
+
+  if (qrow < Sq) {
+    T* dqp = (T*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qrow * a.dqs[2];
+    const float sc = a.sm_scale;
+#pragma unroll
+    for (int d = 0; d < DB; d++)
+#pragma unroll
+      for (int vq = 0; vq < 4; vq++) {
+        const f32x16& o = dqacc[d];
+        *(u32x2*)(dqp + d * 32 + 8 * vq + 4 * g) =
+            pack4<T>(o[4 * vq] * sc, o[4 * vq + 1] * sc, o[4 * vq + 2] * sc, o[4 * vq + 3] * sc);
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
 // host dispatch
 // ------------------------------------------------------------------------------------------------
 template <typename K>
@@ -1733,7 +1993,20 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
   }
   mark(ev, 2, st);
   // dQ
-  {
+  if constexpr (!SEG && DQK == DV && DQK <= 128) {
+    constexpr int BM = 128;
+    const size_t smem = 4 * (size_t)DmaTile<DQK, true>::BYTES;
+    auto kern = attn_bwd_dq_plain_kernel<T, DQK, CAUSAL>;
+    static bool attr_set = false;
+    if (!attr_set) {
+      int rc = set_max_lds(kern, "tp_attn_bwd(dq)");
+      if (rc) return rc;
+      attr_set = true;
+    }
+    kern<<<dim3(xcd_grid((a.Sq + BM - 1) / BM, a.n_rep, a.B * a.Hkv)), dim3(256), smem, st>>>(a);
+    int rc = check_launch("tp_attn_bwd(dq)");
+    if (rc) return rc;
+  } else {
     // eight waves (two per SIMD) where a wave's registers fit in half a SIMD's file
     // (the non-causal 128-wide variant does not fit 256 registers without spilling: it keeps four waves)
     constexpr int NW = (DQK == DV && (DQK <= 64 || (DQK <= 128 && CAUSAL))) ? 8 : 4;
