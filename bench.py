@@ -595,6 +595,231 @@ def cpu_baseline(max_seconds=24.0):
   }  # fmt: skip
 
 
+# ---- summaries of rocprofv3 runs of this script -----------------------------------------------------------------
+_PRE = "from the repository root, after `cd /tmp && export TMPDIR=/tmp && cd -`"
+_PROFILE_COMMANDS = {
+  "kt_c2": "rocprofv3 --kernel-trace --stats --output-format csv -d {d}/kt_c2 -o kt -- python3 bench.py --steps 10 --warmup 3 --no-cpu --no-extra > {d}/kt_c2.log",
+  "pmc_fetch": "rocprofv3 --pmc FETCH_SIZE --output-format csv -d {d}/pmc_fetch -o p -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-extra --calib-copy",
+  "pmc_write": "rocprofv3 --pmc WRITE_SIZE --output-format csv -d {d}/pmc_write -o p -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-extra --calib-copy",
+  "pmc_a": "rocprofv3 --pmc SQ_BUSY_CU_CYCLES SQ_VALU_MFMA_BUSY_CYCLES SQ_ACTIVE_INST_VALU SQ_VALU_MFMA_COEXEC_CYCLES SQ_INSTS_VALU SQ_WAIT_INST_ANY SQ_ACTIVE_INST_ANY SQ_WAVE_CYCLES --output-format csv -d {d}/pmc_a -o p -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-extra > {d}/pmc_a.log",
+  "pmc_b": "rocprofv3 --pmc SQ_INSTS_MFMA SQ_INSTS_LDS SQ_LDS_ADDR_CONFLICT SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE SQ_ACTIVE_INST_LDS SQ_WAIT_INST_LDS SQ_BUSY_CU_CYCLES --output-format csv -d {d}/pmc_b -o p -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-extra",
+  "kt_oc": "rocprofv3 --kernel-trace --stats --output-format csv -d {d}/kt_oc -o kt -- python3 bench.py --other-configs all --steps 5 > {d}/kt_oc.log",
+  "kt_extra": "rocprofv3 --kernel-trace --stats --output-format csv -d {d}/kt_extra -o kt -- python3 bench.py --steps 10 --warmup 3 --no-cpu > {d}/kt_extra.log",
+}  # fmt: skip
+
+
+def _short_kernel_name(n):
+  """tp::name<dtype, integer / boolean template arguments in declaration order> from a mangled or demangled name."""
+  import re
+
+  m = re.match(r"_ZN2tp\d+([a-z_0-9]+?)I(.*)", n)
+  if not m:
+    return re.sub(r"^void ", "", n).split("(")[0][:70]
+  rest = m.group(2)
+  ty = "f16" if rest.startswith("DF16_") else "bf16" if rest.startswith("DF16b") else "f32" if rest.startswith("f") else "?"
+  ints = ",".join(re.findall(r"L[ib](\d+)E", rest))
+  return f"tp::{m.group(1)}<{ty},{ints}>"
+
+
+def _attn_kernel_of(name):
+  for key, short in (("dkdv", "attn_bwd_dkdv"), ("bwd_dq", "attn_bwd_dq"), ("attn_fwd", "attn_fwd"), ("delta", "attn_delta")):
+    if key in name:
+      return short
+  return None
+
+
+def summarize_profiles(d, commit):
+  """Turn the rocprofv3 output of the commands in _PROFILE_COMMANDS (run with -d ``d``/<name>, this script's stdout
+  in ``d``/<name>.log) into the text summaries and the traffic data file under profiles/.  Parts whose input is
+  absent are left as they are."""
+  import collections
+  import csv
+
+  prof = os.path.join(ROOT, "profiles")
+  have = lambda *rel: all(os.path.exists(os.path.join(d, r)) for r in rel)  # noqa: E731
+  bench_line = lambda rel: [json.loads(l) for l in open(os.path.join(d, rel)) if l.startswith("{")][-1]  # noqa: E731
+  cmd = lambda name: "    " + _PROFILE_COMMANDS[name].format(d=d)  # noqa: E731
+  head = f"Library and script at commit {commit}.  "
+
+  def stats_table(rel, keep, min_pct=0.0):
+    rows = list(csv.DictReader(open(os.path.join(d, rel))))
+    out = ["| kernel | calls | avg us | min us | max us | % of GPU time |", "|---|---:|---:|---:|---:|---:|"]
+    for r in rows:
+      if keep(r["Name"]) and float(r["Percentage"]) >= min_pct:
+        out.append(f"| {_short_kernel_name(r['Name'])} | {r['Calls']} | {float(r['AverageNs']) / 1e3:.1f} | "
+                   f"{float(r['MinNs']) / 1e3:.1f} | {float(r['MaxNs']) / 1e3:.1f} | {float(r['Percentage']):.2f} |")
+    return out
+
+  ours = lambda n: n.startswith("_ZN2tp") or "tp::" in n  # noqa: E731
+
+  # 1. the headline workload alone: per-kernel averages with and without the warm-up launches
+  if have("kt_c2/kt_kernel_stats.csv", "kt_c2/kt_kernel_trace.csv", "kt_c2.log"):
+    b = bench_line("kt_c2.log")
+    per = collections.defaultdict(list)
+    for r in csv.DictReader(open(os.path.join(d, "kt_c2/kt_kernel_trace.csv"))):
+      k = _attn_kernel_of(r["Kernel_Name"])
+      if k and "f32" not in r["Kernel_Name"]:
+        per[k].append((int(r["Start_Timestamp"]), int(r["End_Timestamp"]) - int(r["Start_Timestamp"])))
+    warm, steps = b["warmup"], b["steps"]
+    o = ["# Kernel trace: attention fwd+bwd at the Llama-3-8B shape (S=8192), the headline workload alone\n",
+         head + "Workload: q (4,32,8192,128), k/v (4,8,8192,128) bf16, causal, no segment ids, inputs resident in HBM.",
+         f"One MI355X, {warm + steps} steps ({warm} warm-up + {steps} timed); nothing else runs in the process.\n",
+         f"Command ({_PRE}):\n", cmd("kt_c2"), "",
+         "`kt_kernel_stats.csv` (times in microseconds; template arguments are the integer and boolean ones in declaration order):\n"]
+    o += stats_table("kt_c2/kt_kernel_stats.csv", ours) + [""]
+    o += ["From `kt_kernel_trace.csv`, the same launches split into warm-up and timed ones, beside the averages this script",
+          "measures itself with HIP events on the launch stream (profiler attached):\n",
+          "| kernel | launches | avg us, all | avg us, warm-up launches | avg us, timed launches | bench.py events, us |",
+          "|---|---:|---:|---:|---:|---:|"]
+    timed_avg = {}
+    for k in ("attn_fwd", "attn_delta", "attn_bwd_dkdv", "attn_bwd_dq"):
+      v = [x[1] for x in sorted(per[k])]
+      if len(v) != warm + steps:
+        o.append(f"| {k} | {len(v)} | (expected {warm + steps} launches) | | | |")
+        continue
+      timed_avg[k] = sum(v[warm:]) / steps
+      o.append(f"| {k} | {len(v)} | {sum(v) / len(v) / 1e3:.1f} | {sum(v[:warm]) / warm / 1e3:.1f} | {timed_avg[k] / 1e3:.1f} | "
+               f"{b['kernels'][k]['ms'] * 1e3:.1f} |")
+    dom = b["roofline"]["kernel"]
+    unit = b["config"]["algorithmic_flop_per_step"] / 6.0
+    share = {"attn_fwd": 2.0, "attn_bwd_dkdv": 3.0, "attn_bwd_dq": 1.0}[dom]
+    if dom in timed_avg:
+      t = timed_avg[dom] * 1e-9
+      o += ["", f"The same run's bench line: ms_per_step {b['ms_per_step']}, value {b['value']} TFLOP/s = {b['pct_of_bf16_mfma_peak']} % of the "
+            "2.5 PFLOP/s bf16 MFMA peak.\n",
+            f"Roofline arithmetic for the longest kernel ({dom}): algorithmic FLOPs per launch = {share:.0f} x B*Hq*S^2*d = {share:.0f} x {unit:.4e}",
+            f"= {share * unit:.4e} (of the 6 x B*Hq*S^2*d that fwd+bwd count, attributed fwd 2 / dK,dV 3 / dQ 1; recomputed products",
+            f"are not counted).  At the traced average of the timed launches, {t * 1e3:.3f} ms, that is {share * unit / t / 1e12:.0f} TFLOP/s = "
+            f"{100 * share * unit / t / 2.5e15:.1f} % of the peak;",
+            f"the bench line's roofline object says {b['roofline']['achieved']} TFLOP/s = {100 * b['roofline']['frac']:.1f} % from its own "
+            f"{b['roofline']['launch_ms']} ms.  The whole step reaches {100 * b['roofline']['step_frac_of_peak']:.1f} %."]
+    open(os.path.join(prof, "attn_fwd_bwd_llama3_8b_S8192_kernel_trace.md"), "w").write("\n".join(o) + "\n")
+
+  # 2. HBM traffic per launch, scaled by the 256 MiB copy
+  if have("pmc_fetch/p_counter_collection.csv", "pmc_write/p_counter_collection.csv"):
+    def counter(rel, name):
+      agg, n, copy = collections.defaultdict(float), collections.defaultdict(set), None
+      for r in csv.DictReader(open(os.path.join(d, rel))):
+        if r["Counter_Name"] != name:
+          continue
+        if "copyBuffer" in r["Kernel_Name"] and int(r["Grid_Size"]) >= 131072 and copy is None:
+          copy = float(r["Counter_Value"])
+        k = _attn_kernel_of(r["Kernel_Name"])
+        if k and "f32" not in r["Kernel_Name"]:
+          agg[k] += float(r["Counter_Value"])
+          n[k].add(r["Dispatch_Id"])
+      return {k: agg[k] / len(n[k]) for k in agg}, {k: len(n[k]) for k in agg}, copy
+    fetch, nf, cf = counter("pmc_fetch/p_counter_collection.csv", "FETCH_SIZE")
+    write, _, cw = counter("pmc_write/p_counter_collection.csv", "WRITE_SIZE")
+    if cf and cw:
+      sf, sw = 262144.0 / cf, 262144.0 / cw
+      o = ["# HBM traffic per launch: attention kernels at the Llama-3-8B shape (S=8192, bf16, causal)\n",
+           head + f"Two counter runs, one counter each ({_PRE}):\n", cmd("pmc_fetch"), cmd("pmc_write"), "",
+           "`--calib-copy` runs one device-to-device copy of 256 MiB (262144 KiB read, 262144 KiB written) before the timed work;",
+           f"the counters read {cf:.1f} (FETCH_SIZE) and {cw:.1f} (WRITE_SIZE) for it, so the scale factors are",
+           f"{sf:.3f} and {sw:.3f} KiB per count.\n",
+           "| kernel | dispatches | FETCH_SIZE avg | WRITE_SIZE avg | HBM read MiB | HBM write MiB |", "|---|---:|---:|---:|---:|---:|"]
+      traffic = {}
+      for k in ("attn_fwd", "attn_delta", "attn_bwd_dkdv", "attn_bwd_dq"):
+        rd, wr = fetch[k] * sf / 1024, write[k] * sw / 1024
+        traffic[k] = float(f"{(rd + wr) * (1 << 20):.3g}")
+        o.append(f"| {k}_kernel | {nf[k]} | {fetch[k]:.0f} | {write[k]:.0f} | {rd:.0f} | {wr:.0f} |")
+      o += ["", "Algorithmic bytes for comparison (each operand once): forward 640 MiB (q, k, v in; out, lse out), dK/dV kernel",
+            "about 770 MiB (q, dO, k, v, row vectors in; dk, dv out), dQ kernel about 900 MiB.  The dK/dV kernel's workgroups",
+            "(one per 128 kv rows) each stream the Q and dO rows at or below their diagonal, 32 passes over Q and dO on",
+            "average; what the table shows beyond the algorithmic bytes is the part of those passes that the L2 shared by a",
+            "(batch, kv head) group's workgroups did not serve.  The kernels are MFMA-issue bound, not HBM-bound: at their",
+            "launch times the read rates are a quarter of the 8 TB/s peak or less."]
+      open(os.path.join(prof, "attn_fwd_bwd_llama3_8b_S8192_hbm_traffic.md"), "w").write("\n".join(o) + "\n")
+      with open(os.path.join(prof, "attn_fwd_bwd_llama3_8b_S8192_hbm_traffic.json"), "w") as f:
+        json.dump({"source": "profiles/attn_fwd_bwd_llama3_8b_S8192_hbm_traffic.md", "written_by": "bench.py --summarize",
+                   "commit": commit, "hbm_bytes_per_launch": traffic}, f, indent=2)
+        f.write("\n")
+
+  # 3. MFMA pipe utilisation and LDS counters
+  if have("pmc_a/p_counter_collection.csv", "pmc_b/p_counter_collection.csv", "pmc_a.log"):
+    def agg(rel):
+      a, disp = collections.defaultdict(lambda: collections.defaultdict(float)), collections.defaultdict(dict)
+      for r in csv.DictReader(open(os.path.join(d, rel))):
+        k = _attn_kernel_of(r["Kernel_Name"])
+        if k and "f32" not in r["Kernel_Name"]:
+          a[k][r["Counter_Name"]] += float(r["Counter_Value"])
+          disp[k][r["Dispatch_Id"]] = int(r["End_Timestamp"]) - int(r["Start_Timestamp"])
+      res = {k: {c: x / len(disp[k]) for c, x in v.items()} for k, v in a.items()}
+      for k in res:
+        res[k]["duration_ns"] = sum(disp[k].values()) / len(disp[k])
+      return res
+    A, Bc = agg("pmc_a/p_counter_collection.csv"), agg("pmc_b/p_counter_collection.csv")
+    b = bench_line("pmc_a.log")
+    o = ["# MFMA pipe utilisation, issue and LDS counters: attention kernels at the Llama-3-8B shape (S=8192, bf16, causal)\n",
+         head + f"Two counter runs of eight SQ counters each ({_PRE}):\n", cmd("pmc_a"), cmd("pmc_b"), "",
+         "Values are averages per launch over the three launches of each run, summed over the chip.  SQ_BUSY_CU_CYCLES counts per compute",
+         "unit (256 of them), SQ_VALU_MFMA_BUSY_CYCLES per SIMD (4 per CU), so the MFMA pipes' busy fraction is MFMA_BUSY / (4 x BUSY_CU).",
+         "The clock column is BUSY_CU_CYCLES / 256 / the duration of the same dispatches (their timestamps in the counter file; a compute",
+         "unit that idles at either end of a launch does not count, so this reads a little under the shader clock).\n",
+         "| kernel | BUSY_CU_CYCLES | VALU_MFMA_BUSY_CYCLES | MFMA pipe busy | VALU_MFMA_COEXEC / (4 x BUSY_CU) | ACTIVE_INST_VALU x 4 / (4 x BUSY_CU) | WAIT_INST_ANY / WAVE_CYCLES | INSTS_MFMA | INSTS_LDS | LDS_BANK_CONFLICT / LDS_IDX_ACTIVE | clock GHz |",
+         "|---|---:|---:|---:|---:|---:|---:|---:|---:|---:|---:|"]
+    tb = tm = 0.0
+    clocks = []
+    for k in ("attn_fwd", "attn_delta", "attn_bwd_dkdv", "attn_bwd_dq"):
+      a, bb = A[k], Bc[k]
+      simd = 4 * a["SQ_BUSY_CU_CYCLES"]
+      tb += simd
+      tm += a["SQ_VALU_MFMA_BUSY_CYCLES"]
+      conf = bb["SQ_LDS_BANK_CONFLICT"] / bb["SQ_LDS_IDX_ACTIVE"] if bb.get("SQ_LDS_IDX_ACTIVE") else 0.0
+      ghz = a["SQ_BUSY_CU_CYCLES"] / 256 / a["duration_ns"]
+      if k != "attn_delta":
+        clocks.append(ghz)
+      o.append(f"| {k} | {a['SQ_BUSY_CU_CYCLES']:.3g} | {a['SQ_VALU_MFMA_BUSY_CYCLES']:.3g} | {100 * a['SQ_VALU_MFMA_BUSY_CYCLES'] / simd:.1f} % | "
+               f"{100 * a['SQ_VALU_MFMA_COEXEC_CYCLES'] / simd:.1f} % | {100 * 4 * a['SQ_ACTIVE_INST_VALU'] / simd:.1f} % | "
+               f"{100 * a['SQ_WAIT_INST_ANY'] / a['SQ_WAVE_CYCLES']:.1f} % | {bb['SQ_INSTS_MFMA']:.3g} | {bb['SQ_INSTS_LDS']:.3g} | {100 * conf:.1f} % | {ghz:.2f} |")
+    clk = sum(clocks) / len(clocks)
+    o += ["", f"All four kernels together: MFMA pipes busy {100 * tm / tb:.1f} % of the SIMD cycles of a step.\n",
+          "Cross-check.  The dK/dV kernel executes four S x S x d products per head (S, dP, dV, dK) on the causal half plus the",
+          "diagonal tiles: 4 x 1.0995e12 / 32768 FLOP per v_mfma_f32_32x32x16_bf16 = 1.34e8 instructions (SQ_INSTS_MFMA counts per wave) x 32",
+          f"cycles = 4.3e9 busy cycles; the counter reads {A['attn_bwd_dkdv']['SQ_VALU_MFMA_BUSY_CYCLES']:.3g}.\n",
+          "What the numbers say about the headline fraction.  bench.py counts 6 product-units per step (forward 2, backward 4: the",
+          "reference's MFU convention); the kernels execute 9 (forward 2, dK/dV 4, dQ 3: S and dP are recomputed in both backward",
+          f"kernels).  Algorithmic fraction of the 2.5 PFLOP/s peak = MFMA-busy fraction x 6/9 x (sustained clock / 2.4 GHz) = {tm / tb:.3f} x 0.667 x",
+          f"{clk / 2.4:.3f} = {100 * tm / tb * 0.6667 * clk / 2.4:.1f} %, against {b['pct_of_bf16_mfma_peak']} % on this run's bench line (the causal diagonal tiles are",
+          f"computed whole and counted half).  With this split of the backward and this clock, MFMA pipes that never idled would give",
+          f"{100 * 0.6667 * clk / 2.4:.0f} %; 40 % asks for {100 * 0.40 / 0.6667 / (clk / 2.4):.0f} % busy."]
+    open(os.path.join(prof, "attn_fwd_bwd_llama3_8b_S8192_mfma_busy.md"), "w").write("\n".join(o) + "\n")
+
+  # 4. the other configurations
+  if have("kt_oc/kt_kernel_stats.csv", "kt_oc.log"):
+    oc = bench_line("kt_oc.log")["other_configs"]
+    o = ["# Kernel trace: attention fwd+bwd at the other benchmark configurations\n",
+         head + "Configurations (bf16, causal, inputs resident in HBM, 1 warm-up + 5 timed launches of forward and of backward each):\n",
+         "- packed documents: q (4,32,8192,128), k/v (4,8,8192,128), segment ids of documents of 64..4096 tokens packed into every row  -> kernels `<...,1,1>` (causal, segments)",
+         "- Llama-3-70B layer: q (1,64,8192,128), k/v (1,8,8192,128)  -> the plain causal kernels, as the headline",
+         "- DeepSeek-V3 head dims: q/k (1,128,4096,192), v (1,128,4096,128)  -> kernels `<bf16,192,128,...>`\n",
+         f"Command ({_PRE}):\n", cmd("kt_oc"), "", "`kt_kernel_stats.csv` (times in microseconds):\n"]
+    o += stats_table("kt_oc/kt_kernel_stats.csv", ours) + ["", "The same run's line (torch events around 5 launches; FLOPs = 3 x 2 x Hq x (dqk + dv) x allowed pairs):\n"]
+    for n, v in oc.items():
+      o.append(f"    {n}: fwd {v['fwd_ms']} ms, bwd {v['bwd_ms']} ms, {v['TFLOPs']} TFLOP/s = {100 * v['frac_of_bf16_mfma_peak']:.1f} % "
+               f"of the bf16 MFMA peak ({v['allowed_pairs']} pairs per head)")
+    open(os.path.join(prof, "attn_fwd_bwd_other_configs_kernel_trace.md"), "w").write("\n".join(o) + "\n")
+
+  # 5. the bandwidth-bound kernels either side of attention
+  if have("kt_extra/kt_kernel_stats.csv", "kt_extra.log"):
+    b = bench_line("kt_extra.log")
+    o = ["# Kernel trace: the bandwidth-bound kernels either side of attention\n",
+         head + "RMSNorm (+ residual add), RoPE (rotate-half, adjacent pairs, interleaved), L2 norm, SwiGLU, shifted cross entropy, at the",
+         "sizes bench.py's `extra` leg uses (Llama-3-8B layer: hidden 4096, 32768 rows; the DeepSeek-V3 norm widths 1536 / 512 at their",
+         "own row count and at 128 Mi elements; vocabulary 128256 x 8192 rows for the loss).\n",
+         f"Command ({_PRE}):\n", cmd("kt_extra"), "",
+         "`kt_kernel_stats.csv`, this library's non-attention kernels above 0.02 % of GPU time (times in microseconds; one kernel",
+         "template serves several sizes, so a row averages them; the last template argument of rmsnorm_bwd_vec tells the residual-add form",
+         "(1) from the plain one (0); the `float` rows with hundreds of calls are the tiny fp32 configuration's launch-by-launch / graph leg):\n"]
+    o += stats_table("kt_extra/kt_kernel_stats.csv", lambda n: ours(n) and "attn" not in n, 0.02)
+    o += ["", "The same run's `extra` leg (torch events around 20 launches each, a 256 MiB fill between launches to empty the caches):\n"]
+    for n, v in b["extra"].items():
+      if isinstance(v, dict) and "ms" in v and "GBps" in v:
+        o.append(f"    {n}: {v['ms']} ms, {v['GBps']} GB/s = {100 * v['frac_of_hbm_peak']:.1f} % of 8 TB/s")
+    open(os.path.join(prof, "norm_rope_mlp_loss_kernel_trace.md"), "w").write("\n".join(o) + "\n")
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -611,7 +836,18 @@ def main():
                   help="run only one Llama-3-8B decoder layer forward + backward (GEMMs included) and print its line")
   ap.add_argument("--tiny-config", action="store_true",
                   help="run only the tiny fp32 configuration's launch-by-launch / HIP graph comparison and print its line")
+  ap.add_argument("--summarize", default=None, metavar="DIR",
+                  help="no GPU work: turn the rocprofv3 output under DIR (see _PROFILE_COMMANDS) into the summaries under profiles/")
+  ap.add_argument("--commit", default=None, help="with --summarize: the commit the profiled tree was at (default: git rev-parse)")
   args = ap.parse_args()
+  if args.summarize:
+    commit = args.commit
+    if commit is None:
+      import subprocess
+
+      commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip() or "unknown"
+    summarize_profiles(args.summarize, commit)
+    return
   if args.gpus != 1:
     sys.exit("bench.py measures the one-GPU hot path only: run with --gpus 1 (no multi-GPU path is part of this build)")
 

@@ -204,6 +204,35 @@ int tp_attn_bwd_masked(const void* dout, const void* q, const void* k, const voi
                        int window_left, int window_right, float logits_soft_cap, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * Additive attention mask: the eager branch of the reference's attention module adds a mask tensor to the
+ * scaled scores before the softmax (torchprime/torch_xla_models/attention.py:137-158:
+ *     attn_weights = matmul(q, k^T) * scaling; attn_weights = attn_weights + causal_mask).
+ * tp_attn_fwd_masked / tp_attn_bwd_masked with, on top of their arguments:
+ *   bias            fp32, element (b, h, i, j) at bias[b*bias_strides[0] + h*bias_strides[1] + i*bias_strides[2] + j]
+ *                   (key axis contiguous; a broadcast batch or head axis has stride 0); it is added to the
+ *                   scaled (and soft-capped) score of query row i of query head h and key j; -inf forbids
+ *                   the pair, large negative finite values behave as in the reference (they underflow to a
+ *                   zero weight unless every key of the row carries one)
+ * The mask gets no gradient (the reference's is a constant).  Every tile is evaluated element by element:
+ * use causal / seg / the band arguments for what they can express, they skip tiles.  Rows whose every key is
+ * forbidden give out = 0, lse = -inf and zero gradients (the reference's softmax would give NaN there).
+ * ---------------------------------------------------------------------------------------------- */
+int tp_attn_fwd_biased(const void* q, const void* k, const void* v, const int32_t* seg,
+                       const int32_t* q_positions, const float* bias, const int64_t bias_strides[3],
+                       void* out, float* lse, int B, int Hq, int Hkv, int Sq, int Skv, int Dqk, int Dv,
+                       const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                       const int64_t o_strides[3], float sm_scale, int causal, int causal_offset,
+                       int window_left, int window_right, float logits_soft_cap, int dtype, void* stream);
+int tp_attn_bwd_biased(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                       const float* lse, const int32_t* seg, const int32_t* q_positions, const float* bias,
+                       const int64_t bias_strides[3], void* dq, void* dk, void* dv, float* ws, int B, int Hq,
+                       int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t do_strides[3],
+                       const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                       const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                       const int64_t dv_strides[3], float sm_scale, int causal, int causal_offset,
+                       int window_left, int window_right, float logits_soft_cap, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * The steps either side of the attention path (HBM-bound, one pass over each tensor).
  * ---------------------------------------------------------------------------------------------- */
 

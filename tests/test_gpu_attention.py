@@ -267,26 +267,30 @@ def test_attention_module_matches_eager_branch(kernel):
 def test_mask_verdict_is_not_reused_for_a_new_mask_at_the_same_address():
   """A model rebuilds its additive mask every forward (model/llama/model.py:347-355).  The allocator hands the freed
   mask's memory to the next one, so a verdict remembered by address would let a padded mask of the same shape pass as
-  the causal one; the verdict belongs to the tensor object."""
+  the causal one (and take the causal kernels, which never read the mask); the verdict belongs to the tensor object."""
   from torchprime_amd import attention as att
 
   B, H, S, D = 1, 2, 96, 64
-  q, k, v = (heads_view(B, H, S, D, s, torch.bfloat16).to(DEV) for s in (1, 2, 3))
+  q, k, v = (heads_view(B, H, S, D, s, torch.bfloat16) for s in (1, 2, 3))
+  qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
   m = tpa.AttentionModule(_cfg(None, H, H))
   causal = orc.causal_additive_mask(S).to(DEV)
-  m(q, k, v, causal)  # accepted, verdict remembered
-  m(q, k, v, causal)  # same tensor again: no second check needed
+  out_causal = m(qd, kd, vd, causal)  # accepted as causal, verdict remembered
+  m(qd, kd, vd, causal)  # same tensor again: no second check needed
   ptr, n_entries = causal.data_ptr(), len(att._MASK_VERDICTS)
   assert n_entries >= 1
   del causal
   assert len(att._MASK_VERDICTS) == n_entries - 1  # the entry left with the tensor
+  padded_cpu = orc.causal_additive_mask(S).clone()
+  padded_cpu[..., 3 * S // 4 :] = float("-inf")  # a padded batch: the last keys masked for every query
+  ref = orc.eager_attention(q.float(), k.float(), v.float(), padded_cpu)
   hit = False
   for _ in range(8):  # (the allocator normally reuses the block at once; a few tries in case it does not)
-    padded = orc.causal_additive_mask(S).to(DEV)
-    padded[..., : S // 4] = float("-inf")  # a padded batch: the first keys masked for every query
+    padded = padded_cpu.to(DEV)
     hit = hit or padded.data_ptr() == ptr
-    with pytest.raises(NotImplementedError):
-      m(q, k, v, padded)
+    out = m(qd, kd, vd, padded)
+    assert_close(out, ref, "padded mask")
+    assert (out.float() - out_causal.float()).abs().max() > 5e-2  # not the causal result
     del padded
   assert hit, "the allocator never reused the freed mask's address: the test did not exercise the aliasing"
 
@@ -303,15 +307,19 @@ def test_attention_module_scale_uses_v_head_dim():
   assert (out.float().cpu() - wrong.float()).abs().max() > 5e-2
 
 
-def test_attention_module_eager_without_mask_is_full_attention_and_bad_mask_raises():
+def test_attention_module_eager_without_mask_is_full_attention_and_other_masks_are_added():
   B, H, S, D = 1, 2, 80, 64
   q, k, v = (heads_view(B, H, S, D, s, torch.bfloat16) for s in (1, 2, 3))
   m = tpa.AttentionModule(_cfg(None, H, H))
   out = m(q.to(DEV), k.to(DEV), v.to(DEV), None)
-  assert_close(out, orc.eager_attention(q.float(), k.float(), v.float(), None), "no mask")
-  bad = torch.zeros((1, 1, S, S), device=DEV)
-  with pytest.raises(NotImplementedError):
-    m(q.to(DEV), k.to(DEV), v.to(DEV), bad)
+  full = orc.eager_attention(q.float(), k.float(), v.float(), None)
+  assert_close(out, full, "no mask")
+  # an all-zero mask is full attention too; a random one is added to the logits (attention.py:153-158)
+  assert_close(m(q.to(DEV), k.to(DEV), v.to(DEV), torch.zeros((1, 1, S, S), device=DEV)), full, "zero mask")
+  noise = torch.randn((1, 1, S, S), generator=torch.Generator().manual_seed(0))
+  assert_close(m(q.to(DEV), k.to(DEV), v.to(DEV), noise.to(DEV)), orc.eager_attention(q.float(), k.float(), v.float(), noise), "noise")
+  with pytest.raises(ValueError, match="attention_mask must be 4-D"):
+    m(q.to(DEV), k.to(DEV), v.to(DEV), torch.zeros((S, S), device=DEV))
 
 
 def test_splash_wrapper_signature_and_segments():

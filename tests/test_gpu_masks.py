@@ -196,3 +196,114 @@ def test_full_size_sliding_window_slice():
   assert_close(qd.grad[b : b + 1, hs], dq_ref, "dq", scale_abs=True)
   assert_close(kd.grad[b : b + 1, g : g + 1], dk_ref, "dk", scale_abs=True)
   assert_close(vd.grad[b : b + 1, g : g + 1], dv_ref, "dv", scale_abs=True)
+
+
+# ---- additive masks: the eager branch's ``attn_weights + causal_mask`` (attention.py:151-158) for any mask ----------
+def _eager_grads(q, k, v, do, mask):
+  """(out, dq, dk, dv) of the oracle's eager attention in float64, by autograd."""
+  q64, k64, v64 = (t.double().requires_grad_(True) for t in (q, k, v))
+  out = orc.eager_attention(q64, k64, v64, None if mask is None else mask.double())
+  dq, dk, dv = torch.autograd.grad(out, (q64, k64, v64), do.double())
+  return out.detach(), dq, dk, dv
+
+
+def _padding_mask(B, S, Skv, lengths, causal, dtype=torch.float32, fill=float("-inf")):
+  """(B,1,S,Skv): keys at or past ``lengths[b]`` are forbidden for batch row b; optionally causal on top."""
+  j = torch.arange(Skv)[None, None, None, :]
+  bad = j >= torch.as_tensor(lengths)[:, None, None, None]
+  if causal:
+    bad = bad | (j > torch.arange(S)[None, None, :, None])
+  return torch.zeros((B, 1, S, Skv), dtype=dtype).masked_fill(bad, fill)
+
+
+def _check_bias(B, Hq, Hkv, S, D, mask, dtype=torch.bfloat16, Skv=None, Dv=None, seed=0, causal=False, ref_mask=None):
+  Skv = S if Skv is None else Skv
+  Dv = D if Dv is None else Dv
+  q, k, v, do = (heads_view(B, h, s_, d, seed + i, dtype)
+                 for i, (h, s_, d) in enumerate(((Hq, S, D), (Hkv, Skv, D), (Hkv, Skv, Dv), (Hq, S, Dv))))
+  qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+  out = tpa.ops.attention(qd, kd, vd, None, None, causal, bias=mask.to(DEV))
+  out.backward(do.to(DEV))
+  o_ref, dq_ref, dk_ref, dv_ref = _eager_grads(q, k, v, do, mask if ref_mask is None else ref_mask)
+  assert torch.isfinite(o_ref).all()
+  assert_close(out, o_ref, "out")
+  assert_close(qd.grad, dq_ref, "dq", scale_abs=True)
+  assert_close(kd.grad, dk_ref, "dk", scale_abs=True)
+  assert_close(vd.grad, dv_ref, "dv", scale_abs=True)
+
+
+@pytest.mark.parametrize("D,Dv", [(128, 128), (64, 64), (192, 128)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_additive_padding_mask_fwd_bwd(D, Dv, dtype):
+  B, S = 3, 200
+  _check_bias(B, 4, 2, S, D, _padding_mask(B, S, S, [200, 131, 64], causal=True), dtype=dtype, Dv=Dv)
+  _check_bias(B, 4, 2, S, D, _padding_mask(B, S, 333, [333, 7, 190], causal=False), dtype=dtype, Dv=Dv, Skv=333, seed=3)
+
+
+@pytest.mark.parametrize("D", [128, 64])
+def test_additive_mask_fp32_operands(D):
+  B, S = 2, 150
+  _check_bias(B, 4, 2, S, D, _padding_mask(B, S, S, [150, 77], causal=True), dtype=torch.float32)
+  bias = 2.0 * torch.randn((1, 4, S, S), generator=torch.Generator().manual_seed(5))
+  _check_bias(B, 4, 2, S, D, bias, dtype=torch.float32, seed=2)
+
+
+def test_additive_mask_with_finite_values_per_head_and_the_causal_flag():
+  """A per-head finite bias (ALiBi-like slopes plus noise), broadcast over the batch; once with causality inside the
+  mask and once through the kernel's own causal flag: both are the eager formula with the summed mask."""
+  B, Hq, Hkv, S, D = 2, 8, 2, 260, 128
+  i, j = torch.arange(S)[:, None], torch.arange(S)[None, :]
+  slopes = 2.0 ** -torch.arange(1, Hq + 1).float()
+  bias = -(i - j).abs().float()[None, None] * slopes[None, :, None, None]
+  bias = bias + 0.5 * torch.randn((1, Hq, S, S), generator=torch.Generator().manual_seed(1))
+  causal = orc.causal_additive_mask(S)
+  _check_bias(B, Hq, Hkv, S, D, bias + causal)
+  _check_bias(B, Hq, Hkv, S, D, bias, causal=True, ref_mask=bias + causal, seed=4)
+  _check_bias(B, Hq, Hkv, S, D, bias)  # no forbidden pair at all
+
+
+def test_additive_mask_with_the_dtype_minimum_instead_of_minus_infinity():
+  """Masks built as ``finfo(dtype).min`` (the other common convention): the weights underflow to zero exactly as in
+  the eager formula, also where the mask is a 16-bit tensor and where it is longer than the keys."""
+  B, S = 2, 180
+  for mdtype in (torch.float32, torch.bfloat16, torch.float16):
+    m = _padding_mask(B, S, S + 20, [S, 99], causal=True, dtype=mdtype, fill=torch.finfo(mdtype).min)
+    q, k, v = (heads_view(B, h, S, 128, s, torch.bfloat16) for h, s in ((4, 1), (2, 2), (2, 3)))
+    mod = tpa.AttentionModule(tpa.Config(attention_kernel=None, num_attention_heads=4, num_key_value_heads=2))
+    out = mod(q.to(DEV), k.to(DEV), v.to(DEV), m.to(DEV))
+    assert_close(out, orc.eager_attention(q.float(), k.float(), v.float(), m.float()), f"mask dtype {mdtype}")
+
+
+def test_rows_with_every_key_forbidden_give_zeros_and_zero_gradients():
+  """The eager softmax gives NaN on such rows (padding queries); the kernels define them as out = 0 with no gradient,
+  as for segment masks, and every other row is unaffected."""
+  B, Hq, Hkv, S, D = 1, 4, 2, 140, 128
+  mask = _padding_mask(B, S, S, [S], causal=True)
+  mask[:, :, 40:75, :] = float("-inf")
+  q, k, v, do = (heads_view(B, h, S, D, s, torch.bfloat16) for h, s in ((Hq, 1), (Hkv, 2), (Hkv, 3), (Hq, 4)))
+  qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+  out = tpa.ops.attention(qd, kd, vd, None, None, False, bias=mask.to(DEV))
+  out.backward(do.to(DEV))
+  assert torch.isfinite(out).all() and torch.isfinite(qd.grad).all() and torch.isfinite(kd.grad).all()
+  assert (out[:, :, 40:75] == 0).all() and (qd.grad[:, :, 40:75] == 0).all()
+  live = torch.ones(S, dtype=torch.bool)
+  live[40:75] = False
+  do_live = do.clone()
+  do_live[:, :, ~live] = 0
+  ref_mask = mask.clone()
+  ref_mask[:, :, 40:75, 0] = 0.0  # any allowed key: with dO = 0 these rows contribute nothing
+  o_ref, dq_ref, dk_ref, dv_ref = _eager_grads(q, k, v, do_live, ref_mask)
+  assert_close(out[:, :, live], o_ref[:, :, live], "out, live rows")
+  assert_close(qd.grad[:, :, live], dq_ref[:, :, live], "dq, live rows", scale_abs=True)
+  assert_close(kd.grad, dk_ref, "dk", scale_abs=True)
+  assert_close(vd.grad, dv_ref, "dv", scale_abs=True)
+
+
+def test_additive_mask_shape_errors():
+  q = torch.zeros((2, 4, 32, 128), dtype=torch.bfloat16, device=DEV)
+  with pytest.raises(ValueError, match="mask must have shape"):
+    tpa.ops.attention(q, q, q, None, None, False, bias=torch.zeros((3, 1, 32, 32), device=DEV))
+  with pytest.raises(ValueError, match="mask must have shape"):
+    tpa.ops.attention(q, q, q, None, None, False, bias=torch.zeros((32, 32), device=DEV))
+  with pytest.raises(RuntimeError, match="no CPU path"):
+    tpa.ops.attention(q, q, q, None, None, False, bias=torch.zeros((1, 1, 32, 32)))

@@ -72,6 +72,16 @@ SIGNATURES = {
     c_int,
     [c_void_p] * 12 + [c_int] * 7 + [_I64x3] * 8 + [c_float, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
   ),
+  "tp_attn_fwd_biased": (
+    c_int,
+    [c_void_p] * 6 + [_I64x3] + [c_void_p] * 2 + [c_int] * 7 + [_I64x3] * 4
+    + [c_float, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+  ),
+  "tp_attn_bwd_biased": (
+    c_int,
+    [c_void_p] * 9 + [_I64x3] + [c_void_p] * 4 + [c_int] * 7 + [_I64x3] * 8
+    + [c_float, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+  ),
   "tp_attn_bwd_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
   "tp_attn_bwd": (
     c_int,

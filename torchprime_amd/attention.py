@@ -110,16 +110,29 @@ class AttentionModule(nn.Module):
       p = getattr(self.config, "attention_dropout", 0.0)
       if p and self.training:
         raise NotImplementedError("attention_dropout > 0 is not supported (every shipped config uses 0)")
+      bias = None
       if attention_mask is None:
         causal = False
       else:
         assume = bool(self.kernel_config and self.kernel_config.get("assume_causal_mask"))
-        if not assume and not _causal_mask_verdict(attention_mask, q_len, kv_seq_len):
-          raise NotImplementedError(
-            "only the causal additive mask (0 on/below the diagonal, -inf above) is supported; "
-            "document masking goes through segment ids (tpu_splash_attention_jax_call_wrapper)"
+        causal = assume or _causal_mask_verdict(attention_mask, q_len, kv_seq_len)
+        if not causal:
+          # any other mask is added to the scaled logits as it is (attention.py:153-158); the causal one, which
+          # the models build, takes the kernels that skip the tiles above the diagonal instead
+          if attention_mask.dim() != 4 or attention_mask.shape[-1] < kv_seq_len:
+            raise ValueError(
+              f"attention_mask must be 4-D with at least {kv_seq_len} keys, got {tuple(attention_mask.shape)}"
+            )
+          bias = attention_mask[:, :, :, :kv_seq_len]
+      if bias is not None:
+        attn_output = ops.attention(
+          query_states, key_states, value_states, None, 1.0 / math.sqrt(head_dim), False, bias=bias
+        )
+        if attn_output.size() != (bsz, num_heads, q_len, head_dim):
+          raise ValueError(
+            f"`attn_output` should be of size {(bsz, num_heads, q_len, head_dim)}, but is {attn_output.size()}"
           )
-        causal = True
+        return attn_output
 
     attn_output = ops.attention(
       query_states, key_states, value_states, None, 1.0 / math.sqrt(head_dim), causal

@@ -343,6 +343,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   const bool has_seg = SEG && (!GEN || a.seg != nullptr);
   const bool ext = GEN && a.mx.on;
   const bool capped = GEN && a.mx.cap_in != 0.f;
+  const bool biased = GEN && a.mx.bias != nullptr;
   const bool has_pos = ext && a.mx.qpos != nullptr;
   const int32_t* segb = has_seg ? a.seg + (int64_t)b * Skv : nullptr;
 
@@ -491,7 +492,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     if (ext) {
       const int plo = pmin[t], phi = pmax[t];
       skip = skip || wkv0 > phi + a.mx.hi_off || wkv0 + 31 < plo - a.mx.lo_off;
-      need_mask = need_mask || capped || !(wkv0 >= phi - a.mx.lo_off && wkv0 + 31 <= plo + a.mx.hi_off);
+      need_mask = need_mask || capped || biased || !(wkv0 >= phi - a.mx.lo_off && wkv0 + 31 <= plo + a.mx.hi_off);
     }
     return skip ? 0 : (need_mask ? 2 : 1);
   };
@@ -597,6 +598,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       const float* deltal = lsel + BMQ;
       const int* segl = (const int*)(deltal + BMQ);
       const int* posl = segl + BMQ;  // query positions of the tile's rows (mask extensions)
+      const float* bias_head = biased ? a.mx.bias + b * a.mx.bias_s[0] + (hk * a.n_rep + c_hl) * a.mx.bias_s[1] : nullptr;
       // LDS destinations of this wave's loads of tile t+2 (scalar byte addresses)
       const unsigned dma_q = lds_base + (unsigned)(Q_AT + buf2 * Q_BYTES) + wave_q;
       const unsigned dma_o = lds_base + (unsigned)(DO_AT + buf2 * DO_BYTES) + wave_o;
@@ -740,6 +742,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
                     const float th = fast_tanh(sval * a.mx.cap_in);
                     fc[qb][v] = 1.f - th * th;
                     sval = a.mx.cap_out * th;
+                  }
+                  if (biased) {  // additive mask, in units of the raw score (-inf stays -inf)
+                    const int qrow_b = min(qi0 + qb * 32 + 8 * vq + 4 * g + e, Sq - 1);
+                    sval += a.mx.bias_mul * bias_head[(int64_t)qrow_b * a.mx.bias_s[2] + min(kvcol, Skv - 1)];
                   }
                 }
                 float pv = fast_exp2(__builtin_fmaf(sval, c, nl[vq][e]));
@@ -886,6 +892,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       const float* deltal = lsel + BMQ;
       const int* segl = (const int*)(deltal + BMQ);
       const int* posl = segl + BMQ;  // query positions of the tile's rows (mask extensions)
+      const float* bias_head = biased ? a.mx.bias + b * a.mx.bias_s[0] + (hk * a.n_rep + c_hl) * a.mx.bias_s[1] : nullptr;
       f32x16 sacc[QB], dpacc[QB];
       float fcap[GEN ? QB : 1][16];  // soft cap: 1 - tanh^2 of every score, kept from P to dS
       v8 pfr[BMQ / 16];
@@ -962,6 +969,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
                   const float th = fast_tanh(sval * a.mx.cap_in);
                   fcap[GEN ? qb : 0][v] = 1.f - th * th;
                   sval = a.mx.cap_out * th;
+                }
+                if (biased) {  // additive mask, in units of the raw score (-inf stays -inf)
+                  const int qrow_b = min(qi0 + qb * 32 + 8 * (v / 4) + 4 * g + e, Sq - 1);
+                  sval += a.mx.bias_mul * bias_head[(int64_t)qrow_b * a.mx.bias_s[2] + min(kvcol, Skv - 1)];
                 }
               }
               float pv = fast_exp2(__builtin_fmaf(sval, c, l4[m][e]));
@@ -1133,6 +1144,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   const bool has_seg = SEG && (!GEN || a.seg != nullptr);
   const bool ext = GEN && a.mx.on;
   const bool capped = GEN && a.mx.cap_in != 0.f;
+  const bool biased = GEN && a.mx.bias != nullptr;
   const int32_t* segb = has_seg ? a.seg + (int64_t)b * Skv : nullptr;
 
   const int kv_end = CAUSAL ? min(Skv, q0 + BM) : Skv;
@@ -1154,6 +1166,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
   const float lse_s = (lraw == -INFINITY) ? INFINITY : lraw * LOG2E;
   const float ndelta_s = a.delta[ro];  // -rowsum(dO o O)
   const int segq = has_seg ? segb[qrow_c] : 0;
+  // additive mask: this lane's query row of it
+  const float* bias_row = biased ? a.mx.bias + b * a.mx.bias_s[0] + h * a.mx.bias_s[1] + (int64_t)qrow_c * a.mx.bias_s[2] : nullptr;
   // band of allowed keys of this lane's query row, and the positions' extent over the wave
   int lo_q = -BAND_INF, hi_q = BAND_INF, wpmin = 0, wpmax = 0;
   if (ext) {
@@ -1413,7 +1427,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
       }
       if (ext) {
         skip = skip || kv0 > wpmax + a.mx.hi_off || kv0 + BN - 1 < wpmin - a.mx.lo_off;
-        need_mask = need_mask || capped || !(kv0 >= wpmax - a.mx.lo_off && kv0 + BN - 1 <= wpmin + a.mx.hi_off);
+        need_mask = need_mask || capped || biased || !(kv0 >= wpmax - a.mx.lo_off && kv0 + BN - 1 <= wpmin + a.mx.hi_off);
       }
       if (need_mask && !skip) make_key_bits(kv0, sl);
       auto body = [&](auto masked_c) {
@@ -1464,6 +1478,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
                   dcap = 1.f - th * th;  // derivative of the capped score; P only feeds dS here, so it rides on P
                   sval = a.mx.cap_out * th;
                 }
+                // additive mask, in units of the raw score (-inf stays -inf)
+                if (biased) sval += a.mx.bias_mul * bias_row[min(kv0 + nb * 32 + 8 * (v / 4) + 4 * g + (v % 4), Skv - 1)];
               }
               float pv = fast_exp2(__builtin_fmaf(sval, c, -lse_s));
               if (MASKED) {
@@ -1533,7 +1549,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
       }
       if (ext) {
         skip = skip || kv0 > wpmax + a.mx.hi_off || kv0 + BN - 1 < wpmin - a.mx.lo_off;
-        need_mask = need_mask || capped || !(kv0 >= wpmax - a.mx.lo_off && kv0 + BN - 1 <= wpmin + a.mx.hi_off);
+        need_mask = need_mask || capped || biased || !(kv0 >= wpmax - a.mx.lo_off && kv0 + BN - 1 <= wpmin + a.mx.hi_off);
       }
       // The tile body is laid out slot by slot (one MFMA each, a scheduling barrier after every slot): the
       // LDS fragment of a slot is requested AHEAD slots earlier, and the element-wise work that turns
@@ -1599,6 +1615,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
                   dcap = 1.f - th * th;
                   sval = a.mx.cap_out * th;
                 }
+                if (biased) sval += a.mx.bias_mul * bias_row[min(kv0 + nb * 32 + 8 * (v / 4) + 4 * g + (v % 4), Skv - 1)];
               }
               float pv = fast_exp2(__builtin_fmaf(sval, c, -lse_s));
               if (MASKED) {
@@ -2172,6 +2189,27 @@ extern "C" int tp_attn_bwd_masked(const void* dout, const void* q, const void* k
   return attn_bwd_impl(dout, q, k, v, out, lse, seg, dq, dk, dv, ws, B, Hq, Hkv, Sq, Skv, Dqk, Dv, do_strides, q_strides,
                        k_strides, v_strides, o_strides, dq_strides, dk_strides, dv_strides, sm_scale, causal, dtype, stream,
                        nullptr, make_mask_ext(q_positions, causal, causal_offset, window_left, window_right, logits_soft_cap, sm_scale));
+}
+
+extern "C" int tp_attn_bwd_biased(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                                  const float* lse, const int32_t* seg, const int32_t* q_positions, const float* bias,
+                                  const int64_t bias_strides[3], void* dq, void* dk, void* dv, float* ws, int B, int Hq,
+                                  int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t do_strides[3],
+                                  const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                                  const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                                  const int64_t dv_strides[3], float sm_scale, int causal, int causal_offset, int window_left,
+                                  int window_right, float logits_soft_cap, int dtype, void* stream) {
+  TP_REQUIRE(sm_scale > 0.f, TP_ERR_BAD_ARG, "tp_attn_bwd_biased: sm_scale must be positive");
+  TP_REQUIRE(window_left < BAND_INF && window_right < BAND_INF && causal_offset > -BAND_INF && causal_offset < BAND_INF, TP_ERR_BAD_ARG,
+             "tp_attn_bwd_biased: window or offset out of range");
+  TP_REQUIRE(bias && bias_strides, TP_ERR_BAD_ARG, "tp_attn_bwd_biased: null bias");
+  TP_REQUIRE(bias_strides[0] >= 0 && bias_strides[1] >= 0 && bias_strides[2] >= 0, TP_ERR_BAD_ARG,
+             "tp_attn_bwd_biased: negative bias stride");
+  return attn_bwd_impl(dout, q, k, v, out, lse, seg, dq, dk, dv, ws, B, Hq, Hkv, Sq, Skv, Dqk, Dv, do_strides, q_strides,
+                       k_strides, v_strides, o_strides, dq_strides, dk_strides, dv_strides, sm_scale, causal, dtype, stream,
+                       nullptr,
+                       make_mask_ext(q_positions, causal, causal_offset, window_left, window_right, logits_soft_cap, sm_scale, bias,
+                                     bias_strides));
 }
 
 extern "C" int tp_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,

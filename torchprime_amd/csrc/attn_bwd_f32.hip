@@ -110,6 +110,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(const BwdArgs32 a)
 
   const int qp = a.mx.on ? (a.mx.qpos ? a.mx.qpos[qrow_c] : qrow_c) : 0;
   const int band_lo = a.mx.on ? qp - a.mx.lo_off : -BAND_INF, band_hi = a.mx.on ? qp + a.mx.hi_off : BAND_INF;
+  const float* bias_row = a.mx.bias ? a.mx.bias + b * a.mx.bias_s[0] + h * a.mx.bias_s[1] + (int64_t)qrow_c * a.mx.bias_s[2] : nullptr;
   const int kv_end = a.causal ? min(Skv, q0 + BM) : Skv;
   const int ntiles = (kv_end + BN - 1) / BN;
   for (int t = 0; t < ntiles; t++) {
@@ -146,6 +147,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(const BwdArgs32 a)
         sv = a.cap2 * th;
         fac = 1.f - th * th;  // derivative of the capped score with respect to the raw one
       }
+      if (bias_row) sv += LOG2E * bias_row[min(kv, Skv - 1)];  // additive mask (-inf stays -inf)
       const float p = ok ? exp2f(sv - lse2) : 0.f;
       s[v] = p * (dp[v] - delta) * fac;
     }
@@ -211,6 +213,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_f32_kernel(const BwdArgs32 
     const float* qb = a.q + b * a.qs[0] + h * a.qs[1];
     const float* dob = a.dout + b * a.dos[0] + h * a.dos[1];
     const int64_t ro = ((int64_t)b * a.Hq + h) * Sq;
+    const float* bias_head = a.mx.bias ? a.mx.bias + b * a.mx.bias_s[0] + h * a.mx.bias_s[1] : nullptr;
     for (int qt = qt_first; qt < nqt; qt++) {
       const int qi0 = qt * BMQ;
       __syncthreads();
@@ -253,6 +256,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_f32_kernel(const BwdArgs32 
           sv = a.cap2 * th;
           fac = 1.f - th * th;
         }
+        if (bias_head) sv += LOG2E * bias_head[(int64_t)min(qrow, Sq - 1) * a.mx.bias_s[2] + min(kvcol, Skv - 1)];  // additive mask
         const float p = ok ? exp2f(sv - lsm[r]) : 0.f;
         s[v] = p;
         dp[v] = p * (dp[v] - dsm[r]) * fac;

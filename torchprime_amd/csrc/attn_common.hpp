@@ -133,11 +133,16 @@ struct MaskExt {
   const int32_t* qpos;
   int lo_off, hi_off;
   float cap_in, cap_out;  // 0: no soft cap
+  // additive mask: bias[b * bias_s[0] + h * bias_s[1] + q * bias_s[2] + kv] is added to the scaled (and capped)
+  // logit of (query row q, key kv) of query head h; a broadcast axis has stride 0; -inf forbids the pair
+  const float* bias;
+  int64_t bias_s[3];
+  float bias_mul;  // 1 / softmax scale: the kernels that add the bias before scaling multiply by this
   int on;
 };
 // window_left / window_right < 0: unbounded on that side; soft_cap <= 0: none
 inline MaskExt make_mask_ext(const int32_t* q_positions, int causal, int causal_offset, int window_left, int window_right,
-                             float soft_cap, float sm_scale) {
+                             float soft_cap, float sm_scale, const float* bias = nullptr, const int64_t* bias_strides = nullptr) {
   MaskExt m;
   m.qpos = q_positions;
   const int hi_c = causal ? causal_offset : BAND_INF, hi_w = window_right >= 0 ? window_right : BAND_INF;
@@ -145,12 +150,17 @@ inline MaskExt make_mask_ext(const int32_t* q_positions, int causal, int causal_
   m.lo_off = window_left >= 0 ? window_left : BAND_INF;
   m.cap_in = soft_cap > 0.f ? sm_scale / soft_cap : 0.f;
   m.cap_out = soft_cap > 0.f ? soft_cap / sm_scale : 0.f;
-  m.on = (q_positions != nullptr || window_left >= 0 || window_right >= 0 || soft_cap > 0.f || (causal && causal_offset != 0)) ? 1 : 0;
+  m.bias = bias;
+  for (int i = 0; i < 3; i++) m.bias_s[i] = bias && bias_strides ? bias_strides[i] : 0;
+  m.bias_mul = 1.f / sm_scale;
+  m.on = (q_positions != nullptr || window_left >= 0 || window_right >= 0 || soft_cap > 0.f || (causal && causal_offset != 0) ||
+          bias != nullptr) ? 1 : 0;
   return m;
 }
 inline MaskExt no_mask_ext() {
   MaskExt m;
   m.qpos = nullptr; m.lo_off = BAND_INF; m.hi_off = BAND_INF; m.cap_in = 0.f; m.cap_out = 0.f; m.on = 0;
+  m.bias = nullptr; m.bias_s[0] = m.bias_s[1] = m.bias_s[2] = 0; m.bias_mul = 1.f;
   return m;
 }
 

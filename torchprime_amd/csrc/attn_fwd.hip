@@ -90,6 +90,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   const bool has_seg = SEG && (!GEN || a.seg != nullptr);
   const bool ext = GEN && a.mx.on;
   const bool capped = GEN && a.mx.cap_in != 0.f;
+  const bool biased = GEN && a.mx.bias != nullptr;
   const int32_t* segb = has_seg ? a.seg + (int64_t)b * Skv : nullptr;
 
   const int kv_end = CAUSAL ? min(Skv, q0 + BM) : Skv;
@@ -104,6 +105,8 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
     for (int ks = 0; ks < KSTEPS; ks++) qf[ks] = *(const v8*)(qp + 16 * ks);
   }
   const int segq = has_seg ? segb[min(qrow, Sq - 1)] : 0;
+  // additive mask: this lane's query row of it
+  const float* bias_row = biased ? a.mx.bias + b * a.mx.bias_s[0] + h * a.mx.bias_s[1] + (int64_t)min(qrow, Sq - 1) * a.mx.bias_s[2] : nullptr;
   // band of allowed keys of this lane's query row, and its extent over the wave
   int lo_q = -BAND_INF, hi_q = BAND_INF, wpmin = 0, wpmax = 0;
   if (ext) {
@@ -319,6 +322,8 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
         // soft cap on the raw score, rescaled so that the common scale c still applies afterwards
         if (GEN) {
           if (capped) s[v] = a.mx.cap_out * fast_tanh(s[v] * a.mx.cap_in);
+          // additive mask, in units of the raw score (-inf stays -inf)
+          if (biased) s[v] += a.mx.bias_mul * bias_row[min(kv0 + 32 * hf + 8 * (v / 4) + 4 * g + (v % 4), Skv - 1)];
         }
         const unsigned keep = (unsigned)__builtin_amdgcn_sbfe((int)kbits[hf], 8 * (v / 4) + (v % 4), 1);  // all ones or zero
         const float x = s[v];
@@ -486,7 +491,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
       if (ext) {
         // outside every row's band: nothing to do; not inside every row's band (or a soft cap): element-wise path
         skip = skip || kv0 > wpmax + a.mx.hi_off || kv0 + BN - 1 < wpmin - a.mx.lo_off;
-        need_mask = need_mask || capped || !(kv0 >= wpmax - a.mx.lo_off && kv0 + BN - 1 <= wpmin + a.mx.hi_off);
+        need_mask = need_mask || capped || biased || !(kv0 >= wpmax - a.mx.lo_off && kv0 + BN - 1 <= wpmin + a.mx.hi_off);
       }
       typedef std::integral_constant<int, -1> RT;
       if (skip) {
@@ -636,4 +641,22 @@ extern "C" int tp_attn_fwd_masked(const void* q, const void* k, const void* v, c
   return attn_fwd_impl(q, k, v, seg, out, lse, B, Hq, Hkv, Sq, Skv, Dqk, Dv, q_strides, k_strides, v_strides, o_strides, sm_scale,
                        causal, dtype, stream,
                        make_mask_ext(q_positions, causal, causal_offset, window_left, window_right, logits_soft_cap, sm_scale));
+}
+
+extern "C" int tp_attn_fwd_biased(const void* q, const void* k, const void* v, const int32_t* seg, const int32_t* q_positions,
+                                  const float* bias, const int64_t bias_strides[3], void* out, float* lse, int B, int Hq,
+                                  int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t q_strides[3],
+                                  const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
+                                  float sm_scale, int causal, int causal_offset, int window_left, int window_right,
+                                  float logits_soft_cap, int dtype, void* stream) {
+  TP_REQUIRE(sm_scale > 0.f, TP_ERR_BAD_ARG, "tp_attn_fwd_biased: sm_scale must be positive");
+  TP_REQUIRE(window_left < BAND_INF && window_right < BAND_INF && causal_offset > -BAND_INF && causal_offset < BAND_INF, TP_ERR_BAD_ARG,
+             "tp_attn_fwd_biased: window or offset out of range");
+  TP_REQUIRE(bias && bias_strides, TP_ERR_BAD_ARG, "tp_attn_fwd_biased: null bias");
+  TP_REQUIRE(bias_strides[0] >= 0 && bias_strides[1] >= 0 && bias_strides[2] >= 0, TP_ERR_BAD_ARG,
+             "tp_attn_fwd_biased: negative bias stride");
+  return attn_fwd_impl(q, k, v, seg, out, lse, B, Hq, Hkv, Sq, Skv, Dqk, Dv, q_strides, k_strides, v_strides, o_strides, sm_scale,
+                       causal, dtype, stream,
+                       make_mask_ext(q_positions, causal, causal_offset, window_left, window_right, logits_soft_cap, sm_scale, bias,
+                                     bias_strides));
 }

@@ -61,6 +61,8 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(const FwdArgs32 a) {
   // the band then, and a.causal is off)
   const int qp = a.mx.on ? (a.mx.qpos ? a.mx.qpos[min(qrow, Sq - 1)] : qrow) : 0;
   const int band_lo = a.mx.on ? qp - a.mx.lo_off : -BAND_INF, band_hi = a.mx.on ? qp + a.mx.hi_off : BAND_INF;
+  const float* bias_row =
+      a.mx.bias ? a.mx.bias + b * a.mx.bias_s[0] + h * a.mx.bias_s[1] + (int64_t)min(qrow, Sq - 1) * a.mx.bias_s[2] : nullptr;
 
   // Q^T fragments: lane (query column ln, group g) holds Q[q][g*HD + s] for s = 0..HD-1, pre-multiplied by the
   // scale in log2 units (an fp32 product: no precision is lost that the fp32 reference keeps)
@@ -120,6 +122,7 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(const FwdArgs32 a) {
       const int kv = kv0 + kvl;
       const bool ok = kv < Skv && (!a.causal || kv <= qrow) && (!segb || ssm[kvl] == segq) && kv >= band_lo && kv <= band_hi;
       if (a.cap2 != 0.f) s[v] = a.cap2 * tanhf(s[v] / a.cap2);  // cap * tanh(score / cap), in log2 units
+      if (bias_row) s[v] += LOG2E * bias_row[min(kv, Skv - 1)];  // additive mask (-inf stays -inf)
       s[v] = ok ? s[v] : -INFINITY;
       mx = fmaxf(mx, s[v]);
     }

@@ -392,12 +392,27 @@ def _prep_qpos(qpos: Tensor | None, Sq: int) -> Tensor | None:
   return qpos.to(torch.int32).contiguous()
 
 
+def _prep_bias(bias: Tensor | None, B: int, Hq: int, Sq: int, Skv: int):
+  """(fp32 tensor with a contiguous key axis, its (batch, head, query) strides with 0 on broadcast axes)."""
+  if bias is None:
+    return None, None
+  if bias.dim() != 4 or bias.shape[0] not in (1, B) or bias.shape[1] not in (1, Hq) or bias.shape[2:] != (Sq, Skv):
+    raise ValueError(f"mask must have shape (1|{B}, 1|{Hq}, {Sq}, {Skv}), got {tuple(bias.shape)}")
+  bias = bias.float()
+  if bias.stride(-1) != 1:
+    bias = bias.contiguous()
+  strides = _lib._I64x3(
+    0 if bias.shape[0] == 1 else bias.stride(0), 0 if bias.shape[1] == 1 else bias.stride(1), bias.stride(2)
+  )
+  return bias, strides
+
+
 @torch.library.custom_op("tprime::attn_fwd_masked", mutates_args=(), device_types="cuda")
 def attn_fwd_masked(
   q: Tensor, k: Tensor, v: Tensor, seg: Tensor | None, qpos: Tensor | None, sm_scale: float, causal: bool,
-  causal_offset: int, window_left: int, window_right: int, soft_cap: float,
+  causal_offset: int, window_left: int, window_right: int, soft_cap: float, bias: Tensor | None = None,
 ) -> tuple[Tensor, Tensor]:  # fmt: skip
-  dev = _lib.require_gpu(q, k, v, seg, qpos)
+  dev = _lib.require_gpu(q, k, v, seg, qpos, bias)
   B, Hq, Hkv, Sq, Skv, Dqk, Dv = _check_attn(q, k, v, seg)
   q, k, v = _prep_heads(q), _prep_heads(k), _prep_heads(v)
   if seg is not None:
@@ -405,18 +420,23 @@ def attn_fwd_masked(
   qpos = _prep_qpos(qpos, Sq)
   out = _empty_like_heads(q, Dv)
   lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=dev)
+  bias, bias_strides = _prep_bias(bias, B, Hq, Sq, Skv)
   if out.numel():
-    _lib.call(
-      "tp_attn_fwd_masked", q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.ptr(seg), _lib.ptr(qpos), out.data_ptr(),
-      lse.data_ptr(), B, Hq, Hkv, Sq, Skv, Dqk, Dv, _lib.strides3(q), _lib.strides3(k), _lib.strides3(v),
-      _lib.strides3(out), float(sm_scale), int(causal), int(causal_offset), int(window_left), int(window_right),
-      float(soft_cap), _lib.dtype_code(q.dtype), _lib.stream_ptr(dev),
+    tail = (
+      B, Hq, Hkv, Sq, Skv, Dqk, Dv, _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
+      float(sm_scale), int(causal), int(causal_offset), int(window_left), int(window_right), float(soft_cap),
+      _lib.dtype_code(q.dtype), _lib.stream_ptr(dev),
     )  # fmt: skip
+    head = (q.data_ptr(), k.data_ptr(), v.data_ptr(), _lib.ptr(seg), _lib.ptr(qpos))
+    if bias is None:
+      _lib.call("tp_attn_fwd_masked", *head, out.data_ptr(), lse.data_ptr(), *tail)
+    else:
+      _lib.call("tp_attn_fwd_biased", *head, bias.data_ptr(), bias_strides, out.data_ptr(), lse.data_ptr(), *tail)
   return out, lse
 
 
 @attn_fwd_masked.register_fake
-def _(q, k, v, seg, qpos, sm_scale, causal, causal_offset, window_left, window_right, soft_cap):
+def _(q, k, v, seg, qpos, sm_scale, causal, causal_offset, window_left, window_right, soft_cap, bias=None):
   B, Hq, Sq, _ = q.shape
   return _empty_like_heads(q, v.shape[-1]), q.new_empty((B, Hq, Sq), dtype=torch.float32)
 
@@ -425,8 +445,9 @@ def _(q, k, v, seg, qpos, sm_scale, causal, causal_offset, window_left, window_r
 def attn_bwd_masked(
   dout: Tensor, q: Tensor, k: Tensor, v: Tensor, out: Tensor, lse: Tensor, seg: Tensor | None, qpos: Tensor | None,
   sm_scale: float, causal: bool, causal_offset: int, window_left: int, window_right: int, soft_cap: float,
+  bias: Tensor | None = None,
 ) -> tuple[Tensor, Tensor, Tensor]:  # fmt: skip
-  dev = _lib.require_gpu(dout, q, k, v, out, lse, seg, qpos)
+  dev = _lib.require_gpu(dout, q, k, v, out, lse, seg, qpos, bias)
   B, Hq, Hkv, Sq, Skv, Dqk, Dv = _check_attn(q, k, v, seg)
   q, k, v, out, dout = _prep_heads(q), _prep_heads(k), _prep_heads(v), _prep_heads(out), _prep_heads(dout)
   lse = lse.contiguous()
@@ -438,26 +459,33 @@ def attn_bwd_masked(
     return dq.zero_(), dk.zero_(), dv.zero_()
   lib = _lib.load()
   ws = torch.empty((lib.tp_attn_bwd_workspace_bytes(B, Hq, Sq) // 4,), dtype=torch.float32, device=dev)
-  _lib.call(
-    "tp_attn_bwd_masked", dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
-    _lib.ptr(seg), _lib.ptr(qpos), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), B, Hq, Hkv, Sq, Skv,
+  bias, bias_strides = _prep_bias(bias, B, Hq, Sq, Skv)
+  head = (
+    dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), _lib.ptr(seg), _lib.ptr(qpos),
+  )  # fmt: skip
+  tail = (
+    dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), B, Hq, Hkv, Sq, Skv,
     Dqk, Dv, _lib.strides3(dout), _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
     _lib.strides3(dq), _lib.strides3(dk), _lib.strides3(dv), float(sm_scale), int(causal), int(causal_offset),
     int(window_left), int(window_right), float(soft_cap), _lib.dtype_code(q.dtype), _lib.stream_ptr(dev),
   )  # fmt: skip
+  if bias is None:
+    _lib.call("tp_attn_bwd_masked", *head, *tail)
+  else:
+    _lib.call("tp_attn_bwd_biased", *head, bias.data_ptr(), bias_strides, *tail)
   return dq, dk, dv
 
 
 @attn_bwd_masked.register_fake
-def _(dout, q, k, v, out, lse, seg, qpos, sm_scale, causal, causal_offset, window_left, window_right, soft_cap):
+def _(dout, q, k, v, out, lse, seg, qpos, sm_scale, causal, causal_offset, window_left, window_right, soft_cap, bias=None):
   return _empty_like_heads(q), _empty_like_heads(k), _empty_like_heads(v)
 
 
 def _attn_masked_setup(ctx, inputs, output):
-  q, k, v, seg, qpos, sm_scale, causal, causal_offset, window_left, window_right, soft_cap = inputs
+  q, k, v, seg, qpos, sm_scale, causal, causal_offset, window_left, window_right, soft_cap, bias = inputs
   out, lse = output
-  ctx.save_for_backward(*(t for t in (q, k, v, out, lse, seg, qpos) if t is not None))
-  ctx.has_seg, ctx.has_qpos = seg is not None, qpos is not None
+  ctx.save_for_backward(*(t for t in (q, k, v, out, lse, seg, qpos, bias) if t is not None))
+  ctx.has_seg, ctx.has_qpos, ctx.has_bias = seg is not None, qpos is not None, bias is not None
   ctx.scalars = (sm_scale, causal, causal_offset, window_left, window_right, soft_cap)
 
 
@@ -467,8 +495,9 @@ def _attn_masked_backward(ctx, dout, _dlse):
   rest = saved[5:]
   seg = rest.pop(0) if ctx.has_seg else None
   qpos = rest.pop(0) if ctx.has_qpos else None
-  dq, dk, dv = attn_bwd_masked(dout, q, k, v, out, lse, seg, qpos, *ctx.scalars)
-  return (dq, dk, dv) + (None,) * 8
+  bias = rest.pop(0) if ctx.has_bias else None
+  dq, dk, dv = attn_bwd_masked(dout, q, k, v, out, lse, seg, qpos, *ctx.scalars, bias)
+  return (dq, dk, dv) + (None,) * 9
 
 
 attn_fwd_masked.register_autograd(_attn_masked_backward, setup_context=_attn_masked_setup)
@@ -477,7 +506,7 @@ attn_fwd_masked.register_autograd(_attn_masked_backward, setup_context=_attn_mas
 def attention(
   q: Tensor, k: Tensor, v: Tensor, segment_ids: Tensor | None = None, sm_scale: float | None = None, causal: bool = True,
   *, window: tuple[int | None, int | None] | None = None, soft_cap: float | None = None,
-  q_positions: Tensor | None = None, causal_offset: int = 0,
+  q_positions: Tensor | None = None, causal_offset: int = 0, bias: Tensor | None = None,
 ) -> Tensor:  # fmt: skip
   """Causal / segment-masked GQA attention: q (B,Hq,S,Dqk), k (B,Hkv,S,Dqk), v (B,Hkv,S,Dv) -> (B,Hq,S,Dv).
 
@@ -487,16 +516,23 @@ def attention(
   ``window=(left, right)``: key j only if ``pos - left <= j <= pos + right`` (None: unbounded; LocalMask,
   kernel_utils.py:266-275).  ``soft_cap``: logits become ``cap * tanh(logits / cap)`` (kernel_utils.py:292).
   ``q_positions`` (Sq) int: query row i stands for position ``q_positions[i]`` of the key order
-  (LoadBalancedCausalMask.q_sequence, parallelism_utils.py:109-132); ``causal_offset``: that mask's ``offset``."""
+  (LoadBalancedCausalMask.q_sequence, parallelism_utils.py:109-132); ``causal_offset``: that mask's ``offset``.
+  ``bias`` (1|B, 1|Hq, Sq, Skv): added to the scaled logits before the softmax, the eager branch's additive mask
+  (torchprime/torch_xla_models/attention.py:151-158); it is a constant (no gradient), -inf forbids a pair, and a
+  query row whose every key is forbidden gives zeros where the reference's softmax gives NaN."""
   if soft_cap is not None and soft_cap <= 0:
     raise ValueError(f"soft_cap must be positive, got {soft_cap}")
-  _lib.require_gpu(q, k, v, segment_ids, q_positions)
+  _lib.require_gpu(q, k, v, segment_ids, q_positions, bias)
   if sm_scale is None:
     sm_scale = 1.0 / math.sqrt(v.shape[-1])
   wl, wr = (-1, -1) if window is None else tuple(-1 if w is None else int(w) for w in window)
-  if q_positions is None and wl < 0 and wr < 0 and soft_cap is None and (causal_offset == 0 or not causal):
+  if bias is None and q_positions is None and wl < 0 and wr < 0 and soft_cap is None and (causal_offset == 0 or not causal):
     return attn_fwd(q, k, v, segment_ids, sm_scale, causal)[0]
-  return attn_fwd_masked(q, k, v, segment_ids, q_positions, sm_scale, causal, causal_offset, wl, wr, float(soft_cap or 0.0))[0]
+  if bias is not None:
+    bias = bias.detach()
+  return attn_fwd_masked(
+    q, k, v, segment_ids, q_positions, sm_scale, causal, causal_offset, wl, wr, float(soft_cap or 0.0), bias
+  )[0]
 
 
 # ------------------------------------------------------------------------------------------------
