@@ -355,7 +355,7 @@ def packed_segment_ids(B, S, lo, hi, seed):
   return seg, lengths
 
 
-def bench_other_configs(dev, iters=5, only=None):
+def bench_other_configs(dev, iters=10, only=None):
   """The other benchmark configurations, forward + backward through the C ABI, inputs resident: packed documents
   (configuration 3), the Llama-3-70B layer (4) and the DeepSeek-V3 head dims (5).  FLOPs are counted like the
   headline: 3 x 2 * Hq * (dqk + dv) * (allowed query/key pairs)."""
@@ -402,6 +402,10 @@ def bench_other_configs(dev, iters=5, only=None):
       _lib.call("tp_attn_bwd", do.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
                 _lib.ptr(seg), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), B, Hq, Hkv, S, S, Dqk, Dv,
                 s3(do), s3(q), s3(k), s3(v), s3(out), s3(dq), s3(dk), s3(dv), sm, 1, code, st)  # fmt: skip
+
+    for _ in range(3):  # warm-up steps, as for the headline workload
+      fwd()
+      bwd()
 
     def timed(fn):
       fn()
@@ -603,7 +607,7 @@ _PROFILE_COMMANDS = {
   "pmc_write": "rocprofv3 --pmc WRITE_SIZE --output-format csv -d {d}/pmc_write -o p -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-extra --calib-copy",
   "pmc_a": "rocprofv3 --pmc SQ_BUSY_CU_CYCLES SQ_VALU_MFMA_BUSY_CYCLES SQ_ACTIVE_INST_VALU SQ_VALU_MFMA_COEXEC_CYCLES SQ_INSTS_VALU SQ_WAIT_INST_ANY SQ_ACTIVE_INST_ANY SQ_WAVE_CYCLES --output-format csv -d {d}/pmc_a -o p -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-extra > {d}/pmc_a.log",
   "pmc_b": "rocprofv3 --pmc SQ_INSTS_MFMA SQ_INSTS_LDS SQ_LDS_ADDR_CONFLICT SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE SQ_ACTIVE_INST_LDS SQ_WAIT_INST_LDS SQ_BUSY_CU_CYCLES --output-format csv -d {d}/pmc_b -o p -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-extra",
-  "kt_oc": "rocprofv3 --kernel-trace --stats --output-format csv -d {d}/kt_oc -o kt -- python3 bench.py --other-configs all --steps 5 > {d}/kt_oc.log",
+  "kt_oc": "rocprofv3 --kernel-trace --stats --output-format csv -d {d}/kt_oc -o kt -- python3 bench.py --other-configs all --steps 10 > {d}/kt_oc.log",
   "kt_extra": "rocprofv3 --kernel-trace --stats --output-format csv -d {d}/kt_extra -o kt -- python3 bench.py --steps 10 --warmup 3 --no-cpu > {d}/kt_extra.log",
 }  # fmt: skip
 
@@ -790,12 +794,12 @@ def summarize_profiles(d, commit):
   if have("kt_oc/kt_kernel_stats.csv", "kt_oc.log"):
     oc = bench_line("kt_oc.log")["other_configs"]
     o = ["# Kernel trace: attention fwd+bwd at the other benchmark configurations\n",
-         head + "Configurations (bf16, causal, inputs resident in HBM, 1 warm-up + 5 timed launches of forward and of backward each):\n",
+         head + "Configurations (bf16, causal, inputs resident in HBM; 3 warm-up steps, then 1 + 10 launches of forward and of backward, the 10 timed):\n",
          "- packed documents: q (4,32,8192,128), k/v (4,8,8192,128), segment ids of documents of 64..4096 tokens packed into every row  -> kernels `<...,1,1>` (causal, segments)",
          "- Llama-3-70B layer: q (1,64,8192,128), k/v (1,8,8192,128)  -> the plain causal kernels, as the headline",
          "- DeepSeek-V3 head dims: q/k (1,128,4096,192), v (1,128,4096,128)  -> kernels `<bf16,192,128,...>`\n",
          f"Command ({_PRE}):\n", cmd("kt_oc"), "", "`kt_kernel_stats.csv` (times in microseconds):\n"]
-    o += stats_table("kt_oc/kt_kernel_stats.csv", ours) + ["", "The same run's line (torch events around 5 launches; FLOPs = 3 x 2 x Hq x (dqk + dv) x allowed pairs):\n"]
+    o += stats_table("kt_oc/kt_kernel_stats.csv", ours) + ["", "The same run's line (torch events around 10 launches; FLOPs = 3 x 2 x Hq x (dqk + dv) x allowed pairs):\n"]
     for n, v in oc.items():
       o.append(f"    {n}: fwd {v['fwd_ms']} ms, bwd {v['bwd_ms']} ms, {v['TFLOPs']} TFLOP/s = {100 * v['frac_of_bf16_mfma_peak']:.1f} % "
                f"of the bf16 MFMA peak ({v['allowed_pairs']} pairs per head)")

@@ -1713,12 +1713,16 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
 // side) instead of 32 additions per lane and tile: the kernels are bound by the instructions a SIMD can issue.
 // Per tile and 32-row half h of it:  S_h (KS MFMAs) | dP_h (KS + 1) | ... | dQ += K_h^T dS_h (2 DB), with P_h computed
 // under dP_h and dS_h under what follows.
-template <typename T, int D, bool CAUSAL>
+// With segment ids (SEG) the kernel visits the kv tiles whose id range meets the workgroup's, a list built once per
+// workgroup; a wave skips the tiles that miss its own 32 rows, and masked tiles take the rows of the lane's id from
+// a ballot over the tile's id vector, which wave 0 fetches with the tile (one more LDS-writing load).
+template <typename T, int D, bool CAUSAL, bool SEG>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs a) {
   typedef typename MT<T>::v8 v8;
   constexpr int BN = 64, BM = 128, KS = D / 16, DB = D / 32;
   typedef DmaTile<D, true> KT;
   constexpr int T_BYTES = KT::BYTES, K_AT = 0, V_AT = 2 * T_BYTES;
+  constexpr int SEG_AT = 4 * T_BYTES, CTL_AT = SEG_AT + 2 * BN * 4;  // two id vectors; 16 bytes per visited tile
   constexpr int NLOAD = KT::PER_WAVE;  // loads per wave, tile and tensor
 
   extern __shared__ __align__(16) unsigned char smem[];
@@ -1760,11 +1764,51 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
     asm volatile("" : "+v"(ones_a), "+v"(ndelta_b));
   }
 
+  // ---- segment ids: the list of kv tiles to visit (tile, min id, max id), this wave's own id range
+  const int32_t* segb = SEG ? a.seg + (int64_t)b * Skv : nullptr;
+  const int segq = SEG ? segb[qrow_c] : 0;
+  const int* ctl = (const int*)(smem + CTL_AT);
+  int nact = ntiles, wqmin = 0, wqmax = 0;
+  if (SEG) {
+    wqmin = segq; wqmax = segq;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) {
+      wqmin = min(wqmin, __shfl_xor(wqmin, o, 64));
+      wqmax = max(wqmax, __shfl_xor(wqmax, o, 64));
+    }
+    wqmin = __builtin_amdgcn_readfirstlane(wqmin);
+    wqmax = __builtin_amdgcn_readfirstlane(wqmax);
+    // the tiles' id ranges are only needed until the list is built: they borrow the tile buffers
+    int* kvmin = (int*)smem;
+    int* kvmax = kvmin + ntiles;
+    int* bq = kvmax + ntiles;
+    if (lane == 0) { bq[2 * wave] = wqmin; bq[2 * wave + 1] = wqmax; }
+    seg_tile_ranges(segb, Skv, 0, ntiles, kvmin, kvmax, tid, 256);
+    __syncthreads();
+    const int bmin = min(min(bq[0], bq[2]), min(bq[4], bq[6])), bmax = max(max(bq[1], bq[3]), max(bq[5], bq[7]));
+    int cnt = 0;
+    for (int base = 0; base < ntiles; base += 64) {
+      const int t = base + lane;
+      const int lo = t < ntiles ? kvmin[t] : 0, hi = t < ntiles ? kvmax[t] : 0;
+      const bool act = t < ntiles && !(hi < bmin || lo > bmax);
+      const unsigned long long m = __ballot(act);
+      if (act && wave == 0) *(i32x4*)(smem + CTL_AT + 16 * (cnt + __popcll(m & ((1ull << lane) - 1ull)))) = i32x4{t, lo, hi, 0};
+      cnt += __popcll(m);
+    }
+    nact = cnt;
+    __syncthreads();  // the list is complete and the ranges are no longer read: the first tile may land on them
+  }
+  auto entry = [&](int it) -> i32x4 {
+    if (SEG) return *(const i32x4*)(ctl + 4 * max(min(it, nact - 1), 0));
+    return i32x4{min(it, ntiles - 1), 0, 0, 0};
+  };
+
   // ---- loads
   const unsigned k_tile_bytes = (unsigned)(BN * a.ks[2] * 2), v_tile_bytes = (unsigned)(BN * a.vs[2] * 2);
   KT kdma, vdma;
   kdma.init(a.ks[2], wave, lane);
   vdma.init(a.vs[2], wave, lane);
+  const u32x4 srw = make_rsrc_words(SEG ? (const void*)segb : (const void*)a.k, SEG ? (unsigned)Skv * 4u : 0u);
   const u32x4 krw = make_rsrc_words((const T*)a.k + b * a.ks[0] + hk * a.ks[1], span_bytes(Skv, a.ks[2], D));
   const u32x4 vrw = make_rsrc_words((const T*)a.v + b * a.vs[0] + hk * a.vs[1], span_bytes(Skv, a.vs[2], D));
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);
@@ -1777,6 +1821,10 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
       kdma.template issue_one_at<p>(krw, __builtin_amdgcn_readfirstlane((unsigned)t * k_tile_bytes), kdst0 + (unsigned)(buf * T_BYTES));
     else
       vdma.template issue_one_at<p - NLOAD>(vrw, __builtin_amdgcn_readfirstlane((unsigned)t * v_tile_bytes), vdst0 + (unsigned)(buf * T_BYTES));
+    // the tile's id vector rides with the first piece (rows past the end arrive as zeros and are masked by position)
+    if constexpr (SEG && p == 0) {
+      if (wave == 0) dma_dword_at(srw, __builtin_amdgcn_readfirstlane((unsigned)(t * BN) * 4u), lds_base + (unsigned)(SEG_AT + buf * BN * 4), lane);
+    }
   };
 
   // ---- per-lane LDS addresses in buffer 0 (opaque registers; reads add immediates)
@@ -1825,6 +1873,18 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
       if (CAUSAL) hi = min(hi, qrow - kv0 + 1);
       if (qrow >= Sq) hi = 0;
       unsigned long long m = hi > 0 ? (~0ull >> (64 - hi)) : 0ull;
+      if (SEG) {
+        const int rowseg = ((const int*)(smem + SEG_AT + buf * BN * 4))[lane];  // lane l: id of the tile's kv row l
+        unsigned long long ms = 0ull, todo = ~0ull;
+        while (todo) {
+          const int x = __builtin_amdgcn_readlane(segq, (int)__builtin_ctzll(todo));
+          const unsigned long long rows = __ballot(rowseg == x);
+          const bool mine = segq == x;
+          ms = mine ? rows : ms;
+          todo &= ~__ballot(mine);
+        }
+        m &= ms;
+      }
       kbits[0] = (unsigned)m >> (4 * g);
       kbits[1] = (unsigned)(m >> 32) >> (4 * g);
     }
@@ -1917,19 +1977,31 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next tile has landed
   };
 
-  if (ntiles > 0) {
-    static_for<0, 2 * NLOAD>([&](auto P) { load_piece(P, 0, 0); });
+  // the list entries of the tile being computed and of the next one, as scalars, read a tile ahead of their use
+  i32x4 cur = entry(0), nxt = entry(1);
+#pragma unroll
+  for (int j = 0; j < 3; j++) {
+    cur[j] = __builtin_amdgcn_readfirstlane(cur[j]);
+    nxt[j] = __builtin_amdgcn_readfirstlane(nxt[j]);
+  }
+  if (nact > 0) {
+    static_for<0, 2 * NLOAD>([&](auto P) { load_piece(P, cur[0], 0); });
   }
   __builtin_amdgcn_s_waitcnt(0);  // the fragments above and the first tile have landed (see the forward kernel)
   __syncthreads();
-  auto iteration = [&](auto BUFc, int t) {
+  auto iteration = [&](auto BUFc, int it) {
+    const int t = cur[0], t_next = nxt[0];
+    const i32x4 after = entry(it + 2);
     const int kv0 = t * BN;
-    const int t_next = t + 1 < ntiles ? t + 1 : t;
-    const bool skip = CAUSAL && kv0 > wq_last;
-    const bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0) || (wq0 + 32 > Sq);
+    bool skip = CAUSAL && kv0 > wq_last;
+    bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0) || (wq0 + 32 > Sq);
+    if (SEG) {
+      skip = skip || cur[2] < wqmin || cur[1] > wqmax;
+      need_mask = need_mask || !(cur[1] == cur[2] && wqmin == wqmax && cur[1] == wqmin);
+    }
     if (skip) {
       constexpr int buf = decltype(BUFc)::value;
-      if (t + 1 < ntiles) {
+      if (it + 1 < nact) {
         static_for<0, 2 * NLOAD>([&](auto P) { load_piece(P, t_next, buf ^ 1); });
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       }
@@ -1939,10 +2011,13 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
       tile_body(std::false_type{}, BUFc, t, t_next);
     }
     __syncthreads();
+    cur = nxt;
+#pragma unroll
+    for (int j = 0; j < 3; j++) nxt[j] = __builtin_amdgcn_readfirstlane(after[j]);
   };
-  for (int t = 0; t < ntiles; t += 2) {
-    iteration(std::integral_constant<int, 0>{}, t);
-    if (t + 1 < ntiles) iteration(std::integral_constant<int, 1>{}, t + 1);
+  for (int it = 0; it < nact; it += 2) {
+    iteration(std::integral_constant<int, 0>{}, it);
+    if (it + 1 < nact) iteration(std::integral_constant<int, 1>{}, it + 1);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-writing load outlives the workgroup
 
@@ -2010,20 +2085,29 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
   }
   mark(ev, 2, st);
   // dQ
-  if constexpr (!SEG && DQK == DV && DQK <= 128) {
-    constexpr int BM = 128;
-    const size_t smem = 4 * (size_t)DmaTile<DQK, true>::BYTES;
-    auto kern = attn_bwd_dq_plain_kernel<T, DQK, CAUSAL>;
-    static bool attr_set = false;
-    if (!attr_set) {
-      int rc = set_max_lds(kern, "tp_attn_bwd(dq)");
+  // (segments with causality; segments alone share an instantiation with the mask extensions: the general kernel below)
+  constexpr bool LEAN_DQ = DQK == DV && DQK <= 128 && (!SEG || CAUSAL);
+  constexpr int DQ_BN = 64;
+  const size_t lean_smem = 4 * (size_t)DmaTile<DQK, true>::BYTES + (SEG ? 2 * DQ_BN * 4 + 16 * (size_t)((a.Skv + DQ_BN - 1) / DQ_BN) : 0);
+  bool lean_done = false;
+  if constexpr (LEAN_DQ) {
+    if (lean_smem <= 160 * 1024) {  // (the list of a very long sequence does not fit: the general kernel then)
+      constexpr int BM = 128;
+      auto kern = attn_bwd_dq_plain_kernel<T, DQK, CAUSAL, SEG>;
+      static bool attr_set = false;
+      if (!attr_set) {
+        int rc = set_max_lds(kern, "tp_attn_bwd(dq)");
+        if (rc) return rc;
+        attr_set = true;
+      }
+      kern<<<dim3(xcd_grid((a.Sq + BM - 1) / BM, a.n_rep, a.B * a.Hkv)), dim3(256), lean_smem, st>>>(a);
+      int rc = check_launch("tp_attn_bwd(dq)");
       if (rc) return rc;
-      attr_set = true;
+      lean_done = true;
     }
-    kern<<<dim3(xcd_grid((a.Sq + BM - 1) / BM, a.n_rep, a.B * a.Hkv)), dim3(256), smem, st>>>(a);
-    int rc = check_launch("tp_attn_bwd(dq)");
-    if (rc) return rc;
-  } else {
+  }
+  if constexpr (!LEAN_DQ || SEG) {
+    if (!lean_done) {
     // eight waves (two per SIMD) where a wave's registers fit in half a SIMD's file
     // (the non-causal 128-wide variant does not fit 256 registers without spilling: it keeps four waves)
     constexpr int NW = (DQK == DV && (DQK <= 64 || (DQK <= 128 && CAUSAL))) ? 8 : 4;
@@ -2043,6 +2127,7 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
     kern<<<dim3(xcd_grid((a.Sq + BM - 1) / BM, a.n_rep, a.B * a.Hkv)), dim3(64 * NW), smem, st>>>(a);
     int rc = check_launch("tp_attn_bwd(dq)");
     if (rc) return rc;
+    }
   }
   mark(ev, 3, st);
   return TP_OK;

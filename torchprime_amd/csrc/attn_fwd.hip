@@ -125,10 +125,13 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   }
 
   // ---- segment bookkeeping: per-tile id ranges, list of tiles that can contain an allowed pair
-  int* kvmin = (int*)(smem + 2 * BUF_BYTES);
+  // (the tiles' id ranges are only needed until the list is built: they borrow the tile buffers, which nothing has
+  // been loaded into yet; the list holds (tile, min id, max id) in 16 bytes per visited tile, which one LDS read
+  // fetches a tile ahead of its use)
+  int* kvmin = (int*)smem;
   int* kvmax = kvmin + ntiles;
-  int* active = kvmax + ntiles;
-  int* bq = active + ntiles;  // 16 ints: per-wave (min,max) of the query rows' ids, then of their positions
+  int* bq = kvmax + ntiles;  // 16 ints: per-wave (min,max) of the query rows' ids, then of their positions
+  const int* ctl = (const int*)(smem + 2 * BUF_BYTES);
   int nact = ntiles;
   int wqmin = 0, wqmax = 0;
   if (SEG) {
@@ -157,14 +160,25 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
     int cnt = 0;
     for (int base = 0; base < ntiles; base += 64) {
       const int t = base + lane;
-      const bool act = t < ntiles && !(kvmax[t] < bqmin || kvmin[t] > bqmax) && t * BN <= b_hi && t * BN + BN - 1 >= b_lo;
+      const int lo = t < ntiles ? kvmin[t] : 0, hi = t < ntiles ? kvmax[t] : 0;
+      const bool act = t < ntiles && !(hi < bqmin || lo > bqmax) && t * BN <= b_hi && t * BN + BN - 1 >= b_lo;
       const unsigned long long m = __ballot(act);
-      if (act && wave == 0) active[cnt + __popcll(m & ((1ull << lane) - 1ull))] = t;
+      if (act && wave == 0)
+        *(i32x4*)(smem + 2 * BUF_BYTES + 16 * (cnt + __popcll(m & ((1ull << lane) - 1ull)))) = i32x4{t, lo, hi, 0};
       cnt += __popcll(m);
     }
     nact = cnt;
-    __syncthreads();
+    __syncthreads();  // the list is complete and the ranges are no longer read: the first tile may land on them
   }
+  // list entry i as scalars (a tile offset in vector registers would put every load into a loop over its values)
+  auto entry = [&](int i) -> i32x4 {
+    i32x4 e = i32x4{min(i, ntiles - 1), 0, 0, 0};
+    if (SEG) e = *(const i32x4*)(ctl + 4 * max(min(i, nact - 1), 0));
+    return e;
+  };
+  auto scalars = [](i32x4 e) {
+    return i32x4{__builtin_amdgcn_readfirstlane(e[0]), __builtin_amdgcn_readfirstlane(e[1]), __builtin_amdgcn_readfirstlane(e[2]), 0};
+  };
 
   // ---- K and V tiles travel from memory into LDS by loads that write LDS themselves (rows past Skv arrive as zeros)
   const unsigned k_tile_bytes = (unsigned)(BN * a.ks[2] * 2), v_tile_bytes = (unsigned)(BN * a.vs[2] * 2);
@@ -331,7 +345,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
       }
     };
     constexpr int PVB = DVB, S1 = KSTEPS, PV0 = 2 * KSTEPS, PV1 = PV0 + 2 * PVB, NS = PV1 + 2 * PVB;
-    constexpr int AHEAD = (STATIC_BUF && DQK <= 128) ? 5 : 3, NF = AHEAD + 1;  // (the plain causal kernel up to head dim 128 has registers left for a deeper ring; seven slots gain nothing)
+    constexpr int AHEAD = (CAUSAL && DQK <= 128) ? 5 : 3, NF = AHEAD + 1;  // (the plain causal kernel up to head dim 128 has registers left for a deeper ring; seven slots gain nothing)
     v8 fr[NF];
     f32x16 s[2];
     v8 pf[2][2];
@@ -423,11 +437,10 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
     if (has_next) store_tile(buf ^ 1);
   };
 
-  // i-th kv tile to visit, as a scalar: a tile offset in vector registers would put every staging load into a
-  // loop over its distinct values
-  auto tile_at = [&](int i) { return SEG ? __builtin_amdgcn_readfirstlane(active[i]) : i; };
+  // the entries of the tile being computed and of the next one; the one after is read at the top of a tile
+  i32x4 cur = scalars(entry(0)), nxt = scalars(entry(1));
   if (nact > 0) {
-    load_tile(tile_at(0), 0);
+    load_tile(cur[0], 0);
     store_tile(0);
   }
   // Everything loaded so far (the Q fragments above all) has landed before the loop starts.  Without
@@ -443,14 +456,15 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   // only on tiles that straddle the diagonal, the tail, or a segment boundary
   auto iteration = [&](auto BUFc, const int it) {
     const int buf = decltype(BUFc)::value >= 0 ? decltype(BUFc)::value : (it & 1);
-    const int t = tile_at(it);
+    const i32x4 after = entry(it + 2);
+    const int t = cur[0];
     const int kv0 = t * BN;
     const bool has_next = it + 1 < nact;
-    const int t_next = has_next ? tile_at(it + 1) : t;
+    const int t_next = has_next ? nxt[0] : t;
     bool skip = CAUSAL && kv0 > wq_last;
     bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0);
     if (SEG) {
-      const int lo = kvmin[t], hi = kvmax[t];
+      const int lo = cur[1], hi = cur[2];
       skip = skip || hi < wqmin || lo > wqmax;
       need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
     }
@@ -465,6 +479,8 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
       tile_body(std::false_type{}, BUFc, buf, t, has_next, t_next);
     }
     __syncthreads();
+    cur = nxt;
+    nxt = scalars(after);
   };
   if constexpr (STATIC_BUF) {
     // the plain causal kernel: the loop alternates two copies of the body, one per buffer
@@ -473,18 +489,21 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
       if (it + 1 < nact) iteration(std::integral_constant<int, 1>{}, it + 1);
     }
   } else {
-    // The masked variants have no registers to spare for two copies.  (Their loop body is written out here:
+    // The masked variants have no registers to spare for two copies: with segment ids the two-copy loop spills, and a
+    // reload from scratch waits, the memory counter being in-order, for the tile loads issued before it.  (Their loop
+    // body is written out here:
     // routed through the closure above, the compiler keeps part of the captured state in scratch memory.)
     for (int it = 0; it < nact; it++) {
       const int buf = it & 1;
-      const int t = tile_at(it);
+      const i32x4 after = entry(it + 2);
+      const int t = cur[0];
       const int kv0 = t * BN;
       const bool has_next = it + 1 < nact;
-      const int t_next = has_next ? tile_at(it + 1) : t;
+      const int t_next = has_next ? nxt[0] : t;
       bool skip = CAUSAL && kv0 > wq_last;
       bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0);
       if (SEG) {
-        const int lo = kvmin[t], hi = kvmax[t];
+        const int lo = cur[1], hi = cur[2];
         skip = skip || hi < wqmin || lo > wqmax;
         need_mask = need_mask || !(lo == hi && wqmin == wqmax && lo == wqmin);
       }
@@ -505,6 +524,8 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
         tile_body(std::false_type{}, RT{}, buf, t, has_next, t_next);
       }
       __syncthreads();
+      cur = nxt;
+      nxt = scalars(after);
     }
   }
 
@@ -540,8 +561,8 @@ static int launch_fwd(const FwdArgs& a, int B, hipStream_t st) {
   constexpr int BN = 64, BM = 128;
   constexpr int BUF = DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES + (SEG ? BN * 4 : 0);
   const int ntiles_max = (a.Skv + BN - 1) / BN;
-  const size_t smem = 2 * (size_t)BUF + (SEG ? (size_t)(3 * ntiles_max + 16) * 4 : 0);
-  TP_REQUIRE(smem <= 160 * 1024, TP_ERR_UNSUPPORTED, "tp_attn_fwd: Skv=%d needs %zu bytes of LDS (max 163840)", a.Skv, smem);
+  const size_t smem = 2 * (size_t)BUF + (SEG ? (size_t)16 * ntiles_max : 0);  // (the id ranges borrow the tile buffers)
+  TP_REQUIRE(smem <= 160 * 1024 && (!SEG || (size_t)(2 * ntiles_max + 16) * 4 <= 2 * (size_t)BUF), TP_ERR_UNSUPPORTED, "tp_attn_fwd: Skv=%d needs %zu bytes of LDS (max 163840)", a.Skv, smem);
   auto kern = attn_fwd_kernel<T, DQK, DV, CAUSAL, SEG>;
   static bool attr_set = false;  // benign race: every thread sets the same value
   if (!attr_set) {
