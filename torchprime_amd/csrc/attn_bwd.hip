@@ -314,9 +314,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   constexpr int BNK = 128;  // kv rows per workgroup, 32 per wave
   constexpr int KS_QK = DQK / 16, KS_DV = DV / 16;
   constexpr int DKB = DQK / 32, DVB = DV / 32;
-  // PIPE: equal head dims up to 128.  Three row-major buffers, no transposed copies: the operands of the two
-  // accumulating products are read from the row-major tiles with transposing LDS reads.
-  constexpr bool PIPE = NBUF == 3 && DQK == DV && DQK <= 128;
+  // PIPE: three row-major buffers, no transposed copies: the operands of the two accumulating products are read
+  // from the row-major tiles with transposing LDS reads (every head-dim pair whose three buffers fit the LDS).
+  constexpr bool PIPE = NBUF == 3;
   static_assert(PIPE || NBUF == 1, "three buffers (pipelined path) or one");
   typedef DmaTile<DQK, PIPE> QT;
   typedef DmaTile<DV, PIPE> OT;
@@ -538,7 +538,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       for (int h2 = 0; h2 < 2; h2++) {
         trq[d][h2] = (unsigned)QT::tr_off(8 * h2 + 4 * g, 2 * d + ((lane >> 4) & 1), lane & 15) + lb;
         asm volatile("" : "+v"(trq[d][h2]));
-        tro[d][h2] = trq[d][h2] + (unsigned)O_BIAS;
+      }
+#pragma unroll
+    for (int d = 0; d < DVB; d++)
+#pragma unroll
+      for (int h2 = 0; h2 < 2; h2++) {
+        tro[d][h2] = (unsigned)OT::tr_off(8 * h2 + 4 * g, 2 * d + ((lane >> 4) & 1), lane & 15) + lb + (unsigned)O_BIAS;
         asm volatile("" : "+v"(tro[d][h2]));
       }
     auto ld16 = [](unsigned addr) { return *(const __attribute__((address_space(3))) v8*)addr; };
@@ -636,16 +641,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         // part 1: S0, S1, dP0, dP1 (the exponentials can start as soon as S0 is complete and are over
         // before part 2, which carries the transposition of the next tile);
         // part 2: dV0, dK0, dV1, dK1 (four accumulators each, used round robin)
-        constexpr int K = KS_QK, CL = 2 * DVB;
-        static_assert(KS_QK == KS_DV && DKB == DVB, "the slot plan assumes equal head dims");
-        constexpr int C0 = 4 * K, NS = C0 + 4 * CL;
-        // VALU groups, 2K slots each: P of a block starts when its S is complete, dS when its dP is; each
+        // (K1 / K2 k-steps per S / dP product; CLV / CLK slots per query block of dV / dK)
+        constexpr int K1 = KS_QK, K2 = KS_DV, CLV = 2 * DVB, CLK = 2 * DKB;
+        constexpr int S1_AT = K1, D0_AT = 2 * K1, D1_AT = 2 * K1 + K2, C0 = 2 * (K1 + K2);
+        constexpr int V0_AT = C0, K0_AT = V0_AT + CLV, V1_AT = K0_AT + CLK, K1_AT = V1_AT + CLV, NS = K1_AT + CLK;
+        // VALU groups of VL slots each: P of a block starts when its S is complete, dS when its dP is; each
         // group is over before the MFMAs that consume its packed operand
-        constexpr int EPS = K >= 8 ? 1 : 2, VL = 16 / EPS;
-        constexpr int VP0 = K, VP1 = 2 * K, VS0 = 3 * K, VS1 = 4 * K;
-        static_assert(VL == 2 * K && VP0 + VL <= C0 && VS0 + VL <= C0 + CL && VP1 + VL <= C0 + 2 * CL &&
-                          VS1 + VL <= C0 + 3 * CL,
-                      "operands not ready");
+        constexpr int EPS = K2 >= 8 ? 1 : 2, VL = 16 / EPS;
+        constexpr int VP0 = S1_AT, VP1 = D0_AT, VS0 = D1_AT, VS1 = C0;
+        static_assert(VP0 + VL <= V0_AT && VS0 + VL <= K0_AT && VP1 + VL <= V1_AT && VS1 + VL <= K1_AT, "operands not ready");
         constexpr int N_DMA = QT::PER_WAVE + OT::PER_WAVE + 1, DMA_EVERY = (NS - C0) / N_DMA;
         static_assert(DMA_EVERY >= 1, "second half too short for the loads");
         const int kvcol = wkv0 + ln;
@@ -686,27 +690,36 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
 
         auto frag = [&](auto I) -> v8 {
           constexpr int i = decltype(I)::value;
-          if constexpr (i < C0) {
-            constexpr int qb = (i / K) % 2, ks = i % K;
-            if constexpr (i < 2 * K) return ld16(aq[ks] + (ql + qb * 32 * QT::ROWB));
-            else return ld16(ao[ks] + (dol + qb * 32 * OT::ROWB));
+          if constexpr (i < D0_AT) {
+            constexpr int qb = i / K1, ks = i % K1;
+            return ld16(aq[ks] + (ql + qb * 32 * QT::ROWB));
+          } else if constexpr (i < C0) {
+            constexpr int qb = (i - D0_AT) / K2, ks = (i - D0_AT) % K2;
+            return ld16(ao[ks] + (dol + qb * 32 * OT::ROWB));
           } else {
             // operand of an accumulating product: rows = head-dim block d, contraction over query rows
             // 32 qb + 16 hh + {4g..4g+3, 8+4g..8+4g+3} (the order in which P / dS hold them), read transposed
-            constexpr int ph = (i - C0) / CL, qb = ph / 2, j = (i - C0) % CL, hh = j / DVB, d = j % DVB;
-            constexpr int rows = (32 * qb + 16 * hh) * QT::ROWB;
-            if constexpr (ph % 2 == 0) return ldtr(tro[d][0] + (dol + rows), tro[d][1] + (dol + rows));
-            else return ldtr(trq[d][0] + (ql + rows), trq[d][1] + (ql + rows));
+            constexpr int qb = i >= V1_AT ? 1 : 0, base = qb ? V1_AT : V0_AT;
+            if constexpr (i - base < CLV) {
+              constexpr int j = i - base, hh = j / DVB, d = j % DVB;
+              constexpr int rows = (32 * qb + 16 * hh) * OT::ROWB;
+              return ldtr(tro[d][0] + (dol + rows), tro[d][1] + (dol + rows));
+            } else {
+              constexpr int j = i - base - CLV, hh = j / DKB, d = j % DKB;
+              constexpr int rows = (32 * qb + 16 * hh) * QT::ROWB;
+              return ldtr(trq[d][0] + (ql + rows), trq[d][1] + (ql + rows));
+            }
           }
         };
         auto mma = [&](auto I, const v8& f) {
           constexpr int i = decltype(I)::value;
           const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          if constexpr (i < C0) {
-            constexpr int qb = (i / K) % 2, ks = i % K;
-            if constexpr (i < 2 * K) {
-              s[qb] = MT<T>::mfma32(f, kf[ks], ks == 0 ? zero : s[qb]);
-            } else if constexpr (ks == 0) {
+          if constexpr (i < D0_AT) {
+            constexpr int qb = i / K1, ks = i % K1;
+            s[qb] = MT<T>::mfma32(f, kf[ks], ks == 0 ? zero : s[qb]);
+          } else if constexpr (i < C0) {
+            constexpr int qb = (i - D0_AT) / K2, ks = (i - D0_AT) % K2;
+            if constexpr (ks == 0) {
               // dP starts from -delta of its rows (C layout: value v belongs to row 8 (v/4) + 4 g + v%4), so
               // that dS = P o dP needs no subtraction
               const f32x4 (&nd)[4] = qb == 0 ? nd0 : nd1;
@@ -717,9 +730,14 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
               dp[qb] = MT<T>::mfma32(f, vf[ks], dp[qb]);
             }
           } else {
-            constexpr int ph = (i - C0) / CL, qb = ph / 2, j = (i - C0) % CL, hh = j / DVB, d = j % DVB;
-            if constexpr (ph % 2 == 0) MT<T>::mfma32_acc(dvacc[d], f, pf[qb][hh]);
-            else MT<T>::mfma32_acc(dkacc[d], f, df[qb][hh]);
+            constexpr int qb = i >= V1_AT ? 1 : 0, base = qb ? V1_AT : V0_AT;
+            if constexpr (i - base < CLV) {
+              constexpr int j = i - base, hh = j / DVB, d = j % DVB;
+              MT<T>::mfma32_acc(dvacc[d], f, pf[qb][hh]);
+            } else {
+              constexpr int j = i - base - CLV, hh = j / DKB, d = j % DKB;
+              MT<T>::mfma32_acc(dkacc[d], f, df[qb][hh]);
+            }
           }
         };
         // VALU group of query block QB starting at slot START: EPS elements per slot for VL slots.
@@ -816,11 +834,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
               if constexpr (i == (r0 < 0 ? 0 : r0)) nl0[vq] = *(const f32x4*)(lsel + 8 * vq + 4 * g);
               if constexpr (i == (r1 < 0 ? 0 : r1)) nl1[vq] = *(const f32x4*)(lsel + 32 + 8 * vq + 4 * g);
             });
-            if constexpr (i == 2 * K - 2) {
+            if constexpr (i == D0_AT - 2) {
 #pragma unroll
               for (int vq = 0; vq < 4; vq++) nd0[vq] = *(const f32x4*)(deltal + 8 * vq + 4 * g);
             }
-            if constexpr (i == 3 * K - 2) {
+            if constexpr (i == D1_AT - 2) {
 #pragma unroll
               for (int vq = 0; vq < 4; vq++) nd1[vq] = *(const f32x4*)(deltal + 32 + 8 * vq + 4 * g);
             }
@@ -1716,14 +1734,18 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdArgs a) {
 // With segment ids (SEG) the kernel visits the kv tiles whose id range meets the workgroup's, a list built once per
 // workgroup; a wave skips the tiles that miss its own 32 rows, and masked tiles take the rows of the lane's id from
 // a ballot over the tile's id vector, which wave 0 fetches with the tile (one more LDS-writing load).
-template <typename T, int D, bool CAUSAL, bool SEG>
-__global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs a) {
+// Unequal head dims (192, 128): the same kernel with one workgroup per CU (its fragments and accumulators need more
+// than half a SIMD's registers) and the dQ accumulators pinned to the accumulation registers.
+template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
+__global__ __launch_bounds__(256, DQK == DV ? 2 : 1) void attn_bwd_dq_plain_kernel(const BwdArgs a) {
   typedef typename MT<T>::v8 v8;
-  constexpr int BN = 64, BM = 128, KS = D / 16, DB = D / 32;
-  typedef DmaTile<D, true> KT;
-  constexpr int T_BYTES = KT::BYTES, K_AT = 0, V_AT = 2 * T_BYTES;
-  constexpr int SEG_AT = 4 * T_BYTES, CTL_AT = SEG_AT + 2 * BN * 4;  // two id vectors; 16 bytes per visited tile
-  constexpr int NLOAD = KT::PER_WAVE;  // loads per wave, tile and tensor
+  constexpr bool WIDE = DQK != DV;
+  constexpr int BN = 64, BM = 128, KS = DQK / 16, KSV = DV / 16, DB = DQK / 32;
+  typedef DmaTile<DQK, true> KT;
+  typedef DmaTile<DV, true> VT;
+  constexpr int K_BYTES = KT::BYTES, V_BYTES = VT::BYTES, K_AT = 0, V_AT = 2 * K_BYTES;
+  constexpr int SEG_AT = 2 * (K_BYTES + V_BYTES), CTL_AT = SEG_AT + 2 * BN * 4;  // two id vectors; 16 bytes per visited tile
+  constexpr int NLOAD_K = KT::PER_WAVE, NLOAD_V = VT::PER_WAVE, NLOAD2 = NLOAD_K + NLOAD_V;  // loads per wave and tile
 
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 5, ln = lane & 31;
@@ -1739,14 +1761,14 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
 
   // ---- Q, dO fragments (B operands: lane = query column), per-lane LSE / -delta
   const int qrow = wq0 + ln, qrow_c = min(qrow, Sq - 1);
-  v8 qf[KS], dof[KS];
+  v8 qf[KS], dof[KSV];
   {
     const T* qp = (const T*)a.q + b * a.qs[0] + h * a.qs[1] + qrow_c * a.qs[2] + 8 * g;
     const T* dp = (const T*)a.dout + b * a.dos[0] + h * a.dos[1] + qrow_c * a.dos[2] + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) qf[ks] = *(const v8*)(qp + 16 * ks);
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++) dof[ks] = *(const v8*)(dp + 16 * ks);
+    for (int ks = 0; ks < KSV; ks++) dof[ks] = *(const v8*)(dp + 16 * ks);
   }
   const int64_t ro = ((int64_t)b * a.Hq + h) * Sq + qrow_c;
   const float lraw = a.lse[ro];
@@ -1805,22 +1827,23 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
 
   // ---- loads
   const unsigned k_tile_bytes = (unsigned)(BN * a.ks[2] * 2), v_tile_bytes = (unsigned)(BN * a.vs[2] * 2);
-  KT kdma, vdma;
+  KT kdma;
+  VT vdma;
   kdma.init(a.ks[2], wave, lane);
   vdma.init(a.vs[2], wave, lane);
   const u32x4 srw = make_rsrc_words(SEG ? (const void*)segb : (const void*)a.k, SEG ? (unsigned)Skv * 4u : 0u);
-  const u32x4 krw = make_rsrc_words((const T*)a.k + b * a.ks[0] + hk * a.ks[1], span_bytes(Skv, a.ks[2], D));
-  const u32x4 vrw = make_rsrc_words((const T*)a.v + b * a.vs[0] + hk * a.vs[1], span_bytes(Skv, a.vs[2], D));
+  const u32x4 krw = make_rsrc_words((const T*)a.k + b * a.ks[0] + hk * a.ks[1], span_bytes(Skv, a.ks[2], DQK));
+  const u32x4 vrw = make_rsrc_words((const T*)a.v + b * a.vs[0] + hk * a.vs[1], span_bytes(Skv, a.vs[2], DV));
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);
   const unsigned lds_base = __builtin_amdgcn_readfirstlane((unsigned)(size_t)smem);
-  const unsigned kdst0 = lds_base + (unsigned)K_AT + (unsigned)(wave_s * NLOAD * 1024);
-  const unsigned vdst0 = lds_base + (unsigned)V_AT + (unsigned)(wave_s * NLOAD * 1024);
+  const unsigned kdst0 = lds_base + (unsigned)K_AT + (unsigned)(wave_s * NLOAD_K * 1024);
+  const unsigned vdst0 = lds_base + (unsigned)V_AT + (unsigned)(wave_s * NLOAD_V * 1024);
   auto load_piece = [&](auto Pc, int t, int buf) {
     constexpr int p = decltype(Pc)::value;
-    if constexpr (p < NLOAD)
-      kdma.template issue_one_at<p>(krw, __builtin_amdgcn_readfirstlane((unsigned)t * k_tile_bytes), kdst0 + (unsigned)(buf * T_BYTES));
+    if constexpr (p < NLOAD_K)
+      kdma.template issue_one_at<p>(krw, __builtin_amdgcn_readfirstlane((unsigned)t * k_tile_bytes), kdst0 + (unsigned)(buf * K_BYTES));
     else
-      vdma.template issue_one_at<p - NLOAD>(vrw, __builtin_amdgcn_readfirstlane((unsigned)t * v_tile_bytes), vdst0 + (unsigned)(buf * T_BYTES));
+      vdma.template issue_one_at<p - NLOAD_K>(vrw, __builtin_amdgcn_readfirstlane((unsigned)t * v_tile_bytes), vdst0 + (unsigned)(buf * V_BYTES));
     // the tile's id vector rides with the first piece (rows past the end arrive as zeros and are masked by position)
     if constexpr (SEG && p == 0) {
       if (wave == 0) dma_dword_at(srw, __builtin_amdgcn_readfirstlane((unsigned)(t * BN) * 4u), lds_base + (unsigned)(SEG_AT + buf * BN * 4), lane);
@@ -1829,13 +1852,18 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
 
   // ---- per-lane LDS addresses in buffer 0 (opaque registers; reads add immediates)
   const unsigned lds0 = (unsigned)(size_t)smem;
-  constexpr bool SWZ3 = KT::CPR % 16 != 0;
-  constexpr int NFO = SWZ3 ? (KS < 4 ? KS : 4) : KS;
-  unsigned kfo[NFO], ktr[DB][2];
+  constexpr bool SWZ3 = KT::CPR % 16 != 0, VSWZ3 = VT::CPR % 16 != 0;
+  constexpr int NFO = SWZ3 ? (KS < 4 ? KS : 4) : KS, NVO = WIDE ? (VSWZ3 ? (KSV < 4 ? KSV : 4) : KSV) : 1;
+  unsigned kfo[NFO], vfo[NVO], ktr[DB][2];
 #pragma unroll
   for (int j = 0; j < NFO; j++) {
-    kfo[j] = lds0 + (unsigned)(ln * KT::ROWB + (((2 * j + g) ^ KT::swz(ln)) << 4));  // K; V lies V_AT further on
+    kfo[j] = lds0 + (unsigned)(ln * KT::ROWB + (((2 * j + g) ^ KT::swz(ln)) << 4));  // K (equal head dims: V lies V_AT further on)
     asm volatile("" : "+v"(kfo[j]));
+  }
+#pragma unroll
+  for (int j = 0; j < NVO; j++) {
+    vfo[j] = lds0 + (unsigned)V_AT + (unsigned)(ln * VT::ROWB + (((2 * j + g) ^ VT::swz(ln)) << 4));
+    asm volatile("" : "+v"(vfo[j]));
   }
 #pragma unroll
   for (int d = 0; d < DB; d++)
@@ -1856,14 +1884,14 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
   const int wq_last = wq0 + 31;
 
   // slots of a tile: S0 | dP0 | S1 | dP1 | dQ0 | dQ1
-  constexpr int KSD = KS + 1, A2 = 2 * DB;
+  constexpr int KSD = KSV + 1, A2 = 2 * DB;
   constexpr int P_S0 = 0, P_D0 = KS, P_S1 = P_D0 + KSD, P_D1 = P_S1 + KS, P_Q0 = P_D1 + KSD, P_Q1 = P_Q0 + A2, NS = P_Q1 + A2;
   constexpr int AHEAD = 4, NF = AHEAD + 1;
 
   auto tile_body = [&](auto masked_c, auto BUFc, int t, int t_next) {
     constexpr bool MASKED = decltype(masked_c)::value;
     constexpr int buf = decltype(BUFc)::value;
-    constexpr unsigned kl = K_AT + buf * T_BYTES, vl = V_AT + buf * T_BYTES;
+    constexpr unsigned kl = K_AT + buf * K_BYTES, vl = V_AT + buf * V_BYTES, vlw = buf * V_BYTES;  // (vlw: on top of vfo[])
     const int kv0 = t * BN;
     // masked tiles: which of the tile's 64 kv rows this lane's query row may see, as bits (value v of a half: bit
     // 8 (v / 4) + v % 4 after the shift by 4 g)
@@ -1897,10 +1925,14 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
       auto rowfrag = [&](unsigned base, int hf, int ks) {
         return ld16(kfo[SWZ3 ? (ks & 3) : ks] + (base + (unsigned)(hf * 32 * KT::ROWB + (SWZ3 ? 128 * (ks >> 2) : 0))));
       };
+      auto vfrag = [&](int hf, int ks) {
+        if constexpr (WIDE) return ld16(vfo[VSWZ3 ? (ks & 3) : ks] + (vlw + (unsigned)(hf * 32 * VT::ROWB + (VSWZ3 ? 128 * (ks >> 2) : 0))));
+        else return rowfrag(vl, hf, ks);
+      };
       if constexpr (i < P_D0) return rowfrag(kl, 0, i - P_S0);
-      else if constexpr (i < P_S1) return rowfrag(vl, 0, i - P_D0 - 1);
+      else if constexpr (i < P_S1) return vfrag(0, i - P_D0 - 1);
       else if constexpr (i < P_D1) return rowfrag(kl, 1, i - P_S1);
-      else if constexpr (i < P_Q0) return rowfrag(vl, 1, i - P_D1 - 1);
+      else if constexpr (i < P_Q0) return vfrag(1, i - P_D1 - 1);
       else {
         // K^T block d, contraction over kv rows 32 hf + 16 kk + {4g..4g+3, 8+4g..8+4g+3}: the order in which dS holds them
         constexpr int hf = i >= P_Q1 ? 1 : 0, j = i - (hf ? P_Q1 : P_Q0), kk = j / DB, d = j % DB;
@@ -1919,7 +1951,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
       else if constexpr (i < P_Q0) dp[1] = MT<T>::mfma32(f, dof[i - P_D1 - 1], dp[1]);
       else {
         constexpr int hf = i >= P_Q1 ? 1 : 0, j = i - (hf ? P_Q1 : P_Q0), kk = j / DB, d = j % DB;
-        dqacc[d] = MT<T>::mfma32(f, df[hf][kk], dqacc[d]);
+        if constexpr (WIDE) MT<T>::mfma32_acc(dqacc[d], f, df[hf][kk]);
+        else dqacc[d] = MT<T>::mfma32(f, df[hf][kk], dqacc[d]);
       }
     };
     // elements [k 16 / LEN, (k + 1) 16 / LEN) of half HF in slot START + k: P = exp2(s c - lse) (masked) ...
@@ -1965,13 +1998,13 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
       if constexpr (i + AHEAD < NS && has_frag(i + AHEAD)) fr[(i + AHEAD) % NF] = frag(std::integral_constant<int, i + AHEAD>{});
       mma(I, fr[i % NF]);
       // the next tile's loads, one per slot (past the last tile they re-read the last one: no branch here)
-      if constexpr (i < 2 * NLOAD) load_piece(I, t_next, buf ^ 1);
+      if constexpr (i < NLOAD2) load_piece(I, t_next, buf ^ 1);
       // P0 under dP0 (its S is complete from slot P_D0 on), dS0 under S1 (dP0 is complete from P_S1 on),
       // P1 under dP1, dS1 under dQ0; each group ends before the MFMAs that need its operand
       p_piece(I, I0{}, std::integral_constant<int, P_D0 + 1>{}, std::integral_constant<int, KSD - 1>{});
-      ds_piece(I, I0{}, std::integral_constant<int, P_S1 + 1>{}, std::integral_constant<int, KS - 1>{});
+      ds_piece(I, I0{}, std::integral_constant<int, P_S1 + 1>{}, std::integral_constant<int, (KS - 1 < 16 ? KS - 1 : 16)>{});
       p_piece(I, I1{}, std::integral_constant<int, P_D1 + 1>{}, std::integral_constant<int, KSD - 1>{});
-      ds_piece(I, I1{}, std::integral_constant<int, P_Q0 + 1>{}, std::integral_constant<int, A2 - 1>{});
+      ds_piece(I, I1{}, std::integral_constant<int, P_Q0 + 1>{}, std::integral_constant<int, (A2 - 1 < 16 ? A2 - 1 : 16)>{});
       __builtin_amdgcn_sched_barrier(0);
     });
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next tile has landed
@@ -1985,7 +2018,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
     nxt[j] = __builtin_amdgcn_readfirstlane(nxt[j]);
   }
   if (nact > 0) {
-    static_for<0, 2 * NLOAD>([&](auto P) { load_piece(P, cur[0], 0); });
+    static_for<0, NLOAD2>([&](auto P) { load_piece(P, cur[0], 0); });
   }
   __builtin_amdgcn_s_waitcnt(0);  // the fragments above and the first tile have landed (see the forward kernel)
   __syncthreads();
@@ -2002,7 +2035,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
     if (skip) {
       constexpr int buf = decltype(BUFc)::value;
       if (it + 1 < nact) {
-        static_for<0, 2 * NLOAD>([&](auto P) { load_piece(P, t_next, buf ^ 1); });
+        static_for<0, NLOAD2>([&](auto P) { load_piece(P, t_next, buf ^ 1); });
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       }
     } else if (need_mask) {
@@ -2020,6 +2053,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_plain_kernel(const BwdArgs
     if (it + 1 < nact) iteration(std::integral_constant<int, 1>{}, it + 1);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no LDS-writing load outlives the workgroup
+  if constexpr (WIDE) {
+    // the pinned accumulators are read by ordinary instructions from here on: past the last MFMA's latency
+#pragma unroll
+    for (int d = 0; d < DB; d++) asm volatile("s_nop 15\n\ts_nop 3" : "+a"(dqacc[d]) :: "memory");
+  }
 
   if (qrow < Sq) {
     T* dqp = (T*)a.dq + b * a.dqs[0] + h * a.dqs[1] + qrow * a.dqs[2];
@@ -2063,8 +2101,8 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
   // dK, dV
   {
     constexpr int BMQ = 64, BNK = 128;
-    // equal head dims up to 128: three row-major buffers (pipelined path); wide heads: one buffer with transposed copies
-    constexpr bool PIPE = DQK == DV && DQK <= 128;
+    // three row-major buffers (pipelined path) where they fit the LDS: every head-dim pair built today
+    constexpr bool PIPE = 3 * (DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES) <= 144 * 1024;
     constexpr int NBUF = PIPE ? 3 : 1;
     constexpr int BUF = DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES + (PIPE ? 0 : (DQK + DV) * TrTile64::ROW_BYTES);
     constexpr int ROWS = 3 * BMQ * 16;
@@ -2086,14 +2124,17 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
   mark(ev, 2, st);
   // dQ
   // (segments with causality; segments alone share an instantiation with the mask extensions: the general kernel below)
-  constexpr bool LEAN_DQ = DQK == DV && DQK <= 128 && (!SEG || CAUSAL);
+  // (unequal head dims without causality stay with the general kernel too: the compiler copies the pinned accumulators
+  // between the branches of that variant's loop, right behind the MFMAs that write them)
+  constexpr bool LEAN_DQ = (!SEG || CAUSAL) && (DQK == DV || CAUSAL);
   constexpr int DQ_BN = 64;
-  const size_t lean_smem = 4 * (size_t)DmaTile<DQK, true>::BYTES + (SEG ? 2 * DQ_BN * 4 + 16 * (size_t)((a.Skv + DQ_BN - 1) / DQ_BN) : 0);
+  const size_t lean_smem = 2 * (size_t)(DmaTile<DQK, true>::BYTES + DmaTile<DV, true>::BYTES) +
+                           (SEG ? 2 * DQ_BN * 4 + 16 * (size_t)((a.Skv + DQ_BN - 1) / DQ_BN) : 0);
   bool lean_done = false;
   if constexpr (LEAN_DQ) {
     if (lean_smem <= 160 * 1024) {  // (the list of a very long sequence does not fit: the general kernel then)
       constexpr int BM = 128;
-      auto kern = attn_bwd_dq_plain_kernel<T, DQK, CAUSAL, SEG>;
+      auto kern = attn_bwd_dq_plain_kernel<T, DQK, DV, CAUSAL, SEG>;
       static bool attr_set = false;
       if (!attr_set) {
         int rc = set_max_lds(kern, "tp_attn_bwd(dq)");
@@ -2158,9 +2199,14 @@ int bwd_by_dims_bf16(const BwdArgs& a, int Dqk, int Dv, int causal, hipStream_t 
 int bwd_by_dims_f16(const BwdArgs& a, int Dqk, int Dv, int causal, hipStream_t st, void* const* ev);
 template <typename T>
 static int bwd_by_dims(const BwdArgs& a, int Dqk, int Dv, int causal, hipStream_t st, void* const* ev) {
+  // (TP_ONLY_HEAD_DIM_128 / TP_ONLY_HEAD_DIM_WIDE: build options for quick timing builds of one head-dim pair)
+#ifndef TP_ONLY_HEAD_DIM_WIDE
   if (Dqk == 128 && Dv == 128) return dispatch_bwd<T, 128, 128>(a, causal, st, ev);
-#ifndef TP_ONLY_HEAD_DIM_128  // (a build option for quick timing builds of the head dim the benchmark runs)
+#endif
+#if !defined(TP_ONLY_HEAD_DIM_128) && !defined(TP_ONLY_HEAD_DIM_WIDE)
   if (Dqk == 64 && Dv == 64) return dispatch_bwd<T, 64, 64>(a, causal, st, ev);
+#endif
+#ifndef TP_ONLY_HEAD_DIM_128
   if (Dqk == 192 && Dv == 128) return dispatch_bwd<T, 192, 128>(a, causal, st, ev);
 #endif
   return TP_DIMS_NOT_BUILT;
