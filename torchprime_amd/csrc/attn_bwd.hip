@@ -6,18 +6,21 @@
 //     dV = P^T dO;  dS = P o (dO V^T - delta);  dQ = sm_scale dS K;  dK = sm_scale dS^T Q
 // and dK, dV summed over the n_rep query heads that share a KV head.
 //
-// Three kernels:
+// Kernels:
 //   attn_delta_kernel     -delta[b,h,i] = -sum_d dO*O, and the LSE in log2 units      (HBM-bound)
 //   attn_bwd_dkdv_kernel  one workgroup = 128 KV rows of one (batch, kv head); K and V fragments stay
-//                         in registers, Q / dO tiles of every query head of the group stream through
-//                         LDS in both orientations (row-major for S = QK^T and dP = dO V^T, transposed
+//                         in registers, row-major Q / dO tiles of every query head of the group stream through
+//                         three LDS buffers (fragment reads for S = QK^T and dP = dO V^T, transposing reads
 //                         for dV^T += dO^T P and dK^T += Q^T dS).  S is computed un-transposed here so
 //                         that a lane owns one KV column: P and dS converted to 16 bit are directly the
 //                         B operands of the two accumulating products.
-//   attn_bwd_dq_kernel    one workgroup = 128 or 256 query rows (4 or 8 waves) of one (batch, head); Q and dO fragments in
-//                         registers, K (row-major + transposed) and V (row-major) tiles stream through
-//                         LDS; S^T, dP^T are computed transposed (a lane owns one query column, so LSE
-//                         and delta are per-lane scalars) and dS^T feeds dQ^T += K^T dS^T.
+//   attn_bwd_dq_plain_kernel  dQ without mask extensions (plain, causal, causal with segment ids): one workgroup =
+//                         128 query rows of one (batch, head); Q and dO fragments in registers, row-major K and V
+//                         tiles stream through two LDS buffers; S^T, dP^T are computed transposed (a lane owns one
+//                         query column, so LSE and delta are per-lane scalars) and dS^T feeds dQ^T += K^T dS^T,
+//                         whose K^T operand comes out of transposing reads.
+//   attn_bwd_dq_kernel    the general dQ kernel (mask extensions, segment ids without causality): 4 or 8 waves,
+//                         K (row-major + transposed copy) and V tiles staged through registers.
 // Splitting dQ from dK/dV recomputes S and dP once more but needs no atomics: fp32 atomic adds reach
 // about 1.3 TB/s on this part, an order of magnitude short of what accumulating dQ tiles would need.
 #include <type_traits>
@@ -183,35 +186,6 @@ struct Stage64 {
   }
 };
 
-// transposed copy of a DmaTile: every thread turns 4-row x 8-column blocks into 8-byte column pieces
-template <int D>
-__device__ __forceinline__ void transpose_tile(const unsigned char* src, unsigned char* dst, int tid) {
-  constexpr int CPR = D / 8, TOT = CPR * 16, ITEMS = (TOT + 255) / 256;
-#pragma unroll
-  for (int i = 0; i < ITEMS; i++) {
-    const int item = tid + 256 * i;
-    if (item < TOT) {
-      const int c8 = item % CPR, rq = item / CPR;
-      u32x4 r[4];
-#pragma unroll
-      for (int ii = 0; ii < 4; ii++) r[ii] = *(const u32x4*)(src + DmaTile<D>::off(4 * rq + ii, c8));
-      // odd column blocks take their columns in the order 1,0,3,2,...: at every step half the lanes write
-      // even LDS rows and half odd ones, which spreads the 8-byte stores over all banks
-      const int flip = c8 & 1;
-      const unsigned sel_even = flip ? 0x07060302u : 0x05040100u, sel_odd = flip ? 0x05040100u : 0x07060302u;
-#pragma unroll
-      for (int j = 0; j < 8; j++) {
-        const unsigned sel = (j & 1) ? sel_odd : sel_even;
-        const int w = j >> 1;
-        u32x2 o;
-        o.x = __builtin_amdgcn_perm(r[1][w], r[0][w], sel);
-        o.y = __builtin_amdgcn_perm(r[3][w], r[2][w], sel);
-        *(u32x2*)(dst + TrTile64::quad_off(c8 * 8 + (j ^ flip), rq)) = o;
-      }
-    }
-  }
-}
-
 // 4 bytes per lane straight into LDS at dst + 4 * lane (a 64-entry row vector per instruction)
 __device__ __forceinline__ void dma_dword(u32x4 rs, unsigned byte_offset, unsigned char* dst, int lane) {
   const unsigned d = __builtin_amdgcn_readfirstlane((unsigned)(size_t)dst);
@@ -223,87 +197,6 @@ __device__ __forceinline__ void dma_dword_at(u32x4 rs, unsigned byte_offset, uns
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, %3 offen lds"
                :: "s"(dst), "v"((unsigned)lane * 4u), "s"(rs), "s"(byte_offset) : "memory", "m0");
 }
-// The same transposition as transpose_tile, cut into steps that can be placed between MFMAs: read() fetches
-// this thread's 4-row x 8-column block, write(J) stores column pair member J (0..7) as 8 bytes.  Threads
-// are assigned to blocks so that the 32 lanes served together write 32 different bank pairs; threads beyond
-// the number of blocks repeat the work of an earlier one (same values to the same addresses).
-template <int D>
-struct TransposeSteps {
-  static constexpr int CPR = D / 8, TOT = CPR * 16;
-  static_assert(TOT <= 256, "one block per thread");
-  u32x4 r[4];
-  unsigned rd, zs, wo[8], sel_even, sel_odd;
-  // bias: added to every store offset (write() is then given destinations less that amount: a caller whose
-  // transposed tiles lie beyond the reach of a 16-bit instruction offset keeps the excess in these registers)
-  __device__ __forceinline__ void init(int tid, unsigned bias) {
-    const int item = tid % TOT, c8 = item % CPR, rqi = item / CPR;
-    const int rq = (rqi & ~3) | ((rqi & 1) << 1) | ((rqi >> 1) & 1);
-    rd = (unsigned)(4 * rq * DmaTile<D>::ROWB);
-    zs = (unsigned)((c8 ^ DmaTile<D>::swz(4 * rq)) << 4);
-    const int flip = c8 & 1;
-    const int k = (((c8 & 1) << 2) ^ (c8 >> 1)) & 7, rqc = 2 * (rq >> 2) + (rq & 1);
-    const unsigned wbase = (unsigned)(c8 * 8 * TrTile64::ROW_BYTES + (((rq >> 1) & 1) << 3));
-    const unsigned y = (unsigned)((flip << 7) | ((rqc ^ k) << 4));
-#pragma unroll
-    for (int j = 0; j < 8; j++) wo[j] = bias + wbase + (y ^ (unsigned)(((j & 1) << 7) | ((j >> 1) << 4)));
-    sel_even = flip ? 0x07060302u : 0x05040100u;
-    sel_odd = flip ? 0x05040100u : 0x07060302u;
-  }
-  __device__ __forceinline__ void read(const unsigned char* src) {
-#pragma unroll
-    for (int ii = 0; ii < 4; ii++) {
-      const unsigned sw = (unsigned)((CPR % 16 == 0 ? ii : (ii >> 1)) << 4);
-      r[ii] = *(const u32x4*)(src + rd + (zs ^ sw) + ii * DmaTile<D>::ROWB);
-    }
-  }
-  template <typename J>
-  __device__ __forceinline__ void write(unsigned char* dst, J) const {
-    constexpr int j = J::value, w = j >> 1;
-    const unsigned sel = (j & 1) ? sel_odd : sel_even;
-    u32x2 o;
-    o.x = __builtin_amdgcn_perm(r[1][w], r[0][w], sel);
-    o.y = __builtin_amdgcn_perm(r[3][w], r[2][w], sel);
-    *(u32x2*)(dst + wo[j] + (j >> 1) * 2 * TrTile64::ROW_BYTES) = o;
-  }
-};
-
-// TransposeSteps with its state cut to six registers (store offsets are formed per store from two of them) and
-// the block's data held by the caller, for kernels that run several of these side by side; any number of
-// blocks per tile (a caller with fewer threads than blocks makes more than one round: init(tid + round * threads)).
-template <int D>
-struct TransposeLean {
-  static constexpr int CPR = D / 8, TOT = CPR * 16;
-  unsigned rd, zs, wb, y, sel_even, sel_odd;
-  __device__ __forceinline__ void init(int idx) {
-    const int item = idx % TOT, c8 = item % CPR, rqi = item / CPR;
-    const int rq = (rqi & ~3) | ((rqi & 1) << 1) | ((rqi >> 1) & 1);
-    rd = (unsigned)(4 * rq * DmaTile<D>::ROWB);
-    zs = (unsigned)((c8 ^ DmaTile<D>::swz(4 * rq)) << 4);
-    const int flip = c8 & 1;
-    const int k = (((c8 & 1) << 2) ^ (c8 >> 1)) & 7, rqc = 2 * (rq >> 2) + (rq & 1);
-    wb = (unsigned)(c8 * 8 * TrTile64::ROW_BYTES + (((rq >> 1) & 1) << 3));
-    y = (unsigned)((flip << 7) | ((rqc ^ k) << 4));
-    sel_even = flip ? 0x07060302u : 0x05040100u;
-    sel_odd = flip ? 0x05040100u : 0x07060302u;
-  }
-  __device__ __forceinline__ void read(const unsigned char* src, u32x4 (&r)[4]) const {
-#pragma unroll
-    for (int ii = 0; ii < 4; ii++) {
-      const unsigned sw = (unsigned)((CPR % 16 == 0 ? ii : (ii >> 1)) << 4);
-      r[ii] = *(const u32x4*)(src + rd + (zs ^ sw) + ii * DmaTile<D>::ROWB);
-    }
-  }
-  template <int J>
-  __device__ __forceinline__ void write(unsigned char* dst, const u32x4 (&r)[4]) const {
-    constexpr int w = J >> 1;
-    const unsigned sel = (J & 1) ? sel_odd : sel_even;
-    u32x2 o;
-    o.x = __builtin_amdgcn_perm(r[1][w], r[0][w], sel);
-    o.y = __builtin_amdgcn_perm(r[3][w], r[2][w], sel);
-    *(u32x2*)(dst + wb + (y ^ (unsigned)(((J & 1) << 7) | ((J >> 1) << 4))) + (J >> 1) * 2 * TrTile64::ROW_BYTES) = o;
-  }
-};
-
 // ------------------------------------------------------------------------------------------------
 // dK / dV
 // ------------------------------------------------------------------------------------------------
@@ -314,20 +207,17 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   constexpr int BNK = 128;  // kv rows per workgroup, 32 per wave
   constexpr int KS_QK = DQK / 16, KS_DV = DV / 16;
   constexpr int DKB = DQK / 32, DVB = DV / 32;
-  // PIPE: three row-major buffers, no transposed copies: the operands of the two accumulating products are read
-  // from the row-major tiles with transposing LDS reads (every head-dim pair whose three buffers fit the LDS).
-  constexpr bool PIPE = NBUF == 3;
-  static_assert(PIPE || NBUF == 1, "three buffers (pipelined path) or one");
-  typedef DmaTile<DQK, PIPE> QT;
-  typedef DmaTile<DV, PIPE> OT;
+  // Three row-major buffers of Q and dO tiles, no transposed copies: the operands of the two accumulating products
+  // are read from the row-major tiles with transposing LDS reads.
+  static_assert(NBUF == 3, "the tile loop rotates three buffers");
+  typedef DmaTile<DQK, true> QT;
+  typedef DmaTile<DV, true> OT;
   constexpr int Q_BYTES = QT::BYTES, DO_BYTES = OT::BYTES;
-  constexpr int QTR_BYTES = PIPE ? 0 : DQK * TrTile64::ROW_BYTES, DOTR_BYTES = PIPE ? 0 : DV * TrTile64::ROW_BYTES;
-  constexpr int ROW_BYTES = BMQ * 4 * 4;  // lse (log2 units), delta, segment id per query row (+1 unused): 3 slots
-  constexpr int BUF_BYTES = Q_BYTES + DO_BYTES + QTR_BYTES + DOTR_BYTES;
-  // LDS layout: the NBUF copies of each kind of tile lie side by side (Q.. dO.. Q^T.. dO^T.., then the row
-  // vectors), so that with the buffer index a constant every fragment address is a loop-invariant per-lane
-  // offset plus an immediate
-  constexpr int Q_AT = 0, DO_AT = NBUF * Q_BYTES, QTR_AT = DO_AT + NBUF * DO_BYTES, DOTR_AT = QTR_AT + NBUF * QTR_BYTES;
+  constexpr int ROW_BYTES = BMQ * 4 * 4;  // lse (log2 units), delta, segment id, position per query row
+  constexpr int BUF_BYTES = Q_BYTES + DO_BYTES;
+  // LDS layout: the NBUF copies of each kind of tile lie side by side (Q.. dO.., then the row vectors), so that with
+  // the buffer index a constant every fragment address is a loop-invariant per-lane offset plus an immediate
+  constexpr int Q_AT = 0, DO_AT = NBUF * Q_BYTES;
 
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -454,13 +344,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   };
 
   // per-lane byte offsets of the MFMA fragments inside a tile (the swizzles are resolved once, here)
-  unsigned faq[KS_QK], fao[KS_DV], ta[4];
+  unsigned faq[KS_QK], fao[KS_DV];
 #pragma unroll
   for (int ks = 0; ks < KS_QK; ks++) faq[ks] = (unsigned)QT::off(ln, 2 * ks + g);
 #pragma unroll
   for (int ks = 0; ks < KS_DV; ks++) fao[ks] = (unsigned)OT::off(ln, 2 * ks + g);
-#pragma unroll
-  for (int m = 0; m < 4; m++) ta[m] = (unsigned)TrTile64::chunk_off(ln, m, g);
 
   f32x16 dkacc[DKB], dvacc[DVB];
   {
@@ -508,7 +396,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
     if (++idx == nact) { idx = 0; hl++; }
   };
 
-  if constexpr (PIPE) {
+  {
     // Software pipeline over query tiles t, three row-major buffers and three row-vector slots (tile t lives in
     // buffer and slot t % 3), one barrier per tile:
     //   part 1 (S, dP: fragment reads of buffer t % 3)
@@ -868,224 +756,6 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
       iteration(std::integral_constant<int, 0>{}, it);
       if (it + 1 < n_iter) iteration(std::integral_constant<int, 1>{}, it + 1);
       if (it + 2 < n_iter) iteration(std::integral_constant<int, 2>{}, it + 2);
-    }
-  } else {
-    // Wide heads: one buffer of each kind; both query blocks go through each step together.  Per tile:
-    //   part 1  S = Q K^T, dP = dO V^T from the row-major tiles; between the S MFMAs the same tile is copied into
-    //           its transposed form (that copy only reads the row-major tiles, and nobody reads the transposed
-    //           ones before the barrier); between the dP MFMAs P = exp2(S c - LSE) is computed and packed
-    //   barrier  row-major tiles free, transposed tiles complete; the next tile's loads are issued into the former
-    //   part 2  dV^T += dO^T P with dS = P o (dP - delta) computed between its MFMAs, then dK^T += Q^T dS
-    //   wait for the loads, barrier
-    // Every MFMA's LDS fragment is requested RING MFMAs ahead; row vectors alternate two slots.
-    constexpr int QB = BMQ / 32, RING = 4;
-    constexpr int NS = KS_QK * QB, NA = NS + KS_DV * QB;          // part 1: S steps, then dP steps
-    constexpr int NV = (BMQ / 16) * DVB, NB = NV + (BMQ / 16) * DKB;  // part 2: dV steps, then dK steps
-    constexpr int NCH = 16 * QB;                                  // values per lane of S (and of dP)
-    static_assert(NA - NS == NCH / 2 && NV >= NCH / 2 && NS >= 18, "two values per step under dP and under dV");
-    TransposeLean<DQK> trq0, trq1;
-    TransposeLean<DV> tro;
-    trq0.init(tid);
-    trq1.init(tid + 256);  // 384 blocks for 256 threads: the second round of threads 128..255 repeats blocks 0..127
-    tro.init(tid);
-    static_assert(TransposeLean<DQK>::TOT <= 512 && TransposeLean<DV>::TOT <= 256, "two rounds for Q, one for dO");
-    unsigned char* const qtw = smem + QTR_AT;
-    unsigned char* const dotw = smem + DOTR_AT;
-    const int kvcol = wkv0 + ln;
-    int c_hl = 0, c_idx = 0, n_hl = 0, n_idx = 0;
-    if (n_iter > 0) {
-      issue_tile(0, 0, 0, 0);
-      advance(n_hl, n_idx);
-      __builtin_amdgcn_s_waitcnt(0);
-      __syncthreads();
-    }
-    for (int it = 0; it < n_iter; it++) {
-      const int qi0 = qtile_of(c_idx) * BMQ;
-      const int mode = tile_mode(c_idx, qi0);
-      const unsigned char* ql = smem + Q_AT;
-      const unsigned char* dol = smem + DO_AT;
-      const unsigned char* qtl = smem + QTR_AT;
-      const unsigned char* dotl = smem + DOTR_AT;
-      const float* lsel = (const float*)(rows_base + (it & 1) * ROW_BYTES);
-      const float* deltal = lsel + BMQ;
-      const int* segl = (const int*)(deltal + BMQ);
-      const int* posl = segl + BMQ;  // query positions of the tile's rows (mask extensions)
-      const float* bias_head = biased ? a.mx.bias + b * a.mx.bias_s[0] + (hk * a.n_rep + c_hl) * a.mx.bias_s[1] : nullptr;
-      f32x16 sacc[QB], dpacc[QB];
-      float fcap[GEN ? QB : 1][16];  // soft cap: 1 - tanh^2 of every score, kept from P to dS
-      v8 pfr[BMQ / 16];
-      u32x4 trd[4];
-      // transposition of this tile in 3 reads and 12 double stores, placed at steps T0.. of part 1
-      auto tr_piece = [&](auto K) {
-        constexpr int k = decltype(K)::value;  // 0..17: per block one read step, one idle step, four store steps
-        constexpr int blk = k / 6, w = k % 6;
-        if constexpr (w == 0) {
-          if constexpr (blk == 0) trq0.read(ql, trd);
-          else if constexpr (blk == 1) trq1.read(ql, trd);
-          else tro.read(dol, trd);
-        } else if constexpr (w >= 2) {
-          constexpr int j = 2 * (w - 2);
-          if constexpr (blk == 0) { trq0.template write<j>(qtw, trd); trq0.template write<j + 1>(qtw, trd); }
-          else if constexpr (blk == 1) { trq1.template write<j>(qtw, trd); trq1.template write<j + 1>(qtw, trd); }
-          else { tro.template write<j>(dotw, trd); tro.template write<j + 1>(dotw, trd); }
-        }
-      };
-      auto part1 = [&](auto masked_c) {
-        constexpr bool MASKED = decltype(masked_c)::value;
-        const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        auto a_frag = [&](auto I) {
-          constexpr int i = decltype(I)::value;
-          if constexpr (i < NS) return *(const v8*)(ql + faq[i / QB] + (i % QB) * 32 * QT::ROWB);
-          else return *(const v8*)(dol + fao[(i - NS) / QB] + ((i - NS) % QB) * 32 * OT::ROWB);
-        };
-        v8 ring[RING];
-        f32x4 l4[NCH / 4];
-        // masked tiles: one bit per query row of the tile for this lane's kv column (see the pipelined path)
-        unsigned rowbits[2] = {0u, 0u};
-        const bool by_bits = MASKED && !(GEN && ext);  // (the mask extensions are evaluated element by element)
-        if (MASKED && by_bits) {
-          const int lo_r = CAUSAL ? max(kvcol - qi0, 0) : 0;
-          const int hi_r = kvcol < Skv ? min(Sq - qi0, BMQ) : 0;
-          unsigned long long m = 0ull;
-          if (hi_r > lo_r) m = (~0ull << lo_r) & (~0ull >> (64 - hi_r));
-          if (SEG && has_seg) {
-            const int rowseg = segl[lane];
-            unsigned long long ms = 0ull, todo = ~0ull;
-            while (todo) {
-              const int x = __builtin_amdgcn_readlane(segk, (int)__builtin_ctzll(todo));
-              const unsigned long long rows = __ballot(rowseg == x);
-              const bool mine = segk == x;
-              ms = mine ? rows : ms;
-              todo &= ~__ballot(mine);
-            }
-            m &= ms;
-          }
-          rowbits[0] = (unsigned)m >> (4 * g);
-          rowbits[1] = (unsigned)(m >> 32) >> (4 * g);
-        }
-        static_for<0, RING>([&](auto R) { ring[decltype(R)::value] = a_frag(R); });
-        static_for<0, NA>([&](auto I) {
-          constexpr int i = decltype(I)::value;
-          if constexpr (i < 18) tr_piece(I);
-          if constexpr (i < NS) sacc[i % QB] = MT<T>::mfma32(ring[i % RING], kf[i / QB], i < QB ? zero16 : sacc[i % QB]);
-          else dpacc[(i - NS) % QB] = MT<T>::mfma32(ring[i % RING], vf[(i - NS) / QB], i - NS < QB ? zero16 : dpacc[(i - NS) % QB]);
-          if constexpr (i + RING < NA) ring[i % RING] = a_frag(std::integral_constant<int, i + RING>{});
-          // row vector quad m is used at steps NS + 2m, NS + 2m + 1 and requested four steps before
-          if constexpr (i + 4 >= NS && (i + 4 - NS) % 2 == 0 && (i + 4 - NS) / 2 < NCH / 4) {
-            constexpr int m = (i + 4 - NS) / 2, qb = m / 4, vq = m % 4;
-            l4[m] = *(const f32x4*)(lsel + qb * 32 + 8 * vq + 4 * g);
-          }
-          if constexpr (i >= NS) {
-            // P = exp2(S c - LSE) for two values (l4 holds -LSE in log2 units); rows of the C tile are queries
-            constexpr int k = i - NS;
-#pragma unroll
-            for (int idx = 2 * k; idx < 2 * k + 2; idx++) {
-              const int qb = idx / 16, v = idx % 16, m = idx / 4, e = idx % 4;
-              float sval = sacc[qb][v];
-              if constexpr (GEN && MASKED) {
-                if (capped) {
-                  const float th = fast_tanh(sval * a.mx.cap_in);
-                  fcap[GEN ? qb : 0][v] = 1.f - th * th;
-                  sval = a.mx.cap_out * th;
-                }
-                if (biased) {  // additive mask, in units of the raw score (-inf stays -inf)
-                  const int qrow_b = min(qi0 + qb * 32 + 8 * (v / 4) + 4 * g + e, Sq - 1);
-                  sval += a.mx.bias_mul * bias_head[(int64_t)qrow_b * a.mx.bias_s[2] + min(kvcol, Skv - 1)];
-                }
-              }
-              float pv = fast_exp2(__builtin_fmaf(sval, c, l4[m][e]));
-              if constexpr (MASKED) {
-                if (by_bits) {
-                  pv = __uint_as_float(__float_as_uint(pv) & (unsigned)__builtin_amdgcn_sbfe((int)rowbits[qb], 8 * (v / 4) + e, 1));
-                } else {
-                  const int r = qb * 32 + 8 * (v / 4) + 4 * g + e;
-                  const int qrow = qi0 + r;
-                  bool ok = qrow < Sq && kvcol < Skv && (!CAUSAL || kvcol <= qrow) && (!SEG || !has_seg || segl[r] == segk);
-                  const int qp = has_pos ? posl[r] : qrow;
-                  ok = ok && kvcol >= qp - a.mx.lo_off && kvcol <= qp + a.mx.hi_off;
-                  pv = ok ? pv : 0.f;
-                }
-              }
-              asm volatile("" : "+v"(pv));  // keeps the computation in this step
-              sacc[qb][v] = pv;
-            }
-            if constexpr (k % 4 == 3) {
-              constexpr int h = k / 4, qb = h / 2, hh = h % 2;
-              const f32x16& x = sacc[qb];
-              pfr[h] = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4], x[8 * hh + 5],
-                                x[8 * hh + 6], x[8 * hh + 7]);
-            }
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        });
-      };
-      if (mode == 0) {
-        static_for<0, 18>([&](auto K) { tr_piece(K); });  // this wave's share of the copy, nothing to multiply
-      } else if (mode == 2) {
-        part1(std::true_type{});
-      } else {
-        part1(std::false_type{});
-      }
-      __syncthreads();  // everyone is done with the row-major tiles; the transposed ones are complete
-      if (it + 1 < n_iter) {
-        issue_tile(n_hl, n_idx, 0, (it + 1) & 1);
-        advance(n_hl, n_idx);
-      }
-      if (mode != 0) {
-        // dV^T += dO^T P,  dK^T += Q^T dS  (contraction over the 64 query rows); the accumulators are pinned to the
-        // accumulation registers, as in the pipelined path
-        auto t_frag = [&](auto I) {
-          constexpr int i = decltype(I)::value;
-          if constexpr (i < NV) {
-            constexpr int ks = i / DVB, d = i % DVB;
-            return *(const v8*)(dotl + ta[ks ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
-          } else {
-            constexpr int ks = (i - NV) / DKB, d = (i - NV) % DKB;
-            return *(const v8*)(qtl + ta[ks ^ (d & 3)] + d * 32 * TrTile64::ROW_BYTES);
-          }
-        };
-        v8 ring[RING], dsf[BMQ / 16];
-        f32x4 d4[NCH / 4];
-        static_for<0, RING>([&](auto R) { ring[decltype(R)::value] = t_frag(R); });
-        static_for<0, 2>([&](auto M) {
-          constexpr int m = decltype(M)::value;
-          d4[m] = *(const f32x4*)(deltal + (m / 4) * 32 + 8 * (m % 4) + 4 * g);
-        });
-        __builtin_amdgcn_sched_barrier(0);
-        static_for<0, NB>([&](auto I) {
-          constexpr int i = decltype(I)::value;
-          if constexpr (i < NV) MT<T>::mfma32_acc_guarded(dvacc[i % DVB], ring[i % RING], pfr[i / DVB]);
-          else MT<T>::mfma32_acc_guarded(dkacc[(i - NV) % DKB], ring[i % RING], dsf[(i - NV) / DKB]);
-          if constexpr (i + RING < NB) ring[i % RING] = t_frag(std::integral_constant<int, i + RING>{});
-          if constexpr (i % 2 == 0 && i / 2 + 2 < NCH / 4) {
-            constexpr int m = i / 2 + 2;
-            d4[m] = *(const f32x4*)(deltal + (m / 4) * 32 + 8 * (m % 4) + 4 * g);
-          }
-          if constexpr (i < NCH / 2) {
-            // dS = P o (dP - delta) for two values (d4 holds -delta)
-#pragma unroll
-            for (int idx = 2 * i; idx < 2 * i + 2; idx++) {
-              const int qb = idx / 16, v = idx % 16, m = idx / 4, e = idx % 4;
-              float dsv = sacc[qb][v] * (dpacc[qb][v] + d4[m][e]);
-              if constexpr (GEN) {
-                if (mode == 2 && capped) dsv *= fcap[GEN ? qb : 0][v];  // derivative of the capped score
-              }
-              asm volatile("" : "+v"(dsv));
-              dpacc[qb][v] = dsv;
-            }
-            if constexpr (i % 4 == 3) {
-              constexpr int h = i / 4, qb = h / 2, hh = h % 2;
-              const f32x16& x = dpacc[qb];
-              dsf[h] = pack8<T>(x[8 * hh + 0], x[8 * hh + 1], x[8 * hh + 2], x[8 * hh + 3], x[8 * hh + 4], x[8 * hh + 5],
-                                x[8 * hh + 6], x[8 * hh + 7]);
-            }
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        });
-      }
-      __builtin_amdgcn_s_waitcnt(0);
-      __syncthreads();  // the next tile has landed; everyone is done with the transposed tiles
-      advance(c_hl, c_idx);
     }
   }
 
@@ -2101,10 +1771,10 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
   // dK, dV
   {
     constexpr int BMQ = 64, BNK = 128;
-    // three row-major buffers (pipelined path) where they fit the LDS: every head-dim pair built today
-    constexpr bool PIPE = 3 * (DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES) <= 144 * 1024;
-    constexpr int NBUF = PIPE ? 3 : 1;
-    constexpr int BUF = DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES + (PIPE ? 0 : (DQK + DV) * TrTile64::ROW_BYTES);
+    // three row-major buffers of Q and dO tiles
+    constexpr int NBUF = 3;
+    constexpr int BUF = DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES;
+    static_assert(NBUF * BUF <= 144 * 1024, "the three buffers must leave room for the row vectors and the tile list");
     constexpr int ROWS = 3 * BMQ * 16;
     const int nqt = (a.Sq + BMQ - 1) / BMQ;
     const size_t smem = (size_t)NBUF * BUF + ROWS + (SEG ? (size_t)(6 * nqt + 8 + 4) * 4 : 0);
