@@ -8,11 +8,11 @@
 //     one query column and 16 key rows per 32x32 block: row max / sum / rescale are per-lane scalars
 //     (one half-wave exchange per tile), and exp(S^T) converted to 16 bit is already the B operand of
 //     O^T += V^T P^T - P never goes through LDS;
-//   * Q fragments stay in registers for the whole KV loop; K tiles are row-major in LDS (dense rows, 16-byte
-//     chunks XOR-swizzled by the row), V tiles are transposed while being written to LDS, so both are read with
-//     conflict-free 16-byte loads;
-//   * the next tile is fetched while the current one is being multiplied: K by buffer loads that write LDS
-//     directly, V from HBM into registers (its transposition needs them); LDS double buffer, one barrier per tile;
+//   * Q fragments stay in registers for the whole KV loop; K and V tiles are row-major in LDS (dense rows, 16-byte
+//     chunks XOR-swizzled by the row): K fragments are conflict-free 16-byte reads, the V^T operand comes out of
+//     transposing 8-byte reads of the same kind of tile;
+//   * the next tile is fetched while the current one is being multiplied, K and V by buffer loads that write LDS
+//     directly (no staging registers, no LDS stores); LDS double buffer, one barrier per tile;
 //   * causal: the KV loop ends at the diagonal, element masks only on tiles that straddle it;
 //     segments: per-tile [min,max] of the ids is computed once per workgroup, tiles whose id range
 //     misses the query rows' range are skipped, element compares only where ranges are not one id.
@@ -40,12 +40,10 @@ struct FwdArgs {
 // or LDS and take one workgroup per CU instead of spilling a hundred registers.
 template <int DQK, bool CAUSAL, bool SEG>
 constexpr int fwd_blocks_per_cu() { return (DQK >= 128 && !CAUSAL) || (DQK > 128 && SEG) ? 1 : 2; }
-// K tiles are filled by buffer loads that write LDS directly (DmaTile): no staging registers for K, no LDS stores
-// for it, and dense swizzled rows instead of padded ones.  For the causal 192-wide heads that is what lets two
-// workgroups share a CU: 254 registers instead of 289, and two double-buffered tile sets of 81920 bytes fill the
-// CU's 160 KB exactly (forward at 128 heads x 4096 rows: 1.16 -> 0.89 ms).  The other variants gain 2-7 % over staging
-// K through registers (same-box A/B: head dim 64 causal 2.6 %, 128 causal 3 %, 128 causal with segment ids 7 % - it
-// also stopped spilling -, 128 and 192 non-causal 3.4 and 3.9 %).
+// The tiles are filled by buffer loads that write LDS directly (DmaTile): no staging registers, no LDS stores, and
+// dense swizzled rows instead of padded ones.  For the causal 192-wide heads that is what lets two workgroups share a
+// CU: two double-buffered tile sets of 81920 bytes fill the CU's 160 KB exactly (forward at 128 heads x 4096 rows:
+// 1.16 -> 0.89 ms with K loaded that way, 0.72 ms with V as well).
 
 template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
 __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void attn_fwd_kernel(const FwdArgs a) {
