@@ -413,6 +413,30 @@ def test_long_packed_sequence_65536_rows():
     assert_close(dv[sl], dv_ref, f"dv, document {d}", scale_abs=True)
 
 
+def test_long_packed_sequence_with_wide_heads():
+  """S = 32768 with packed documents at head dims (192, 128), two query heads on one kv head: the tile lists of the
+  three-buffer dK/dV pipeline (120 KB of tiles) and of the lean dQ kernel at their longest tested; checked document by
+  document like the case above."""
+  B, Hq, Hkv, S, D, Dv = 1, 2, 1, 32768, 192, 128
+  seg, lengths = packed_segment_ids(B, S, 200, 3000, seed=12)
+  q, k, v, do = (heads_view(B, h, S, d, 30 + i, torch.bfloat16)
+                 for i, (h, d) in enumerate(((Hq, D), (Hkv, D), (Hkv, Dv), (Hq, Dv))))
+  out, lse, dq, dk, dv = _run(q, k, v, do, seg, True, Dv**-0.5)
+  for t in (out, dq, dk, dv):
+    assert torch.isfinite(t.float()).all()
+  starts = [0]
+  for L in lengths[0]:
+    starts.append(starts[-1] + L)
+  for d in (0, len(lengths[0]) // 2, len(lengths[0]) - 1):
+    a, b_ = starts[d], starts[d + 1]
+    sl = (slice(None), slice(None), slice(a, b_))
+    o_ref, dq_ref, dk_ref, dv_ref = orc.attention_grads_ref(q[sl], k[sl], v[sl], do[sl], None, True, Dv**-0.5, torch.float32)
+    assert_close(out[sl], o_ref, f"out, document {d}")
+    assert_close(dq[sl], dq_ref, f"dq, document {d}", scale_abs=True)
+    assert_close(dk[sl], dk_ref, f"dk, document {d}", scale_abs=True)
+    assert_close(dv[sl], dv_ref, f"dv, document {d}", scale_abs=True)
+
+
 def test_unsupported_inputs_raise():
   q = torch.zeros((1, 2, 16, 96), dtype=torch.bfloat16, device=DEV)
   with pytest.raises(NotImplementedError):
