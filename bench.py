@@ -146,12 +146,19 @@ def bench_attention(args, dev):
 
   unit = B * Hq * S * S * D  # one causal matmul over the attention matrix: 2 * (S^2/2) * d per (b, h)
   flops_step = 6.0 * unit
-  # event layout per step: [before fwd, before delta, before dkdv, before dq, after dq]
+  # events per step: [0] before fwd, [1] after fwd, [2] after the delta kernel, [3] after dK/dV, [4] after dQ.  Where
+  # the dQ kernel computes delta itself there is no delta kernel and dQ runs before dK/dV ([4] is recorded before [3]).
+  from torchprime_amd import _lib
+
+  dq_first = bool(_lib.load().tp_attn_bwd_dq_first(S, D, D, 1, 0, 0, _lib.dtype_code(q.dtype)))
   names = ["attn_fwd", "attn_delta", "attn_bwd_dkdv", "attn_bwd_dq"]
+  spans = {"attn_fwd": (0, 1), "attn_delta": (1, 2), "attn_bwd_dkdv": (4, 3) if dq_first else (2, 3),
+           "attn_bwd_dq": (2, 4) if dq_first else (3, 4)}  # fmt: skip
   algo = {"attn_fwd": 2.0 * unit, "attn_delta": 0.0, "attn_bwd_dkdv": 3.0 * unit, "attn_bwd_dq": 1.0 * unit}
   avg = {}
-  for j, n in enumerate(names):
-    avg[n] = sum(hipev.elapsed_ms(ev[i][j], ev[i][j + 1]) for i in range(args.steps)) / args.steps
+  for n in names:
+    j0, j1 = spans[n]
+    avg[n] = sum(hipev.elapsed_ms(ev[i][j0], ev[i][j1]) for i in range(args.steps)) / args.steps
   kernels = {
     n: {"ms": round(avg[n], 4), "algorithmic_TFLOPs": round(algo[n] / (avg[n] * 1e-3) / 1e12, 2) if avg[n] > 0 else None}
     for n in names
@@ -678,6 +685,8 @@ def summarize_profiles(d, commit):
     timed_avg = {}
     for k in ("attn_fwd", "attn_delta", "attn_bwd_dkdv", "attn_bwd_dq"):
       v = [x[1] for x in sorted(per[k])]
+      if not v:
+        continue  # (no delta kernel where the dQ kernel computes delta itself)
       if len(v) != warm + steps:
         o.append(f"| {k} | {len(v)} | (expected {warm + steps} launches) | | | |")
         continue
@@ -725,6 +734,8 @@ def summarize_profiles(d, commit):
            "| kernel | dispatches | FETCH_SIZE avg | WRITE_SIZE avg | HBM read MiB | HBM write MiB |", "|---|---:|---:|---:|---:|---:|"]
       traffic = {}
       for k in ("attn_fwd", "attn_delta", "attn_bwd_dkdv", "attn_bwd_dq"):
+        if k not in fetch or k not in write:
+          continue
         rd, wr = fetch[k] * sf / 1024, write[k] * sw / 1024
         traffic[k] = float(f"{(rd + wr) * (1 << 20):.3g}")
         o.append(f"| {k}_kernel | {nf[k]} | {fetch[k]:.0f} | {write[k]:.0f} | {rd:.0f} | {wr:.0f} |")
@@ -766,6 +777,8 @@ def summarize_profiles(d, commit):
     tb = tm = 0.0
     clocks = []
     for k in ("attn_fwd", "attn_delta", "attn_bwd_dkdv", "attn_bwd_dq"):
+      if k not in A or k not in Bc:
+        continue
       a, bb = A[k], Bc[k]
       simd = 4 * a["SQ_BUSY_CU_CYCLES"]
       tb += simd

@@ -163,8 +163,11 @@ int tp_attn_bwd(const void* dout, const void* q, const void* k, const void* v, c
 
 /* tp_attn_bwd with timing marks.  No counterpart in the reference; for benchmarks and profilers that
  * want per-kernel times without an external tracer.  `events` is NULL or an array of four
- * hipEvent_t (as void*; individual entries may be NULL) recorded on `stream` before the delta
- * kernel, before the dK/dV kernel, before the dQ kernel and after it.  Nothing is synchronised. */
+ * hipEvent_t (as void*; individual entries may be NULL) recorded on `stream`: [0] before the first
+ * kernel, [1] after the delta kernel, [2] after the dK/dV kernel, [3] after the dQ kernel.  The kernels
+ * run in the order delta, dK/dV, dQ - or, where the dQ kernel computes delta itself
+ * (tp_attn_bwd_dq_first(...) != 0: no delta kernel, [1] follows [0] at once), dQ then dK/dV, so that
+ * [3] is recorded before [2].  Nothing is synchronised. */
 int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, const void* v, const void* out,
                    const float* lse, const int32_t* seg, void* dq, void* dk, void* dv, float* ws, int B,
                    int Hq, int Hkv, int Sq, int Skv, int Dqk, int Dv, const int64_t do_strides[3],
@@ -172,6 +175,11 @@ int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, const void* v
                    const int64_t o_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
                    const int64_t dv_strides[3], float sm_scale, int causal, int dtype, void* stream,
                    void* const* events);
+
+/* 1 when tp_attn_bwd / tp_attn_bwd_ex run the dQ kernel first for such a problem (it then computes
+ * rowsum(dO o O) itself and there is no separate pass over dO and O), else 0.  `masked`: called through
+ * tp_attn_bwd_masked / tp_attn_bwd_biased.  No counterpart in the reference (see tp_attn_bwd_ex). */
+int tp_attn_bwd_dq_first(int Skv, int Dqk, int Dv, int causal, int has_seg, int masked, int dtype);
 
 /* ------------------------------------------------------------------------------------------------
  * Mask extensions of the functional API (torchprime/utils/kernel_utils.py:259-294,

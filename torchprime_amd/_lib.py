@@ -83,6 +83,7 @@ SIGNATURES = {
     + [c_float, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
   ),
   "tp_attn_bwd_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+  "tp_attn_bwd_dq_first": (c_int, [c_int] * 7),
   "tp_attn_bwd": (
     c_int,
     [c_void_p] * 11 + [c_int] * 7 + [_I64x3] * 8 + [c_float, c_int, c_int, c_void_p],

@@ -1443,7 +1443,26 @@ __global__ __launch_bounds__(256, DQK == DV ? 2 : 1) void attn_bwd_dq_plain_kern
   const int64_t ro = ((int64_t)b * a.Hq + h) * Sq + qrow_c;
   const float lraw = a.lse[ro];
   const float nlse = (lraw == -INFINITY) ? -INFINITY : -lraw * LOG2E;  // (a row without keys: P = exp2(-inf) = 0)
-  const float ndelta = a.delta[ro];                                     // -rowsum(dO o O)
+  // -delta = -rowsum(dO o O) of this lane's row, computed here from the dO fragments and the matching pieces of O
+  // (the two lanes that share a row hold the two halves of the head dim), and left in the workspace together with
+  // -LSE in log2 units for the dK/dV kernel, which runs after this one: no separate pass over dO and O
+  float ndelta;
+  {
+    const T* op = (const T*)a.out + b * a.os[0] + h * a.os[1] + qrow_c * a.os[2] + 8 * g;
+    float acc = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KSV; ks++) {
+      const v8 of = *(const v8*)(op + 16 * ks);
+#pragma unroll
+      for (int e = 0; e < 8; e++) acc = __builtin_fmaf((float)of[e], (float)dof[ks][e], acc);
+    }
+    acc += __shfl_xor(acc, 32, 64);
+    ndelta = -acc;
+    if (g == 0 && qrow < Sq) {
+      a.delta[ro] = ndelta;
+      a.delta[(int64_t)a.B * a.Hq * Sq + ro] = nlse;
+    }
+  }
   v8 ones_a, ndelta_b;
   {
     const float hi = (float)(T)ndelta, lo = ndelta - hi;
@@ -1757,52 +1776,45 @@ static inline void mark(void* const* events, int i, hipStream_t st) {
   if (events && events[i]) (void)hipEventRecord((hipEvent_t)events[i], st);
 }
 
+// The lean dQ kernel (attn_bwd_dq_plain_kernel) serves the plain and causal problems and segment ids with causality;
+// it computes delta itself and runs first.  Everything else (mask extensions, segment ids without causality, unequal
+// head dims without causality, a tile list too long for the LDS) takes the delta kernel and the general dQ kernel.
+template <int DQK, int DV, bool CAUSAL, bool SEG>
+struct LeanDq {
+  // (unequal head dims without causality stay with the general kernel: the compiler copies the pinned accumulators
+  // between the branches of that variant's loop, right behind the MFMAs that write them)
+  static constexpr bool BUILT = (!SEG || CAUSAL) && (DQK == DV || CAUSAL);
+  static size_t lds_bytes(int Skv) {
+    constexpr int BN = 64;
+    return 2 * (size_t)(DmaTile<DQK, true>::BYTES + DmaTile<DV, true>::BYTES) + (SEG ? 2 * BN * 4 + 16 * (size_t)((Skv + BN - 1) / BN) : 0);
+  }
+  static bool taken(int Skv) { return BUILT && lds_bytes(Skv) <= 160 * 1024; }
+};
+
 template <typename T, int DQK, int DV, bool CAUSAL, bool SEG>
 static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
+  typedef LeanDq<DQK, DV, CAUSAL, SEG> Lean;
+  const bool lean = Lean::taken(a.Skv);
+  // dK/dV: three row-major buffers of Q and dO tiles, the row vectors, the tile list (checked before anything is launched)
+  constexpr int DKDV_NBUF = 3, DKDV_BMQ = 64, DKDV_BNK = 128;
+  constexpr int DKDV_BUF = DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES;
+  static_assert(DKDV_NBUF * DKDV_BUF <= 144 * 1024, "the three buffers must leave room for the row vectors and the tile list");
+  const int nqt = (a.Sq + DKDV_BMQ - 1) / DKDV_BMQ;
+  const size_t dkdv_smem = (size_t)DKDV_NBUF * DKDV_BUF + 3 * DKDV_BMQ * 16 + (SEG ? (size_t)(6 * nqt + 8 + 4) * 4 : 0);
+  TP_REQUIRE(dkdv_smem <= 160 * 1024 && (size_t)3 * nqt * 4 <= (size_t)DKDV_NBUF * DKDV_BUF, TP_ERR_UNSUPPORTED,
+             "tp_attn_bwd: Sq=%d needs %zu bytes of LDS (max 163840)", a.Sq, dkdv_smem);
   mark(ev, 0, st);
-  // delta
-  {
+  if (!lean) {
+    // delta
     const int64_t threads = (int64_t)a.B * a.Hq * a.Sq * (DV / 8);
     attn_delta_kernel<T, DV><<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st>>>(a);
     int rc = check_launch("tp_attn_bwd(delta)");
     if (rc) return rc;
   }
   mark(ev, 1, st);
-  // dK, dV
-  {
-    constexpr int BMQ = 64, BNK = 128;
-    // three row-major buffers of Q and dO tiles
-    constexpr int NBUF = 3;
-    constexpr int BUF = DmaTile<DQK>::BYTES + DmaTile<DV>::BYTES;
-    static_assert(NBUF * BUF <= 144 * 1024, "the three buffers must leave room for the row vectors and the tile list");
-    constexpr int ROWS = 3 * BMQ * 16;
-    const int nqt = (a.Sq + BMQ - 1) / BMQ;
-    const size_t smem = (size_t)NBUF * BUF + ROWS + (SEG ? (size_t)(6 * nqt + 8 + 4) * 4 : 0);
-    TP_REQUIRE(smem <= 160 * 1024 && (size_t)3 * nqt * 4 <= (size_t)NBUF * BUF, TP_ERR_UNSUPPORTED,
-               "tp_attn_bwd: Sq=%d needs %zu bytes of LDS (max 163840)", a.Sq, smem);
-    auto kern = attn_bwd_dkdv_kernel<T, DQK, DV, NBUF, CAUSAL, SEG>;
-    static bool attr_set = false;
-    if (!attr_set) {
-      int rc = set_max_lds(kern, "tp_attn_bwd(dkdv)");
-      if (rc) return rc;
-      attr_set = true;
-    }
-    kern<<<dim3(xcd_grid((a.Skv + BNK - 1) / BNK, 1, a.B * a.Hkv)), dim3(256), smem, st>>>(a);
-    int rc = check_launch("tp_attn_bwd(dkdv)");
-    if (rc) return rc;
-  }
-  mark(ev, 2, st);
-  // dQ
-  // (segments with causality; segments alone share an instantiation with the mask extensions: the general kernel below)
-  // (unequal head dims without causality stay with the general kernel too: the compiler copies the pinned accumulators
-  // between the branches of that variant's loop, right behind the MFMAs that write them)
-  constexpr bool LEAN_DQ = (!SEG || CAUSAL) && (DQK == DV || CAUSAL);
-  constexpr int DQ_BN = 64;
-  const size_t lean_smem = 2 * (size_t)(DmaTile<DQK, true>::BYTES + DmaTile<DV, true>::BYTES) +
-                           (SEG ? 2 * DQ_BN * 4 + 16 * (size_t)((a.Skv + DQ_BN - 1) / DQ_BN) : 0);
-  bool lean_done = false;
-  if constexpr (LEAN_DQ) {
-    if (lean_smem <= 160 * 1024) {  // (the list of a very long sequence does not fit: the general kernel then)
+  if constexpr (Lean::BUILT) {
+    if (lean) {
+      // dQ first: it leaves -delta and -LSE (log2 units) of every query row in the workspace for the dK/dV kernel
       constexpr int BM = 128;
       auto kern = attn_bwd_dq_plain_kernel<T, DQK, DV, CAUSAL, SEG>;
       static bool attr_set = false;
@@ -1811,14 +1823,29 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
         if (rc) return rc;
         attr_set = true;
       }
-      kern<<<dim3(xcd_grid((a.Sq + BM - 1) / BM, a.n_rep, a.B * a.Hkv)), dim3(256), lean_smem, st>>>(a);
+      kern<<<dim3(xcd_grid((a.Sq + BM - 1) / BM, a.n_rep, a.B * a.Hkv)), dim3(256), Lean::lds_bytes(a.Skv), st>>>(a);
       int rc = check_launch("tp_attn_bwd(dq)");
       if (rc) return rc;
-      lean_done = true;
+      mark(ev, 3, st);
     }
   }
-  if constexpr (!LEAN_DQ || SEG) {
-    if (!lean_done) {
+  // dK, dV
+  {
+    auto kern = attn_bwd_dkdv_kernel<T, DQK, DV, DKDV_NBUF, CAUSAL, SEG>;
+    static bool attr_set = false;
+    if (!attr_set) {
+      int rc = set_max_lds(kern, "tp_attn_bwd(dkdv)");
+      if (rc) return rc;
+      attr_set = true;
+    }
+    kern<<<dim3(xcd_grid((a.Skv + DKDV_BNK - 1) / DKDV_BNK, 1, a.B * a.Hkv)), dim3(256), dkdv_smem, st>>>(a);
+    int rc = check_launch("tp_attn_bwd(dkdv)");
+    if (rc) return rc;
+  }
+  mark(ev, 2, st);
+  // dQ, the general kernel
+  if constexpr (!Lean::BUILT || SEG) {
+    if (!lean) {
     // eight waves (two per SIMD) where a wave's registers fit in half a SIMD's file
     // (the non-causal 128-wide variant does not fit 256 registers without spilling: it keeps four waves)
     constexpr int NW = (DQK == DV && (DQK <= 64 || (DQK <= 128 && CAUSAL))) ? 8 : 4;
@@ -1840,7 +1867,7 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
     if (rc) return rc;
     }
   }
-  mark(ev, 3, st);
+  if (!lean) mark(ev, 3, st);
   return TP_OK;
 }
 
@@ -1895,6 +1922,22 @@ int bwd_by_dims_bf16(const BwdArgs& a, int Dqk, int Dv, int causal, hipStream_t 
 
 #if !TP_BWD_F16
 using namespace tp;
+
+extern "C" int tp_attn_bwd_dq_first(int Skv, int Dqk, int Dv, int causal, int has_seg, int masked, int dtype) {
+  if (masked || (dtype != TP_BF16 && dtype != TP_F16)) return 0;
+  auto pick = [&](auto dq, auto dv) -> int {
+    constexpr int DQ = decltype(dq)::value, DVV = decltype(dv)::value;
+    if (causal) return has_seg ? LeanDq<DQ, DVV, true, true>::taken(Skv) : LeanDq<DQ, DVV, true, false>::taken(Skv);
+    return has_seg ? LeanDq<DQ, DVV, false, true>::taken(Skv) : LeanDq<DQ, DVV, false, false>::taken(Skv);
+  };
+  typedef std::integral_constant<int, 64> I64;
+  typedef std::integral_constant<int, 128> I128;
+  typedef std::integral_constant<int, 192> I192;
+  if (Dqk == 128 && Dv == 128) return pick(I128{}, I128{});
+  if (Dqk == 64 && Dv == 64) return pick(I64{}, I64{});
+  if (Dqk == 192 && Dv == 128) return pick(I192{}, I128{});
+  return 0;
+}
 
 extern "C" size_t tp_attn_bwd_workspace_bytes(int B, int Hq, int Sq) {
   if (B <= 0 || Hq <= 0 || Sq <= 0) return 0;
