@@ -740,7 +740,8 @@ def summarize_profiles(d, commit):
         traffic[k] = float(f"{(rd + wr) * (1 << 20):.3g}")
         o.append(f"| {k}_kernel | {nf[k]} | {fetch[k]:.0f} | {write[k]:.0f} | {rd:.0f} | {wr:.0f} |")
       o += ["", "Algorithmic bytes for comparison (each operand once): forward 640 MiB (q, k, v in; out, lse out), dK/dV kernel",
-            "about 770 MiB (q, dO, k, v, row vectors in; dk, dv out), dQ kernel about 900 MiB.  The dK/dV kernel's workgroups",
+            "about 770 MiB (q, dO, k, v, row vectors in; dk, dv out), dQ kernel about 1160 MiB (q, dO, out, k, v, lse in; dq and",
+            "the two row vectors for dK/dV out: it computes rowsum(dO o O) itself, there is no delta kernel).  The dK/dV kernel's workgroups",
             "(one per 128 kv rows) each stream the Q and dO rows at or below their diagonal, 32 passes over Q and dO on",
             "average; what the table shows beyond the algorithmic bytes is the part of those passes that the L2 shared by a",
             "(batch, kv head) group's workgroups did not serve.  The kernels are MFMA-issue bound, not HBM-bound: at their",
@@ -791,13 +792,13 @@ def summarize_profiles(d, commit):
                f"{100 * a['SQ_VALU_MFMA_COEXEC_CYCLES'] / simd:.1f} % | {100 * 4 * a['SQ_ACTIVE_INST_VALU'] / simd:.1f} % | "
                f"{100 * a['SQ_WAIT_INST_ANY'] / a['SQ_WAVE_CYCLES']:.1f} % | {bb['SQ_INSTS_MFMA']:.3g} | {bb['SQ_INSTS_LDS']:.3g} | {100 * conf:.1f} % | {ghz:.2f} |")
     clk = sum(clocks) / len(clocks)
-    o += ["", f"All four kernels together: MFMA pipes busy {100 * tm / tb:.1f} % of the SIMD cycles of a step.\n",
+    o += ["", f"All kernels of a step together: MFMA pipes busy {100 * tm / tb:.1f} % of the SIMD cycles.\n",
           "Cross-check.  The dK/dV kernel executes four S x S x d products per head (S, dP, dV, dK) on the causal half plus the",
           "diagonal tiles: 4 x 1.0995e12 / 32768 FLOP per v_mfma_f32_32x32x16_bf16 = 1.34e8 instructions (SQ_INSTS_MFMA counts per wave) x 32",
           f"cycles = 4.3e9 busy cycles; the counter reads {A['attn_bwd_dkdv']['SQ_VALU_MFMA_BUSY_CYCLES']:.3g}.\n",
           "What the numbers say about the headline fraction.  bench.py counts 6 product-units per step (forward 2, backward 4: the",
           "reference's MFU convention); the kernels execute 9 (forward 2, dK/dV 4, dQ 3: S and dP are recomputed in both backward",
-          f"kernels).  Algorithmic fraction of the 2.5 PFLOP/s peak = MFMA-busy fraction x 6/9 x (sustained clock / 2.4 GHz) = {tm / tb:.3f} x 0.667 x",
+          f"kernels; the dQ kernel's -delta k-steps add 4 % to its MFMA count).  Algorithmic fraction of the 2.5 PFLOP/s peak = MFMA-busy fraction x 6/9 x (sustained clock / 2.4 GHz) = {tm / tb:.3f} x 0.667 x",
           f"{clk / 2.4:.3f} = {100 * tm / tb * 0.6667 * clk / 2.4:.1f} %, against {b['pct_of_bf16_mfma_peak']} % on this run's bench line (the causal diagonal tiles are",
           f"computed whole and counted half).  With this split of the backward and this clock, MFMA pipes that never idled would give",
           f"{100 * 0.6667 * clk / 2.4:.0f} %; 40 % asks for {100 * 0.40 / 0.6667 / (clk / 2.4):.0f} % busy."]
