@@ -265,7 +265,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   // per visited tile, in visiting order: (query tile, min id, max id, index into the position ranges), 16 bytes that
   // one LDS read fetches a whole tile ahead of their use (the tile loop would otherwise start every tile by waiting
   // out a chain of dependent LDS reads: list entry -> its ranges -> which body to run)
-  int* ctl = (int*)(((size_t)(pmax + nqt) + 15) & ~(size_t)15);
+  // (its address is formed as an offset from the LDS array: rounded through an integer the pointer loses its address
+  // space, every read of an entry becomes a flat load, and waiting for a flat load waits, the vector-memory counter
+  // being in-order, for the tile loads issued before it)
+  const unsigned ctl_off = ((unsigned)((const unsigned char*)(pmax + nqt) - smem) + 15u) & ~15u;
+  int* ctl = (int*)(smem + ctl_off);
   int nact = nqt;
   int wkmin = 0, wkmax = 0;
   if (SEG) {
