@@ -177,8 +177,10 @@ int tp_attn_bwd_ex(const void* dout, const void* q, const void* k, const void* v
                    void* const* events);
 
 /* 1 when tp_attn_bwd / tp_attn_bwd_ex run the dQ kernel first for such a problem (it then computes
- * rowsum(dO o O) itself and there is no separate pass over dO and O), else 0.  `masked`: called through
- * tp_attn_bwd_masked / tp_attn_bwd_biased.  No counterpart in the reference (see tp_attn_bwd_ex). */
+ * rowsum(dO o O) itself and there is no separate pass over dO and O), else 0.  `masked`: the call uses
+ * q_positions, a soft cap or an additive mask (tp_attn_bwd_masked / tp_attn_bwd_biased; a window or a causal
+ * offset alone does not count: those run through the same kernels as plain causality).  No counterpart in
+ * the reference (see tp_attn_bwd_ex). */
 int tp_attn_bwd_dq_first(int Skv, int Dqk, int Dv, int causal, int has_seg, int masked, int dtype);
 
 /* ------------------------------------------------------------------------------------------------
@@ -192,7 +194,10 @@ int tp_attn_bwd_dq_first(int Skv, int Dqk, int Dv, int causal, int has_seg, int 
  *                   window_right (LocalMask, kernel_utils.py:266-275); < 0: unbounded on that side
  *   logits_soft_cap > 0: scores become cap * tanh(sm_scale * q.k / cap) before masking and softmax
  *                   (attn_logits_soft_cap, kernel_utils.py:292); <= 0: none
- * Tiles outside every row's band are skipped.  Rows left without any allowed key give out = 0, lse = -inf and
+ * Tiles outside every row's band are skipped.  A window and / or a causal offset without q_positions and soft
+ * cap runs through the causal kernels of tp_attn_fwd / tp_attn_bwd (their causal bound generalised to the
+ * band), the other combinations through a general instantiation that evaluates them element by element where a
+ * tile is not wholly inside the band.  Rows left without any allowed key give out = 0, lse = -inf and
  * zero gradients.  Dtypes and head dims as tp_attn_fwd.  With none of the extensions in use the calls are
  * tp_attn_fwd / tp_attn_bwd.
  * ---------------------------------------------------------------------------------------------- */

@@ -64,6 +64,9 @@ struct BwdArgs {
   int64_t qs[3], ks[3], vs[3], os[3], dos[3], dqs[3], dks[3], dvs[3];
   float scale_log2;  // sm_scale * log2(e)
   float sm_scale;
+  // the causal kernels' band: query row i sees keys i - band_lo .. i + band_hi (plain causality: no lower bound, 0).
+  // Sliding windows and causal offsets without the other mask extensions run through these kernels.
+  int band_lo, band_hi;
   MaskExt mx;
 };
 
@@ -251,8 +254,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   const int segk = has_seg ? segb[kvrow] : 0;
 
   // ---- query tiles to visit: causal => tiles that reach the first kv row; segments => id ranges overlap
-  const int nqt_all = (Sq + BMQ - 1) / BMQ;
-  const int qt_first = CAUSAL ? min(kv0 / BMQ, nqt_all) : 0;
+  // (band: row i sees keys i - band_lo .. i + band_hi, so key j is seen by rows j - band_hi .. j + band_lo)
+  const int band_lo = CAUSAL ? a.band_lo : BAND_INF, band_hi = CAUSAL ? a.band_hi : BAND_INF;
+  const int nqt_tot = (Sq + BMQ - 1) / BMQ;
+  const int nqt_all = CAUSAL ? min((kv0 + BNK - 1 + band_lo) / BMQ + 1, nqt_tot) : nqt_tot;  // one past the last tile in reach
+  const int qt_first = CAUSAL ? min(max(kv0 - band_hi, 0) / BMQ, nqt_all) : 0;
   const int nqt = nqt_all - qt_first;
   // id ranges of all query tiles and the list of those to visit: only needed until the control entries below are
   // built, so they borrow the tile buffers, which nothing has been loaded into yet
@@ -375,8 +381,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   // wave-level decisions for a query tile (uniform): skip if every query row precedes every kv row
   // (lo, hi: id range of the query tile; t: its index into the position ranges)
   auto tile_mode_of = [&](int lo, int hi, int t, int qi0) {  // 0 = nothing to compute, 1 = no masking needed, 2 = masked
-    bool skip = (CAUSAL && qi0 + BMQ - 1 < wkv0) || wkv0 >= Skv;
-    bool need_mask = (qi0 + BMQ > Sq) || (wkv0 + 32 > Skv) || (CAUSAL && qi0 < wkv0 + 31);
+    bool skip = (CAUSAL && (qi0 + BMQ - 1 + band_hi < wkv0 || qi0 - band_lo > wkv0 + 31)) || wkv0 >= Skv;
+    bool need_mask = (qi0 + BMQ > Sq) || (wkv0 + 32 > Skv) ||
+                     (CAUSAL && (qi0 + band_hi < wkv0 + 31 || qi0 + BMQ - 1 - band_lo > wkv0));
     if (SEG) {
       skip = skip || hi < wkmin || lo > wkmax;
       need_mask = need_mask || !(lo == hi && wkmin == wkmax && lo == wkmin);
@@ -560,8 +567,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
         unsigned rowbits[2] = {0u, 0u};
         const bool by_bits = MASKED && !(GEN && ext);
         if (MASKED && by_bits) {
-          const int lo_r = CAUSAL ? max(kvcol - qi0, 0) : 0;
-          const int hi_r = kvcol < Skv ? min(Sq - qi0, BMQ) : 0;
+          const int lo_r = CAUSAL ? max(kvcol - band_hi - qi0, 0) : 0;
+          int hi_r = kvcol < Skv ? min(Sq - qi0, BMQ) : 0;
+          if (CAUSAL) hi_r = min(hi_r, kvcol + band_lo - qi0 + 1);
           unsigned long long m = 0ull;
           if (hi_r > lo_r) m = (~0ull << lo_r) & (~0ull >> (64 - hi_r));
           if (SEG && has_seg) {
@@ -1430,8 +1438,10 @@ __global__ __launch_bounds__(256, DQK == DV ? 2 : 1) void attn_bwd_dq_plain_kern
   const int b = group / a.Hkv, hk = group - b * a.Hkv, h = hk * a.n_rep + inner;
   const int q0 = qt * BM, wq0 = q0 + wave * 32;
   const int Sq = a.Sq, Skv = a.Skv;
-  const int kv_end = CAUSAL ? min(Skv, q0 + BM) : Skv;
+  const int band_lo = CAUSAL ? a.band_lo : BAND_INF, band_hi = CAUSAL ? a.band_hi : BAND_INF;
+  const int kv_end = CAUSAL ? max(min(Skv, q0 + BM + band_hi), 0) : Skv;
   const int ntiles = (kv_end + BN - 1) / BN;
+  const int t_first = CAUSAL ? min(max(q0 - band_lo, 0) / BN, ntiles) : 0;  // (tiles before it lie left of every row's band)
 
   // ---- Q, dO fragments (B operands: lane = query column), per-lane LSE / -delta
   const int qrow = wq0 + ln, qrow_c = min(qrow, Sq - 1);
@@ -1483,7 +1493,7 @@ __global__ __launch_bounds__(256, DQK == DV ? 2 : 1) void attn_bwd_dq_plain_kern
   const int32_t* segb = SEG ? a.seg + (int64_t)b * Skv : nullptr;
   const int segq = SEG ? segb[qrow_c] : 0;
   const int* ctl = (const int*)(smem + CTL_AT);
-  int nact = ntiles, wqmin = 0, wqmax = 0;
+  int nact = ntiles - t_first, wqmin = 0, wqmax = 0;
   if (SEG) {
     wqmin = segq; wqmax = segq;
 #pragma unroll
@@ -1505,7 +1515,7 @@ __global__ __launch_bounds__(256, DQK == DV ? 2 : 1) void attn_bwd_dq_plain_kern
     for (int base = 0; base < ntiles; base += 64) {
       const int t = base + lane;
       const int lo = t < ntiles ? kvmin[t] : 0, hi = t < ntiles ? kvmax[t] : 0;
-      const bool act = t < ntiles && !(hi < bmin || lo > bmax);
+      const bool act = t >= t_first && t < ntiles && !(hi < bmin || lo > bmax);
       const unsigned long long m = __ballot(act);
       if (act && wave == 0) *(i32x4*)(smem + CTL_AT + 16 * (cnt + __popcll(m & ((1ull << lane) - 1ull)))) = i32x4{t, lo, hi, 0};
       cnt += __popcll(m);
@@ -1515,7 +1525,7 @@ __global__ __launch_bounds__(256, DQK == DV ? 2 : 1) void attn_bwd_dq_plain_kern
   }
   auto entry = [&](int it) -> i32x4 {
     if (SEG) return *(const i32x4*)(ctl + 4 * max(min(it, nact - 1), 0));
-    return i32x4{min(it, ntiles - 1), 0, 0, 0};
+    return i32x4{min(t_first + it, ntiles - 1), 0, 0, 0};
   };
 
   // ---- loads
@@ -1590,10 +1600,13 @@ __global__ __launch_bounds__(256, DQK == DV ? 2 : 1) void attn_bwd_dq_plain_kern
     // 8 (v / 4) + v % 4 after the shift by 4 g)
     unsigned kbits[2] = {0u, 0u};
     if (MASKED) {
-      int hi = min(Skv - kv0, BN);
-      if (CAUSAL) hi = min(hi, qrow - kv0 + 1);
+      int hi = min(Skv - kv0, BN), lo = 0;
+      if (CAUSAL) {
+        hi = min(hi, qrow + band_hi - kv0 + 1);
+        lo = max(qrow - band_lo - kv0, 0);
+      }
       if (qrow >= Sq) hi = 0;
-      unsigned long long m = hi > 0 ? (~0ull >> (64 - hi)) : 0ull;
+      unsigned long long m = hi > lo ? ((~0ull << lo) & (~0ull >> (64 - hi))) : 0ull;
       if (SEG) {
         const int rowseg = ((const int*)(smem + SEG_AT + buf * BN * 4))[lane];  // lane l: id of the tile's kv row l
         unsigned long long ms = 0ull, todo = ~0ull;
@@ -1719,8 +1732,9 @@ __global__ __launch_bounds__(256, DQK == DV ? 2 : 1) void attn_bwd_dq_plain_kern
     const int t = cur[0], t_next = nxt[0];
     const i32x4 after = entry(it + 2);
     const int kv0 = t * BN;
-    bool skip = CAUSAL && kv0 > wq_last;
-    bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0) || (wq0 + 32 > Sq);
+    bool skip = CAUSAL && (kv0 > wq_last + band_hi || kv0 + BN - 1 < wq0 - band_lo);
+    bool need_mask = (kv0 + BN > Skv) || (wq0 + 32 > Sq) ||
+                     (CAUSAL && (kv0 + BN - 1 > wq0 + band_hi || kv0 < wq_last - band_lo));
     if (SEG) {
       skip = skip || cur[2] < wqmin || cur[1] > wqmax;
       need_mask = need_mask || !(cur[1] == cur[2] && wqmin == wqmax && cur[1] == wqmin);
@@ -1878,7 +1892,18 @@ static int launch_bwd(const BwdArgs& a, hipStream_t st, void* const* ev) {
 template <typename T, int DQK, int DV>
 static int dispatch_bwd(const BwdArgs& a, int causal, hipStream_t st, void* const* ev) {
   if (a.mx.on) {
-    // mask extensions: the general instantiation (causality is part of the band then)
+    // a window and / or a causal offset and nothing else: the causal kernels, with that band instead of (-inf, 0]
+    // (where the lean dQ kernel serves the problem; the general dQ kernel knows plain causality only)
+    const bool lean = a.seg ? LeanDq<DQK, DV, true, true>::taken(a.Skv) : LeanDq<DQK, DV, true, false>::taken(a.Skv);
+    if (band_only(a.mx) && lean) {
+      BwdArgs b = a;
+      b.band_lo = a.mx.lo_off;
+      b.band_hi = a.mx.hi_off;
+      b.mx = no_mask_ext();
+      if (a.seg) return launch_bwd<T, DQK, DV, true, true>(b, st, ev);
+      return launch_bwd<T, DQK, DV, true, false>(b, st, ev);
+    }
+    // the other mask extensions: the general instantiation (causality is part of the band then)
     return launch_bwd<T, DQK, DV, false, true>(a, st, ev);
   }
   if (causal) {
@@ -2005,6 +2030,8 @@ static int attn_bwd_impl(const void* dout, const void* q, const void* k, const v
   a.scale_log2 = sm_scale * LOG2E;
   a.sm_scale = sm_scale;
   a.mx = mx;
+  a.band_lo = BAND_INF;  // plain causality (used by the causal kernels only)
+  a.band_hi = 0;
   hipStream_t st = (hipStream_t)stream;
   const int rc = dtype == TP_BF16 ? bwd_by_dims_bf16(a, Dqk, Dv, causal, st, events) : bwd_by_dims_f16(a, Dqk, Dv, causal, st, events);
   TP_REQUIRE(rc != TP_DIMS_NOT_BUILT, TP_ERR_UNSUPPORTED, "tp_attn_bwd: head dims (qk=%d, v=%d) not built", Dqk, Dv);

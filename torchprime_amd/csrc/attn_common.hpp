@@ -157,6 +157,9 @@ inline MaskExt make_mask_ext(const int32_t* q_positions, int causal, int causal_
           bias != nullptr) ? 1 : 0;
   return m;
 }
+// a band of key positions around the row's own index and nothing else (no per-row positions, soft cap or additive
+// mask): the causal kernels evaluate it themselves
+inline bool band_only(const MaskExt& m) { return m.on && !m.qpos && m.cap_in == 0.f && !m.bias; }
 inline MaskExt no_mask_ext() {
   MaskExt m;
   m.qpos = nullptr; m.lo_off = BAND_INF; m.hi_off = BAND_INF; m.cap_in = 0.f; m.cap_out = 0.f; m.on = 0;

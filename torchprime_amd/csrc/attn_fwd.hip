@@ -32,6 +32,9 @@ struct FwdArgs {
   int B, Hq, Hkv, Sq, Skv, n_rep;
   int64_t qs[3], ks[3], vs[3], os[3];
   float scale_log2;  // sm_scale * log2(e)
+  // the causal kernels' band: query row i sees keys i - band_lo .. i + band_hi (plain causality: no lower bound, 0).
+  // Sliding windows and causal offsets without the other mask extensions run through these kernels.
+  int band_lo, band_hi;
   MaskExt mx;
 };
 
@@ -91,8 +94,10 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   const bool biased = GEN && a.mx.bias != nullptr;
   const int32_t* segb = has_seg ? a.seg + (int64_t)b * Skv : nullptr;
 
-  const int kv_end = CAUSAL ? min(Skv, q0 + BM) : Skv;
+  const int band_lo = CAUSAL ? a.band_lo : BAND_INF, band_hi = CAUSAL ? a.band_hi : BAND_INF;
+  const int kv_end = CAUSAL ? max(min(Skv, q0 + BM + band_hi), 0) : Skv;
   const int ntiles = (kv_end + BN - 1) / BN;
+  const int t_first = CAUSAL ? min(max(q0 - band_lo, 0) / BN, ntiles) : 0;  // (tiles before it lie left of every row's band)
 
   // ---- Q fragments (B operand of S^T = K Q^T): lane = query column, 8 head-dim values per k-step
   v8 qf[KSTEPS];
@@ -130,7 +135,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   int* kvmax = kvmin + ntiles;
   int* bq = kvmax + ntiles;  // 16 ints: per-wave (min,max) of the query rows' ids, then of their positions
   const int* ctl = (const int*)(smem + 2 * BUF_BYTES);
-  int nact = ntiles;
+  int nact = ntiles - t_first;
   int wqmin = 0, wqmax = 0;
   if (SEG) {
     wqmin = segq; wqmax = segq;
@@ -152,7 +157,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
     const int bqmin = min(min(bq[0], bq[2]), min(bq[4], bq[6]));
     const int bqmax = max(max(bq[1], bq[3]), max(bq[5], bq[7]));
     // keys any row of the workgroup may see
-    const int b_lo = ext ? min(min(bq[8], bq[10]), min(bq[12], bq[14])) - a.mx.lo_off : -BAND_INF;
+    const int b_lo = ext ? min(min(bq[8], bq[10]), min(bq[12], bq[14])) - a.mx.lo_off : t_first * BN;
     const int b_hi = ext ? max(max(bq[9], bq[11]), max(bq[13], bq[15])) + a.mx.hi_off : BAND_INF;
     // every wave builds the same list redundantly (no second barrier needed for the count)
     int cnt = 0;
@@ -170,7 +175,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
   }
   // list entry i as scalars (a tile offset in vector registers would put every load into a loop over its values)
   auto entry = [&](int i) -> i32x4 {
-    i32x4 e = i32x4{min(i, ntiles - 1), 0, 0, 0};
+    i32x4 e = i32x4{min(t_first + i, ntiles - 1), 0, 0, 0};
     if (SEG) e = *(const i32x4*)(ctl + 4 * max(min(i, nact - 1), 0));
     return e;
   };
@@ -306,7 +311,10 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
     unsigned kbits[2] = {0u, 0u};
     if (MASKED) {
       int lo = 0, hi = min(Skv - kv0, BN);
-      if (CAUSAL) hi = min(hi, qrow - kv0 + 1);
+      if (CAUSAL) {
+        hi = min(hi, qrow + band_hi - kv0 + 1);
+        lo = max(qrow - band_lo - kv0, 0);
+      }
       if (GEN) {
         lo = max(lo_q - kv0, 0);
         hi = min(hi, hi_q - kv0 + 1);
@@ -459,8 +467,8 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
     const int kv0 = t * BN;
     const bool has_next = it + 1 < nact;
     const int t_next = has_next ? nxt[0] : t;
-    bool skip = CAUSAL && kv0 > wq_last;
-    bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0);
+    bool skip = CAUSAL && (kv0 > wq_last + band_hi || kv0 + BN - 1 < wq0 - band_lo);
+    bool need_mask = (kv0 + BN > Skv) || (CAUSAL && (kv0 + BN - 1 > wq0 + band_hi || kv0 < wq_last - band_lo));
     if (SEG) {
       const int lo = cur[1], hi = cur[2];
       skip = skip || hi < wqmin || lo > wqmax;
@@ -498,8 +506,8 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
       const int kv0 = t * BN;
       const bool has_next = it + 1 < nact;
       const int t_next = has_next ? nxt[0] : t;
-      bool skip = CAUSAL && kv0 > wq_last;
-      bool need_mask = (kv0 + BN > Skv) || (CAUSAL && kv0 + BN - 1 > wq0);
+      bool skip = CAUSAL && (kv0 > wq_last + band_hi || kv0 + BN - 1 < wq0 - band_lo);
+      bool need_mask = (kv0 + BN > Skv) || (CAUSAL && (kv0 + BN - 1 > wq0 + band_hi || kv0 < wq_last - band_lo));
       if (SEG) {
         const int lo = cur[1], hi = cur[2];
         skip = skip || hi < wqmin || lo > wqmax;
@@ -576,7 +584,16 @@ static int launch_fwd(const FwdArgs& a, int B, hipStream_t st) {
 template <typename T, int DQK, int DV>
 static int dispatch_fwd(const FwdArgs& a, int B, int causal, hipStream_t st) {
   if (a.mx.on) {
-    // mask extensions: the general instantiation (causality is part of the band then)
+    if (band_only(a.mx)) {
+      // a window and / or a causal offset and nothing else: the causal kernels, with that band instead of (-inf, 0]
+      FwdArgs b = a;
+      b.band_lo = a.mx.lo_off;
+      b.band_hi = a.mx.hi_off;
+      b.mx = no_mask_ext();
+      if (a.seg) return launch_fwd<T, DQK, DV, true, true>(b, B, st);
+      return launch_fwd<T, DQK, DV, true, false>(b, B, st);
+    }
+    // the other mask extensions: the general instantiation (causality is part of the band then)
     return launch_fwd<T, DQK, DV, false, true>(a, B, st);
   }
   if (causal) {
@@ -626,6 +643,8 @@ static int attn_fwd_impl(const void* q, const void* k, const void* v, const int3
              TP_ERR_UNSUPPORTED, "tp_attn_fwd: one (batch, head) slice of k or v spans 2 GiB or more");
   a.scale_log2 = sm_scale * LOG2E;
   a.mx = mx;
+  a.band_lo = BAND_INF;  // plain causality (used by the causal kernels only)
+  a.band_hi = 0;
   hipStream_t st = (hipStream_t)stream;
 #define TP_FWD(T, DQ, DVV) return dispatch_fwd<T, DQ, DVV>(a, B, causal, st)
   if (dtype == TP_BF16) {
