@@ -7,7 +7,8 @@
 // and dK, dV summed over the n_rep query heads that share a KV head.
 //
 // Kernels:
-//   attn_delta_kernel     -delta[b,h,i] = -sum_d dO*O, and the LSE in log2 units      (HBM-bound)
+//   attn_delta_kernel     -delta[b,h,i] = -sum_d dO*O, and the LSE in log2 units      (HBM-bound; only where the
+//                         general dQ kernel runs: the lean dQ kernel computes both itself and runs first)
 //   attn_bwd_dkdv_kernel  one workgroup = 128 KV rows of one (batch, kv head); K and V fragments stay
 //                         in registers, row-major Q / dO tiles of every query head of the group stream through
 //                         three LDS buffers (fragment reads for S = QK^T and dP = dO V^T, transposing reads
@@ -331,7 +332,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
   dodma.init(a.dos[2], wave, lane);
   const unsigned q_span = span_bytes(Sq, a.qs[2], DQK), do_span = span_bytes(Sq, a.dos[2], DV);
   const unsigned q_tile_bytes = (unsigned)(BMQ * a.qs[2] * 2), do_tile_bytes = (unsigned)(BMQ * a.dos[2] * 2);
-  const float* lse2 = a.delta + (int64_t)a.B * a.Hq * Sq;  // second half of the workspace (delta kernel)
+  const float* lse2 = a.delta + (int64_t)a.B * a.Hq * Sq;  // second half of the workspace (written by the kernel before this one)
   unsigned char* const rows_base = smem + NBUF * BUF_BYTES;
   // Query tiles are visited from the last one down.  The workgroups of a (batch, kv head) run side by side on one XCD
   // and all stream the same Q / dO tiles; each needs the tiles from its own kv rows on, so counting up they would start
