@@ -198,6 +198,42 @@ def test_full_size_sliding_window_slice():
   assert_close(vd.grad[b : b + 1, g : g + 1], dv_ref, "dv", scale_abs=True)
 
 
+def _random_band_case(seed):
+  """A random window / causal offset problem: sizes around the tile edges (32, 64, 128 rows), every head-dim pair, GQA
+  group sizes 1..4, ragged key lengths, segment ids now and then, windows from zero to beyond the sequence."""
+  g = torch.Generator().manual_seed(9000 + seed)
+  r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))  # noqa: E731
+  D, Dv = ((64, 64), (128, 128), (192, 128))[r(0, 2)]
+  Hkv = r(1, 2)
+  Hq = Hkv * r(1, 4)
+  S = (r(1, 70), r(100, 200), r(250, 420))[r(0, 2)]
+  use_seg = r(0, 3) == 0
+  # (a handful of keys under hundreds of queries would put a thousand rounded dS terms into every dK element: that is
+  # a question for the tolerance, not for the band arithmetic this test is about)
+  Skv = S if use_seg or r(0, 2) else max(r(1, 450), S // 6)
+  causal = bool(r(0, 2))
+  left = None if r(0, 3) == 0 else r(0, (5, 40, 150, 500)[r(0, 3)])
+  right = None if (causal and r(0, 1)) or r(0, 3) == 0 else r(0, (3, 30, 200)[r(0, 2)])
+  if left is None and right is None and not causal:
+    left = r(0, 60)
+  offset = r(-6, 50) if causal and r(0, 1) else 0
+  seg = packed_segment_ids(1 + r(0, 1), S, 1, max(2, S // 2), seed)[0] if use_seg else None
+  B = seg.shape[0] if use_seg else r(1, 2)
+  dtype = (torch.bfloat16, torch.float16)[r(0, 1)]
+  return dict(B=B, Hq=Hq, Hkv=Hkv, S=S, D=D, Dv=Dv, Skv=Skv, causal=causal, window=(left, right), causal_offset=offset,
+              seg=seg, dtype=dtype)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_randomised_windows_and_offsets(seed):
+  """The causal kernels evaluate a window and / or a causal offset as a band around the row's own index (first and
+  last tile of a workgroup's loop, per-wave skips, which tiles need masks, the bit range of a masked tile): 48 random
+  problems against the oracle, forward and gradients, rows without any allowed key included."""
+  c = _random_band_case(seed)
+  _check(c["B"], c["Hq"], c["Hkv"], c["S"], c["D"], dtype=c["dtype"], causal=c["causal"], seg=c["seg"], window=c["window"],
+         causal_offset=c["causal_offset"], Skv=c["Skv"], seed=seed, Dv=c["Dv"])
+
+
 # ---- additive masks: the eager branch's ``attn_weights + causal_mask`` (attention.py:151-158) for any mask ----------
 def _eager_grads(q, k, v, do, mask):
   """(out, dq, dk, dv) of the oracle's eager attention in float64, by autograd."""
