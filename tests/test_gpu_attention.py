@@ -493,3 +493,44 @@ def test_deepseek_v3_shape_slice():  # benchmark configuration 4: B=1, S=4096, 1
 def test_deepseek_v3_shape_slice_qk_scale():
   # the same configuration with the scale a 192-wide q.k product would usually take (the reference uses the v head dim)
   _slice_check(1, 128, 128, 4096, 192, 128, None, 1234 + 4, b_sel=0, g_sel=3, sm_scale=192 ** -0.5)
+
+
+def _closed_form_check(B, Hq, Hkv, S, Dqk, Dv, seg, seed):
+  """What the mathematics fixes on the WHOLE full-size problem, every (batch, head), no oracle needed.  With V constant
+  along the sequence (one value per (batch, kv head, column)) every output row is that value whatever the scores are,
+  dP = dO V^T is constant along a row, so dS = P o (dP - rowsum(P o dP)) = 0 and with it dQ = dK = 0; and because the
+  rows of P sum to one, the sum of dV over the keys equals the sum of dO over the queries of the group's heads.  A wrong
+  LSE, a wrong delta, a mask that empties a row or a tile visited twice or not at all breaks one of the three."""
+  n_rep = Hq // Hkv
+  dt = torch.bfloat16
+  g = torch.Generator().manual_seed(seed)
+  q, k, do = (heads_view(B, h, S, d, seed + i, dt) for i, (h, d) in enumerate(((Hq, Dqk), (Hkv, Dqk), (Hq, Dv))))
+  vals = torch.randn((B, Hkv, 1, Dv), generator=g).to(dt)
+  v = vals.expand(B, Hkv, S, Dv).transpose(1, 2).contiguous().transpose(1, 2)  # (B,H,S,D) view of a (B,S,H,D) buffer
+  out, lse, dq, dk, dv = _run(q, k, v, do, seg, True, 1.0 / math.sqrt(Dv))
+  expect = vals.to(DEV).float().repeat_interleave(n_rep, dim=1)  # (B, Hq, 1, Dv)
+  assert (out.float() - expect).abs().max().item() <= 2.0**-7 * vals.abs().max().item() + 1e-3  # P is rounded to 16 bit for PV
+  # dQ and dK against the size of one of their terms, |dO| |V| |K|: with a random V of the same size the same kernels
+  # give |dQ|, |dK| of 0.03-0.08 on average and 4-7 at most, so a delta or LSE off by one percent would show up as
+  # 0.04-0.07 here; what the cancellation leaves in 16-bit arithmetic is 3e-5 (plain) to 7e-3 (packed documents)
+  scale = do.float().abs().mean().item() * vals.float().abs().mean().item() * k.float().abs().mean().item()
+  assert dq.float().abs().max().item() <= 0.05 * scale, (dq.float().abs().max().item(), scale)
+  assert dk.float().abs().max().item() <= 0.05 * scale, (dk.float().abs().max().item(), scale)
+  dv_sum = dv.double().sum(dim=2)  # (B, Hkv, Dv)
+  do_sum = do.to(DEV).double().sum(dim=2).view(B, Hkv, n_rep, Dv).sum(dim=2)
+  rel = (dv_sum - do_sum).abs().max().item() / do_sum.abs().max().item()
+  assert rel <= 2e-3, rel
+  assert torch.isfinite(lse).all()
+
+
+def test_llama3_8b_shape_closed_forms():
+  _closed_form_check(4, 32, 8, 8192, 128, 128, None, 4321)
+
+
+def test_llama3_8b_packed_segments_closed_forms():
+  seg, _ = packed_segment_ids(4, 8192, 64, 4096, seed=1234 + 2)
+  _closed_form_check(4, 32, 8, 8192, 128, 128, seg, 4322)
+
+
+def test_deepseek_v3_shape_closed_forms():
+  _closed_form_check(1, 128, 128, 4096, 192, 128, None, 4323)
