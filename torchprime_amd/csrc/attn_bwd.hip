@@ -1446,6 +1446,7 @@ __global__ __launch_bounds__(256, DQK == DV ? 2 : 1) void attn_bwd_dq_plain_kern
 
   // ---- Q, dO fragments (B operands: lane = query column), per-lane LSE / -delta
   const int qrow = wq0 + ln, qrow_c = min(qrow, Sq - 1);
+  const int wq0_s = __builtin_amdgcn_readfirstlane(wq0);  // (for the masked tiles, which form the row again)
   v8 qf[KS], dof[KSV];
   {
     const T* qp = (const T*)a.q + b * a.qs[0] + h * a.qs[1] + qrow_c * a.qs[2] + 8 * g;
@@ -1601,15 +1602,24 @@ __global__ __launch_bounds__(256, DQK == DV ? 2 : 1) void attn_bwd_dq_plain_kern
     // 8 (v / 4) + v % 4 after the shift by 4 g)
     unsigned kbits[2] = {0u, 0u};
     if (MASKED) {
+      // (what only a masked tile needs is formed here from an opaque copy of lane * 4, which the loads of the
+      // segment ids keep in a register anyway: the query row, the band offsets added to it and the address of the
+      // lane's segment id, held across the loop as registers of their own, were spilled in the variant with
+      // segment ids, and a reload waits behind the tile loads in flight)
+      unsigned l4 = (unsigned)lane * 4u;
+      asm volatile("" : "+v"(l4));
+      const int qrow_m = wq0_s + (int)((l4 >> 2) & 31u);
       int hi = min(Skv - kv0, BN), lo = 0;
       if (CAUSAL) {
-        hi = min(hi, qrow + band_hi - kv0 + 1);
-        lo = max(qrow - band_lo - kv0, 0);
+        int bh = band_hi - kv0 + 1, bl = band_lo + kv0;
+        asm volatile("" : "+s"(bh), "+s"(bl));
+        hi = min(hi, qrow_m + bh);
+        lo = max(qrow_m - bl, 0);
       }
-      if (qrow >= Sq) hi = 0;
+      if (qrow_m >= Sq) hi = 0;
       unsigned long long m = hi > lo ? ((~0ull << lo) & (~0ull >> (64 - hi))) : 0ull;
       if (SEG) {
-        const int rowseg = ((const int*)(smem + SEG_AT + buf * BN * 4))[lane];  // lane l: id of the tile's kv row l
+        const int rowseg = *(const int*)(smem + SEG_AT + buf * BN * 4 + l4);  // lane l: id of the tile's kv row l
         unsigned long long ms = 0ull, todo = ~0ull;
         while (todo) {
           const int x = __builtin_amdgcn_readlane(segq, (int)__builtin_ctzll(todo));
