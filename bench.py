@@ -550,6 +550,128 @@ def bench_decoder_layer(dev, iters=5):
           "layer_TFLOPs": round((gemm_flops + attn_flops) / (ms * 1e-3) / 1e12, 1)}  # fmt: skip
 
 
+class ClockSampler:
+  """Reads the shader clock every 50 ms on a thread while a region runs: the starred line of the first
+  /sys/class/drm/card*/device/pp_dpm_sclk that has one (no child process, so it is safe under a profiler); where that
+  file is missing or unreadable, `rocm-smi --showclocks` as a child process."""
+
+  def __init__(self):
+    import glob
+
+    self.path = None
+    for p in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")):
+      if self._sysfs(p) is not None:
+        self.path = p
+        break
+    self.samples = []
+    self._stop = False
+    self._thread = None
+
+  @staticmethod
+  def _sysfs(path):
+    import re
+
+    try:
+      with open(path) as f:
+        for line in f:
+          if "*" in line:
+            m = re.search(r"(\d+)\s*Mhz", line, re.IGNORECASE)
+            return int(m.group(1)) if m else None
+    except OSError:
+      pass
+    return None
+
+  @staticmethod
+  def _smi():
+    import re
+    import subprocess
+
+    try:
+      out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=10).stdout
+    except (OSError, subprocess.SubprocessError):
+      return None
+    m = re.search(r"sclk clock level: \S+ \((\d+)Mhz\)", out)
+    return int(m.group(1)) if m else None
+
+  def _run(self):
+    while not self._stop:
+      v = self._sysfs(self.path) if self.path else self._smi()
+      if v is not None:
+        self.samples.append((time.time(), v))
+      time.sleep(0.05)
+
+  def start(self):
+    import threading
+
+    self._thread = threading.Thread(target=self._run, daemon=True)
+    self._thread.start()
+
+  def stop(self):
+    self._stop = True
+    if self._thread is not None:
+      self._thread.join(timeout=15)
+
+  def mean_mhz(self, t0, t1):
+    xs = [v for (t, v) in self.samples if t0 <= t <= t1]
+    return round(sum(xs) / len(xs)) if xs else None
+
+
+def bench_clock_probe(dev, seconds=2.5):
+  """What the part sustains under load, and how much of that is the data: the headline attention step and one
+  hipBLASLt GEMM (torch.matmul, 8192^3 bf16), each run back to back for `seconds` on normal-distributed inputs (the
+  benchmark's data) and on zeros, with the shader clock sampled meanwhile.  The quoted MFMA peak assumes 2.4 GHz; with
+  operands that toggle the matrix pipes' inputs the part lowers its clock to hold its power limit, with zeros it does
+  not.  A diagnostic: the zero-input rates are no benchmark figures."""
+  import torch
+
+  B, Hq, Hkv, S, D = 4, 32, 8, 8192, 128
+  sampler = ClockSampler()
+  sampler.start()
+  res = {"clock_source": sampler.path or "rocm-smi --showclocks"}
+
+  def sustained(fn):
+    for _ in range(3):
+      fn(0)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    n = 0
+    t0 = time.time()
+    e0.record()
+    while time.time() - t0 < seconds:
+      for _ in range(5):
+        fn(0)
+      n += 5
+      torch.cuda.synchronize()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.time()
+    return e0.elapsed_time(e1) / n, sampler.mean_mhz(t0 + 0.5, t1)
+
+  try:
+    for kind in ("normal", "zeros"):
+      n = 8192
+      a = torch.randn((n, n), dtype=torch.bfloat16, device=dev) if kind == "normal" else torch.zeros((n, n), dtype=torch.bfloat16, device=dev)
+      b = a.clone()
+      c = torch.empty_like(a)
+      ms, mhz = sustained(lambda i: torch.matmul(a, b, out=c))
+      res[f"gemm_8192_{kind}"] = {"ms": round(ms, 4), "TFLOPs": round(2.0 * n**3 / (ms * 1e-3) / 1e12, 1), "sclk_mhz": mhz}
+      del a, b, c
+      q, k, v, do = make_inputs(B, Hq, Hkv, S, D, dev)
+      if kind == "zeros":
+        q, k, v, do = (torch.zeros_like(t.transpose(1, 2)).transpose(1, 2) for t in (q, k, v, do))
+      step, _bufs = attention_step_fn(q, k, v, do, 1.0 / math.sqrt(D))
+      ms, mhz = sustained(step)
+      res[f"attn_step_{kind}"] = {
+        "ms": round(ms, 4), "algorithmic_TFLOPs": round(6.0 * B * Hq * S * S * D / (ms * 1e-3) / 1e12, 1),
+        "executed_TFLOPs": round(9.0 * B * Hq * S * S * D / (ms * 1e-3) / 1e12, 1), "sclk_mhz": mhz,
+      }  # fmt: skip
+      del q, k, v, do, step, _bufs
+      torch.cuda.empty_cache()
+  finally:
+    sampler.stop()
+  return res
+
+
 def cpu_baseline(max_seconds=24.0):
   """The oracle's eager attention (attention.py:151-170 restated), fwd + bwd by autograd, bf16 inputs, on
   this host's cores: one batch element and one kv-head group (4 q heads) of the benchmark workload."""
@@ -854,6 +976,9 @@ def main():
                   help="run only one Llama-3-8B decoder layer forward + backward (GEMMs included) and print its line")
   ap.add_argument("--tiny-config", action="store_true",
                   help="run only the tiny fp32 configuration's launch-by-launch / HIP graph comparison and print its line")
+  ap.add_argument("--clock-probe", action="store_true",
+                  help="run only the sustained-clock diagnostic (attention step and a hipBLASLt GEMM on normal and on zero inputs, "
+                       "shader clock sampled meanwhile) and print its line")
   ap.add_argument("--summarize", default=None, metavar="DIR",
                   help="no GPU work: turn the rocprofv3 output under DIR (see _PROFILE_COMMANDS) into the summaries under profiles/")
   ap.add_argument("--commit", default=None, help="with --summarize: the commit the profiled tree was at (default: git rev-parse)")
@@ -892,12 +1017,16 @@ def main():
   if args.tiny_config:
     print(json.dumps({"tiny_fp32_config_hip_graph": bench_tiny_config_graph(dev, iters=args.steps)}))
     return
+  if args.clock_probe:
+    print(json.dumps({"clock_probe": bench_clock_probe(dev)}))
+    return
   ms_per_step, flops_step, roofline, kernels, shape = bench_attention(args, dev)
   extra = None if args.no_extra else bench_norm_rope(dev)
   if extra is not None:
     extra["other_configs"] = bench_other_configs(dev)
     extra["tiny_fp32_config_hip_graph"] = bench_tiny_config_graph(dev)
     extra["llama3_8b_decoder_layer"] = bench_decoder_layer(dev, iters=3)
+    extra["clock_probe"] = bench_clock_probe(dev, seconds=2.0)
     torch.cuda.empty_cache()
   torch.cuda.empty_cache()
   cpu = None if args.no_cpu else cpu_baseline()
