@@ -178,6 +178,40 @@ __global__ __launch_bounds__(512) void two(float* out, int iters, long long* cyc
   if (blockIdx.x == 0 && l == 0) cyc[w] = t1 - t0;
 }
 
+// ---- (4) where the accumulators live: NW waves per SIMD, per MFMA NV independent FMAs; the MFMA is an asm statement
+// whose accumulator is pinned to the architectural registers (ACC 0) or to the accumulation registers (ACC 1);
+// CHAIN accumulators in rotation (1: every MFMA depends on the one before, as the k-steps of one product do)
+template <int ACC, int CHAIN, int NV, int THREADS>
+__global__ __launch_bounds__(THREADS) void acc_kind(float* out, int iters, long long* cyc) {
+  const int t = threadIdx.x, l = t & 63;
+  bf16x8 a, b;
+  for (int e = 0; e < 8; e++) { a[e] = (__bf16)(1.0f + l * 0.001f); b[e] = (__bf16)1.0f; }
+  f32x16 c[4];
+  for (int i = 0; i < 4; i++) for (int v = 0; v < 16; v++) c[i][v] = 0.f;
+  float x[8];
+  for (int i = 0; i < 8; i++) x[i] = l * 0.001f + i;
+  if (ACC) { asm volatile("" : "+a"(c[0]), "+a"(c[1]), "+a"(c[2]), "+a"(c[3])); }
+  long long t0 = __builtin_readcyclecounter();
+  for (int i = 0; i < iters; i++) {
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+      if (ACC) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c[j % CHAIN]) : "v"(a), "v"(b));
+      else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c[j % CHAIN]) : "v"(a), "v"(b));
+#pragma unroll
+      for (int k = 0; k < NV; k++) x[(j + k) % 8] = x[(j + k) % 8] * 0.999f + 0.5f;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  long long t1 = __builtin_readcyclecounter();
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");  // past the last MFMA's latency before ordinary instructions read c
+  if (ACC) { asm volatile("" : "+a"(c[0]), "+a"(c[1]), "+a"(c[2]), "+a"(c[3])); }
+  float s = 0;
+  for (int i = 0; i < 4; i++) s += c[i][0];
+  for (int i = 0; i < 8; i++) s += x[i];
+  out[blockIdx.x * THREADS + t] = s;
+  if (blockIdx.x == 0 && t == 0) cyc[0] = t1 - t0;
+}
+
 int main() {
   hipDeviceProp_t p; CK(hipGetDeviceProperties(&p, 0));
   const int ncu = p.multiProcessorCount;
@@ -211,6 +245,16 @@ int main() {
     TWO(0, 32, 5, 1) TWO(1, 32, 5, 1) TWO(2, 32, 5, 1) TWO(4, 32, 5, 1) TWO(5, 32, 5, 1)
     TWO(0, 16, 5, 1) TWO(2, 16, 5, 1) TWO(5, 16, 5, 1)
     TWO(0, 32, 2, 1) TWO(2, 32, 2, 1)
+  }
+  {
+    const int it = 2000;
+#define ACCK(A, CH, NV, TH) { float ms = timeit([&] { acc_kind<A, CH, NV, TH><<<ncu, TH>>>(out, it, cyc); }); CK(hipMemcpy(h, cyc, 8, hipMemcpyDeviceToHost)); \
+    printf("%d wave(s)/SIMD, accumulators in %s, %d in rotation, valu/mfma=%d: %.3f ms for %d MFMAs per wave\n", TH / 256, A ? "AGPRs" : "VGPRs", CH, NV, ms, it * 16); fflush(stdout); }
+    ACCK(0, 4, 0, 256) ACCK(1, 4, 0, 256) ACCK(0, 1, 0, 256) ACCK(1, 1, 0, 256)
+    ACCK(0, 4, 4, 256) ACCK(1, 4, 4, 256) ACCK(0, 4, 8, 256) ACCK(1, 4, 8, 256) ACCK(0, 1, 8, 256) ACCK(1, 1, 8, 256)
+    ACCK(0, 4, 0, 512) ACCK(1, 4, 0, 512)
+    ACCK(0, 4, 4, 512) ACCK(1, 4, 4, 512) ACCK(0, 4, 6, 512) ACCK(1, 4, 6, 512) ACCK(0, 4, 8, 512) ACCK(1, 4, 8, 512)
+    ACCK(0, 1, 6, 512) ACCK(1, 1, 6, 512)
   }
   printf("done\n");
   return 0;
