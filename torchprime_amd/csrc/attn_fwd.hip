@@ -382,7 +382,8 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
       }
     };
     // exponentials of half HF: its 16 values spread over the LEN slots from START on (plain adds for the row
-    // sum: v_dot2 shares the matrix pipe and would serialise with the MFMAs)
+    // sum: v_dot2 shares the matrix pipe and would serialise with the MFMAs).  A slot's values join the row sum and
+    // the 16-bit operand one slot later (sum_part), so that no instruction waits for an exponential just issued.
     auto exp_part = [&](auto I, auto HFc, auto STARTc, auto LENc) {
       constexpr int i = decltype(I)::value, hf = decltype(HFc)::value, st = decltype(STARTc)::value, len = decltype(LENc)::value;
       if constexpr (i >= st && i < st + len) {
@@ -392,8 +393,17 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
           float pv = fast_exp2(__builtin_fmaf(s[hf][v], c, -m_use));
           asm volatile("" : "+v"(pv));  // keeps the computation in this slot
           s[hf][v] = pv;
-          if (v & 1) rs1 += pv;
-          else rs0 += pv;
+        }
+      }
+    };
+    auto sum_part = [&](auto I, auto HFc, auto STARTc, auto LENc) {
+      constexpr int i = decltype(I)::value, hf = decltype(HFc)::value, st = decltype(STARTc)::value + 1, len = decltype(LENc)::value;
+      if constexpr (i >= st && i < st + len) {
+        constexpr int k = i - st, lo = (k * 16 + len - 1) / len, hi = ((k + 1) * 16 + len - 1) / len;
+#pragma unroll
+        for (int v = lo; v < hi; v++) {
+          if (v & 1) rs1 += s[hf][v];
+          else rs0 += s[hf][v];
         }
         static_for<0, 2>([&](auto H) {
           constexpr int hh = decltype(H)::value;
@@ -423,6 +433,8 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
         if (MASKED) mask_half(s[0], 0);
         if (row_max_update(s[0], alpha0)) rescale_o(alpha0);
       }
+      // (the last values of half 0 join the sums before the sums join l_run below)
+      sum_part(I, I0{}, std::integral_constant<int, S1 + 1>{}, std::integral_constant<int, KSTEPS - 1>{});
       if constexpr (i == PV0) {
         if (MASKED) mask_half(s[1], 1);
         // half 0's row sums join l_run before the update can rescale it; P0 itself is relative to the
@@ -433,6 +445,7 @@ __global__ __launch_bounds__(256, (fwd_blocks_per_cu<DQK, CAUSAL, SEG>())) void 
         moved1 = row_max_update(s[1], alpha1);
       }
       exp_part(I, I0{}, std::integral_constant<int, S1 + 1>{}, std::integral_constant<int, KSTEPS - 1>{});
+      sum_part(I, I1{}, std::integral_constant<int, PV0 + 1>{}, std::integral_constant<int, 2 * PVB - 1>{});
       exp_part(I, I1{}, std::integral_constant<int, PV0 + 1>{}, std::integral_constant<int, 2 * PVB - 1>{});
       if constexpr (i == PV1 - 1) {
         if (moved1) rescale_o(alpha1);
