@@ -212,6 +212,40 @@ __global__ __launch_bounds__(THREADS) void acc_kind(float* out, int iters, long 
   if (blockIdx.x == 0 && t == 0) cyc[0] = t1 - t0;
 }
 
+// ---- (5) what the vector-ALU work reads: per MFMA (compiler-known, four accumulators in rotation) NV FMAs that
+// read x only (SRC 0), or one value each of the accumulator written two MFMAs earlier (SRC 1), or that and feed the
+// next MFMAs' B operand through a conversion (SRC 2: the MFMA -> VALU -> MFMA chain of an attention tile)
+template <int SRC, int NV, int THREADS>
+__global__ __launch_bounds__(THREADS) void valu_src(float* out, int iters, long long* cyc) {
+  const int t = threadIdx.x, l = t & 63;
+  bf16x8 a, b;
+  for (int e = 0; e < 8; e++) { a[e] = (__bf16)(1.0f + l * 0.001f); b[e] = (__bf16)1.0f; }
+  f32x16 c[4];
+  for (int i = 0; i < 4; i++) for (int v = 0; v < 16; v++) c[i][v] = 0.f;
+  float x[8];
+  for (int i = 0; i < 8; i++) x[i] = l * 0.001f + i;
+  long long t0 = __builtin_readcyclecounter();
+  for (int i = 0; i < iters; i++) {
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+      c[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c[j & 3], 0, 0, 0);
+#pragma unroll
+      for (int k = 0; k < NV; k++) {
+        if (SRC == 0) x[(j + k) % 8] = x[(j + k) % 8] * 0.999f + 0.5f;
+        else x[(j + k) % 8] = c[(j + 2) & 3][(4 * (j >> 2) + k) & 15] * 0.999f + x[(j + k) % 8];
+      }
+      if (SRC == 2 && (j & 3) == 3) b[0] = (__bf16)x[j % 8];
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  long long t1 = __builtin_readcyclecounter();
+  float s = 0;
+  for (int i = 0; i < 4; i++) s += c[i][0];
+  for (int i = 0; i < 8; i++) s += x[i];
+  out[blockIdx.x * THREADS + t] = s;
+  if (blockIdx.x == 0 && t == 0) cyc[0] = t1 - t0;
+}
+
 int main() {
   hipDeviceProp_t p; CK(hipGetDeviceProperties(&p, 0));
   const int ncu = p.multiProcessorCount;
@@ -235,6 +269,7 @@ int main() {
 #define ONE(RK, NV, NE) { float ms = timeit([&] { one<RK, NV, NE><<<ncu, 256>>>(out, it, cyc); }); CK(hipMemcpy(h, cyc, 8, hipMemcpyDeviceToHost)); \
     printf("one wave/SIMD: reads=%d valu=%d exp=%d: %.1f cycles per MFMA (%.3f ms)\n", RK, NV, NE, (double)h[0] / (it * 16.0), ms); fflush(stdout); }
     ONE(0, 0, 0) ONE(1, 0, 0) ONE(2, 0, 0) ONE(1, 2, 0) ONE(2, 2, 0) ONE(1, 3, 1) ONE(2, 3, 1) ONE(1, 4, 1) ONE(1, 6, 1) ONE(0, 3, 1) ONE(0, 6, 0) ONE(0, 8, 0)
+    ONE(0, 0, 1) ONE(0, 0, 2) ONE(0, 0, 3) ONE(0, 2, 2) ONE(1, 2, 2) ONE(2, 2, 2) ONE(2, 0, 0) ONE(2, 2, 1)
   }
   {
     const int it = 500;
@@ -255,6 +290,14 @@ int main() {
     ACCK(0, 4, 0, 512) ACCK(1, 4, 0, 512)
     ACCK(0, 4, 4, 512) ACCK(1, 4, 4, 512) ACCK(0, 4, 6, 512) ACCK(1, 4, 6, 512) ACCK(0, 4, 8, 512) ACCK(1, 4, 8, 512)
     ACCK(0, 1, 6, 512) ACCK(1, 1, 6, 512)
+  }
+  {
+    const int it = 2000;
+#define VSRC(S, NV, TH) { float ms = timeit([&] { valu_src<S, NV, TH><<<ncu, TH>>>(out, it, cyc); }); \
+    printf("%d wave(s)/SIMD, FMAs read %s, valu/mfma=%d: %.3f ms for %d MFMAs per wave\n", TH / 256, \
+           S == 0 ? "their own registers" : S == 1 ? "an accumulator written two MFMAs earlier" : "an accumulator and feed the B operand", NV, ms, it * 16); fflush(stdout); }
+    VSRC(0, 4, 256) VSRC(1, 4, 256) VSRC(2, 4, 256) VSRC(0, 4, 512) VSRC(1, 4, 512) VSRC(2, 4, 512)
+    VSRC(0, 2, 256) VSRC(1, 2, 256) VSRC(0, 2, 512) VSRC(1, 2, 512) VSRC(0, 6, 512) VSRC(1, 6, 512)
   }
   printf("done\n");
   return 0;
