@@ -737,7 +737,7 @@ _PROFILE_COMMANDS = {
   "pmc_a": "rocprofv3 --pmc SQ_BUSY_CU_CYCLES SQ_VALU_MFMA_BUSY_CYCLES SQ_ACTIVE_INST_VALU SQ_VALU_MFMA_COEXEC_CYCLES SQ_INSTS_VALU SQ_WAIT_INST_ANY SQ_ACTIVE_INST_ANY SQ_WAVE_CYCLES --output-format csv -d {d}/pmc_a -o p -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-extra > {d}/pmc_a.log",
   "pmc_b": "rocprofv3 --pmc SQ_INSTS_MFMA SQ_INSTS_LDS SQ_LDS_ADDR_CONFLICT SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE SQ_ACTIVE_INST_LDS SQ_WAIT_INST_LDS SQ_BUSY_CU_CYCLES --output-format csv -d {d}/pmc_b -o p -- python3 bench.py --steps 2 --warmup 1 --no-cpu --no-extra",
   "kt_oc": "rocprofv3 --kernel-trace --stats --output-format csv -d {d}/kt_oc -o kt -- python3 bench.py --other-configs all --steps 10 > {d}/kt_oc.log",
-  "kt_extra": "rocprofv3 --kernel-trace --stats --output-format csv -d {d}/kt_extra -o kt -- python3 bench.py --steps 10 --warmup 3 --no-cpu > {d}/kt_extra.log",
+  "kt_extra": "rocprofv3 --kernel-trace --stats --output-format csv -d {d}/kt_extra -o kt -- python3 bench.py --steps 10 --warmup 3 --no-cpu --no-clock-probe > {d}/kt_extra.log",
 }  # fmt: skip
 
 
@@ -976,6 +976,7 @@ def main():
                   help="run only one Llama-3-8B decoder layer forward + backward (GEMMs included) and print its line")
   ap.add_argument("--tiny-config", action="store_true",
                   help="run only the tiny fp32 configuration's launch-by-launch / HIP graph comparison and print its line")
+  ap.add_argument("--no-clock-probe", action="store_true", help="leave the sustained-clock diagnostic out of the default run's extra")
   ap.add_argument("--clock-probe", action="store_true",
                   help="run only the sustained-clock diagnostic (attention step and a hipBLASLt GEMM on normal and on zero inputs, "
                        "shader clock sampled meanwhile) and print its line")
@@ -1026,7 +1027,8 @@ def main():
     extra["other_configs"] = bench_other_configs(dev)
     extra["tiny_fp32_config_hip_graph"] = bench_tiny_config_graph(dev)
     extra["llama3_8b_decoder_layer"] = bench_decoder_layer(dev, iters=3)
-    extra["clock_probe"] = bench_clock_probe(dev, seconds=2.0)
+    if not args.no_clock_probe:
+      extra["clock_probe"] = bench_clock_probe(dev, seconds=2.0)
     torch.cuda.empty_cache()
   torch.cuda.empty_cache()
   cpu = None if args.no_cpu else cpu_baseline()
