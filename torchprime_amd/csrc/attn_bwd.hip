@@ -1921,7 +1921,17 @@ static int dispatch_bwd(const BwdArgs& a, int causal, hipStream_t st, void* cons
     if (a.seg) return launch_bwd<T, DQK, DV, true, true>(a, st, ev);
     return launch_bwd<T, DQK, DV, true, false>(a, st, ev);
   }
-  if (a.seg) return launch_bwd<T, DQK, DV, false, true>(a, st, ev);
+  if (a.seg) {
+    // segment ids without causality: the causal kernels with a band that covers every key, where the lean dQ kernel
+    // serves the problem (else the general instantiation)
+    if (LeanDq<DQK, DV, true, true>::taken(a.Skv)) {
+      BwdArgs b = a;
+      b.band_lo = BAND_INF;
+      b.band_hi = BAND_INF;
+      return launch_bwd<T, DQK, DV, true, true>(b, st, ev);
+    }
+    return launch_bwd<T, DQK, DV, false, true>(a, st, ev);
+  }
   return launch_bwd<T, DQK, DV, false, false>(a, st, ev);
 }
 
@@ -1968,7 +1978,8 @@ extern "C" int tp_attn_bwd_dq_first(int Skv, int Dqk, int Dv, int causal, int ha
   auto pick = [&](auto dq, auto dv) -> int {
     constexpr int DQ = decltype(dq)::value, DVV = decltype(dv)::value;
     if (causal) return has_seg ? LeanDq<DQ, DVV, true, true>::taken(Skv) : LeanDq<DQ, DVV, true, false>::taken(Skv);
-    return has_seg ? LeanDq<DQ, DVV, false, true>::taken(Skv) : LeanDq<DQ, DVV, false, false>::taken(Skv);
+    // (segment ids without causality run the causal kernels with an all-covering band where the lean kernel serves them)
+    return has_seg ? LeanDq<DQ, DVV, true, true>::taken(Skv) : LeanDq<DQ, DVV, false, false>::taken(Skv);
   };
   typedef std::integral_constant<int, 64> I64;
   typedef std::integral_constant<int, 128> I128;
