@@ -1932,6 +1932,15 @@ static int dispatch_bwd(const BwdArgs& a, int causal, hipStream_t st, void* cons
     }
     return launch_bwd<T, DQK, DV, false, true>(a, st, ev);
   }
+  if constexpr (!LeanDq<DQK, DV, false, false>::BUILT) {
+    // (head dims for which the lean dQ kernel exists with causality only: the same band)
+    if (LeanDq<DQK, DV, true, false>::taken(a.Skv)) {
+      BwdArgs b = a;
+      b.band_lo = BAND_INF;
+      b.band_hi = BAND_INF;
+      return launch_bwd<T, DQK, DV, true, false>(b, st, ev);
+    }
+  }
   return launch_bwd<T, DQK, DV, false, false>(a, st, ev);
 }
 
@@ -1979,7 +1988,8 @@ extern "C" int tp_attn_bwd_dq_first(int Skv, int Dqk, int Dv, int causal, int ha
     constexpr int DQ = decltype(dq)::value, DVV = decltype(dv)::value;
     if (causal) return has_seg ? LeanDq<DQ, DVV, true, true>::taken(Skv) : LeanDq<DQ, DVV, true, false>::taken(Skv);
     // (segment ids without causality run the causal kernels with an all-covering band where the lean kernel serves them)
-    return has_seg ? LeanDq<DQ, DVV, true, true>::taken(Skv) : LeanDq<DQ, DVV, false, false>::taken(Skv);
+    if (has_seg || !LeanDq<DQ, DVV, false, false>::BUILT) return has_seg ? LeanDq<DQ, DVV, true, true>::taken(Skv) : LeanDq<DQ, DVV, true, false>::taken(Skv);
+    return LeanDq<DQ, DVV, false, false>::taken(Skv);
   };
   typedef std::integral_constant<int, 64> I64;
   typedef std::integral_constant<int, 128> I128;
