@@ -381,6 +381,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const BwdArgs a) {
 
   // wave-level decisions for a query tile (uniform): skip if every query row precedes every kv row
   // (lo, hi: id range of the query tile; t: its index into the position ranges)
+  // (The decisions are taken on the wave's first kv row as it arrives, in a vector register.  With a scalar copy the
+  // compiler turns the choice of the tile body into scalar branches and copies the pinned accumulators between them,
+  // right behind the MFMAs that write them: the build's hazard check rejects that code.  The same change in the
+  // forward and the lean dQ kernel passed the check and ran 45 % and 64 % slower.)
   auto tile_mode_of = [&](int lo, int hi, int t, int qi0) {  // 0 = nothing to compute, 1 = no masking needed, 2 = masked
     bool skip = (CAUSAL && (qi0 + BMQ - 1 + band_hi < wkv0 || qi0 - band_lo > wkv0 + 31)) || wkv0 >= Skv;
     bool need_mask = (qi0 + BMQ > Sq) || (wkv0 + 32 > Skv) ||
