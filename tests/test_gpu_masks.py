@@ -181,6 +181,25 @@ def test_wrapper_and_module_paths():
   assert_close(out, pu.reorder_sequence(plain_dev.float().cpu(), cp, seq_dim=2), "vs the plain causal kernel")
 
 
+@pytest.mark.parametrize("cp,offset", [(2, 0), (4, 0), (4, 3), (16, 0)])
+def test_load_balanced_mask_fwd_bwd(cp, offset):
+  """A load-balanced causal mask through the wrapper, forward and backward, against the oracle on the positions
+  themselves (cp 2 .. 16: three to 31 runs of consecutive positions, down to 16 rows each)."""
+  B, Hq, Hkv, S, D = 1, 4, 2, 512, 128
+  q, k, v, do = (heads_view(B, h, S, D, 70 + i, torch.bfloat16) for i, h in enumerate((Hq, Hkv, Hkv, Hq)))
+  mask = pu.LoadBalancedCausalMask(shape=(S, S), offset=offset, cp_size=cp)
+  scale = 1 / math.sqrt(D)
+  qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+  out = tpa.tpu_splash_attention_jax_call_wrapper(mask, qd, kd, vd, None, None, False, q_seq_shards=cp, sm_scale=scale)[0]
+  out.backward(do.to(DEV))
+  o_ref, dq_ref, dk_ref, dv_ref = orc.attention_grads_ref(q, k, v, do, None, True, scale, torch.float32,
+                                                          q_positions=mask.q_sequence, causal_offset=offset)
+  assert_close(out, o_ref, "out")
+  assert_close(qd.grad, dq_ref, "dq", scale_abs=True)
+  assert_close(kd.grad, dk_ref, "dk", scale_abs=True)
+  assert_close(vd.grad, dv_ref, "dv", scale_abs=True)
+
+
 def test_full_size_sliding_window_slice():
   """Llama-3-8B layer shape with a 1024-token causal window: one (batch, kv group) slice against the oracle."""
   B, Hq, Hkv, S, D, W = 2, 32, 8, 8192, 128, 1024
