@@ -9,6 +9,9 @@
 //       issues MFMAs while the other does its element-wise work, with and without barriers and wave priorities).
 // Build and run:  make -C torchprime_amd/csrc probes && torchprime_amd/csrc/build/issue_and_lds_probe
 #include <hip/hip_runtime.h>
+#include <cmath>
+#include <cstring>
+#include <cstdlib>
 #include <cstdio>
 #include <cstdlib>
 #define CK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("HIP error %s at %d\n", hipGetErrorString(e), __LINE__); exit(1);} } while (0)
@@ -246,6 +249,34 @@ __global__ __launch_bounds__(THREADS) void valu_src(float* out, int iters, long 
   if (blockIdx.x == 0 && t == 0) cyc[0] = t1 - t0;
 }
 
+// ---- (6) does the order of the MFMAs matter for the clock the part sustains?  MFMAs alone (one wave per SIMD, every
+// CU), operands from eight A and eight B fragments of normal-distributed values held in registers, long enough for
+// the power management to settle.  The matrix pipe takes 32 cycles per MFMA whatever the operands, so the time of a
+// fixed count is the reciprocal of the sustained clock.  REUSE 0: A and B both change with every MFMA; 1: B stays
+// for four consecutive MFMAs (A changes); 2: A and B stay for four; 3: all-zero operands.
+template <int REUSE>
+__global__ __launch_bounds__(256) void mfma_order(const unsigned* __restrict__ src, float* out, int iters) {
+  const int t = threadIdx.x, l = t & 63;
+  u32x4 a[8], b[8];
+  for (int i = 0; i < 8; i++) {
+    a[i] = *(const u32x4*)(src + ((i * 64 + l) * 4));
+    b[i] = *(const u32x4*)(src + ((512 + i * 64 + l) * 4));
+    if (REUSE == 3) { a[i] = u32x4{0, 0, 0, 0}; b[i] = u32x4{0, 0, 0, 0}; }
+  }
+  f32x16 c[4];
+  for (int i = 0; i < 4; i++) for (int v = 0; v < 16; v++) c[i][v] = 0.f;
+  for (int i = 0; i < iters; i++) {
+#pragma unroll
+    for (int j = 0; j < 32; j++) {
+      const int ia = REUSE == 2 ? (j / 4) % 8 : j % 8, ib = REUSE >= 1 ? (j / 4) % 8 : (j + j / 8) % 8;
+      c[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[ia]), __builtin_bit_cast(bf16x8, b[ib]), c[j & 3], 0, 0, 0);
+    }
+  }
+  float s = 0;
+  for (int i = 0; i < 4; i++) s += c[i][0];
+  out[blockIdx.x * 256 + t] = s;
+}
+
 int main() {
   hipDeviceProp_t p; CK(hipGetDeviceProperties(&p, 0));
   const int ncu = p.multiProcessorCount;
@@ -298,6 +329,28 @@ int main() {
            S == 0 ? "their own registers" : S == 1 ? "an accumulator written two MFMAs earlier" : "an accumulator and feed the B operand", NV, ms, it * 16); fflush(stdout); }
     VSRC(0, 4, 256) VSRC(1, 4, 256) VSRC(2, 4, 256) VSRC(0, 4, 512) VSRC(1, 4, 512) VSRC(2, 4, 512)
     VSRC(0, 2, 256) VSRC(1, 2, 256) VSRC(0, 2, 512) VSRC(1, 2, 512) VSRC(0, 6, 512) VSRC(1, 6, 512)
+  }
+  {
+    // normal-distributed bf16 values (Box-Muller on a fixed LCG), scaled by 1/16 so that the sums stay small
+    unsigned* hsrc = (unsigned*)malloc(1024 * 4 * 4);
+    unsigned long long st = 88172645463325252ull;
+    auto uni = [&]() { st = st * 6364136223846793005ull + 1442695040888963407ull; return (double)((st >> 11) + 1) / 9007199254740993.0; };
+    auto nbf = [&]() {
+      const float f = (float)(sqrt(-2.0 * log(uni())) * cos(6.283185307179586 * uni()) / 16.0);
+      unsigned u; memcpy(&u, &f, 4);
+      return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    };
+    for (int i = 0; i < 4096; i++) hsrc[i] = nbf() | (nbf() << 16);
+    unsigned* dsrc; CK(hipMalloc(&dsrc, 4096 * 4)); CK(hipMemcpy(dsrc, hsrc, 4096 * 4, hipMemcpyHostToDevice));
+    const int it = 4000;  // 128000 MFMAs per wave and launch: about 2 ms
+#define ORD(R, name) { for (int w = 0; w < 150; w++) mfma_order<R><<<ncu, 256>>>(dsrc, out, it); CK(hipDeviceSynchronize()); \
+    float ms = timeit([&] { for (int w = 0; w < 50; w++) mfma_order<R><<<ncu, 256>>>(dsrc, out, it); }, 3) / 50; \
+    printf("MFMAs alone, %-44s %.3f ms per launch = %.0f MHz sustained\n", name, ms, 32.0 * 32 * it / (ms * 1e3)); fflush(stdout); }
+    ORD(0, "A and B change with every MFMA:")
+    ORD(1, "B stays for four MFMAs:")
+    ORD(2, "A and B stay for four MFMAs:")
+    ORD(3, "all-zero operands:")
+    ORD(0, "A and B change with every MFMA (again):")
   }
   printf("done\n");
   return 0;
