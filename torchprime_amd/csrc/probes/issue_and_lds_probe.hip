@@ -1,4 +1,4 @@
-// A stand-alone measurement program (not part of libtprime_hip.so): the three facts about gfx950 that the attention
+// A stand-alone measurement program (not part of libtprime_hip.so): the facts about gfx950 that the attention
 // kernels' LDS layouts and slot schedules rest on.
 //   (1) LDS read rates of ds_read_b128 / ds_read_b64 / ds_read_b64_tr_b16 with nothing else in the instruction
 //       stream, for the address patterns the kernels use (MFMA fragment reads and transposing reads of a dense
@@ -7,13 +7,17 @@
 //       reads) and n vector-ALU instructions / exponentials: what an instruction slot costs;
 //   (3) two waves per SIMD: an evenly mixed instruction stream against phase-separated streams (one group of waves
 //       issues MFMAs while the other does its element-wise work, with and without barriers and wave priorities).
+//   (4) accumulators in architectural or accumulation registers, chains of dependent MFMAs, independent FMAs under them;
+//   (5) FMAs that read MFMA results and feed MFMA operands (build with -mllvm -amdgpu-mfma-vgpr-form=1 for this part:
+//       with the compiler's default form the accumulators are copied between the register halves around every read);
+//   (6) MFMAs alone on normal-distributed and on zero operands: the clock the part sustains, and whether the order of
+//       the MFMAs (re-use of an operand across consecutive ones) changes it.
 // Build and run:  make -C torchprime_amd/csrc probes && torchprime_amd/csrc/build/issue_and_lds_probe
 #include <hip/hip_runtime.h>
 #include <cmath>
 #include <cstring>
 #include <cstdlib>
 #include <cstdio>
-#include <cstdlib>
 #define CK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("HIP error %s at %d\n", hipGetErrorString(e), __LINE__); exit(1);} } while (0)
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
